@@ -1,0 +1,125 @@
+/*
+ * sage_oracle.h — CPU oracle for the quantized-SDPA hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is the checker: tests, the smoke
+ * check and the bench's cpu_baseline leg may call it; the product library
+ * (libmi355_sage.so) never links, loads or falls back to it.
+ *
+ * Every tensor is addressed as logical [B, H, N, D] through four ELEMENT
+ * strides, the convention of the reference's native attention seam
+ * (serenitymojo/ops/cshim/cudnn_sdpa.cpp:375-387; the Mojo caller describes
+ * its [B,S,H,Dh] memory as {S*H*Dh, Dh, H*Dh, 1},
+ * serenitymojo/ops/attention_flash.mojo:46-54).
+ *
+ * Pinning status (what fixes each function independently of this file):
+ *   sage_oracle_sdpa_f32 / _online_f32 ... reference golden vectors
+ *       (ops/parity/sdpa_math_ref.txt, ops_smoke2.mojo:239-278) + closed forms.
+ *   bf16 / fp16 / e4m3 codecs ............. reference KATs
+ *       (ops/tests/fp8_quant_smoke.mojo:108-143) + torch / numpy library codecs.
+ *   sage_oracle_quant_q / _kmean / _quant_k / _quant_v_* , sage_oracle_attn:
+ *       PARITY UNPINNED by the reference — it holds no INT8 / SageAttention
+ *       code, test or vector.  They are pinned only by closed forms, invariants
+ *       and an independent numpy restatement (tests/), never by reference data.
+ */
+#ifndef SAGE_ORACLE_H
+#define SAGE_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scalar codecs ------------------------------------------------------ */
+float    sage_oracle_bf16_to_f32(uint16_t b);
+uint16_t sage_oracle_f32_to_bf16(float f);   /* RNE, ops/torch_bf16.mojo:27-60 */
+float    sage_oracle_f16_to_f32(uint16_t h);
+uint16_t sage_oracle_f32_to_f16(float f);    /* RNE, finite overflow saturates to 65504 */
+float    sage_oracle_e4m3_to_f32(uint8_t b); /* ops/fp8.mojo:60-78 */
+uint8_t  sage_oracle_f32_to_e4m3(float f);   /* RNE + saturate, ops/fp8_quant.mojo:61-93 */
+
+/* vector forms for the tests */
+void sage_oracle_f32_to_bf16_n(const float* x, uint16_t* y, int64_t n);
+void sage_oracle_f32_to_f16_n(const float* x, uint16_t* y, int64_t n);
+void sage_oracle_f32_to_e4m3_n(const float* x, uint8_t* y, int64_t n);
+void sage_oracle_e4m3_to_f32_n(const uint8_t* x, float* y, int64_t n);
+
+/* ---- full-precision SDPA (the referee) ---------------------------------- */
+/* Exact two-pass softmax attention, double accumulation.  Restates
+ * serenitymojo/ops/attention.mojo:18-27 and the numpy generator
+ * ops/parity/sdpa_math_oracle.py:39-52.  Returns 0, or -1 on bad arguments
+ * (same checks as cudnn_sdpa.cpp:391-393). */
+int sage_oracle_sdpa_f32(const float* q, const float* k, const float* v, float* o,
+                         int B, int H, int Nq, int Nkv, int D, float scale,
+                         const int64_t* qs, const int64_t* ks,
+                         const int64_t* vs, const int64_t* os);
+
+/* One-key-at-a-time online-softmax recurrence in fp32, restating
+ * serenitymojo/ops/attention.mojo:744-801 (m starts at -3e38, natural exp). */
+int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, float* o,
+                                int B, int H, int Nq, int Nkv, int D, float scale,
+                                const int64_t* qs, const int64_t* ks,
+                                const int64_t* vs, const int64_t* os);
+
+/* ---- quantizers --------------------------------------------------------- */
+/* Padded token count used by every quantized tensor: N rounded up to `mult`. */
+int64_t sage_oracle_pad(int64_t n, int64_t mult);
+
+/* Q: qs = f32(bf16) * c, c = fp32(scale*log2(e)) (rounded once from double);
+ * per (b,h,block of blkq tokens): amax -> sc = amax/127 (1.0 if amax==0),
+ * code = clamp(rne(qs/sc), -127, 127).  q8: [B,H,Npad,D] contiguous (pad rows 0),
+ * qscale: [B,H,ceil(N/blkq)].  Npad = pad(N, npad_mult). */
+int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
+                        const int64_t* strides, float scale, int blkq, int npad_mult,
+                        int8_t* q8, float* qscale);
+
+/* K mean over tokens per (b,h,d): 64-token partial sums in double (tokens
+ * ascending), partials added in ascending order, divided by N in double,
+ * rounded once to fp32.  kmean: [B,H,D]. */
+int sage_oracle_kmean(const uint16_t* k, int B, int H, int N, int D,
+                      const int64_t* strides, float* kmean);
+
+/* K: ks = f32(bf16) - kmean[b,h,d] (kmean may be NULL = no smoothing), then
+ * the same per-block INT8 rule with blocks of blkk tokens. */
+int sage_oracle_quant_k(const uint16_t* k, int B, int H, int N, int D,
+                        const int64_t* strides, const float* kmean, int blkk, int npad_mult,
+                        int8_t* k8, float* kscale);
+
+/* V variant 0: fp16 RNE of the bf16 value; plain [B,H,Npad,D], pad rows 0. */
+int sage_oracle_quant_v_f16(const uint16_t* v, int B, int H, int N, int D,
+                            const int64_t* strides, int npad_mult, uint16_t* v16);
+
+/* V variant 1: per (b,h,d) amax over tokens -> vscale = amax/448 (1.0 if 0),
+ * byte = e4m3(v / vscale).  v8 plain [B,H,Npad,D], vscale [B,H,D]. */
+int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
+                            const int64_t* strides, int npad_mult,
+                            uint8_t* v8, float* vscale);
+
+/* ---- quantized attention ------------------------------------------------ */
+/* s[i,j] = float(sum_d q8*k8) * (qscale*kscale)   (log2 domain)
+ * p = exp2(s - max_j s);  variant 0: P16 = f16(p), O = sum P16*V16 / sum p
+ *                         variant 1: P8 = e4m3(p*448), O = sum P8*V8 * vscale / (448 * sum p)
+ * O -> bf16 RNE in the caller's strides; o_f32 (optional, same strides) gets
+ * the unrounded value.  Padded tensors as produced by the quantizers above
+ * with token pads NqPad / NkvPad. */
+int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t NqPad,
+                     const int8_t* k8, const float* kscale, int blkk, int64_t NkvPad,
+                     const void* vq, const float* vscale, int variant,
+                     int B, int H, int Nq, int Nkv, int D,
+                     uint16_t* o_bf16, float* o_f32, const int64_t* os);
+
+/* Whole path on bf16 inputs (quantize + attention), the CPU baseline's unit
+ * of work.  Allocates its own temporaries.  smooth_k: 0/1. */
+int sage_oracle_sdpa_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                          uint16_t* o, float* o_f32,
+                          int B, int H, int Nq, int Nkv, int D, float scale,
+                          const int64_t* qs, const int64_t* ks,
+                          const int64_t* vs, const int64_t* os,
+                          int variant, int blkq, int blkk, int smooth_k);
+
+int sage_oracle_num_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

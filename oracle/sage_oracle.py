@@ -1,0 +1,249 @@
+"""ctypes binding of the CPU oracle (oracle/libsage_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+bench.py's cpu_baseline leg as the checker.  The product package
+(mojodiffusion_amd) never imports this module.
+
+All tensors are numpy arrays; bf16 / fp16 tensors are carried as uint16 bit
+patterns, e4m3 as uint8.  Tensors are addressed as logical [B, H, N, D] via
+element strides, so a [B, S, H, Dh] array is passed with strides_bshd(...).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libsage_oracle.so")
+_lib = None
+
+_i64p = ctypes.POINTER(ctypes.c_int64)
+
+
+def build(force=False):
+    """Compile the oracle with the Makefile next to this file."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.sage_oracle_bf16_to_f32.restype = ctypes.c_float
+        L.sage_oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
+        L.sage_oracle_f32_to_bf16.restype = ctypes.c_uint16
+        L.sage_oracle_f32_to_bf16.argtypes = [ctypes.c_float]
+        L.sage_oracle_f16_to_f32.restype = ctypes.c_float
+        L.sage_oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.sage_oracle_f32_to_f16.restype = ctypes.c_uint16
+        L.sage_oracle_f32_to_f16.argtypes = [ctypes.c_float]
+        L.sage_oracle_e4m3_to_f32.restype = ctypes.c_float
+        L.sage_oracle_e4m3_to_f32.argtypes = [ctypes.c_uint8]
+        L.sage_oracle_f32_to_e4m3.restype = ctypes.c_uint8
+        L.sage_oracle_f32_to_e4m3.argtypes = [ctypes.c_float]
+        L.sage_oracle_pad.restype = ctypes.c_int64
+        L.sage_oracle_pad.argtypes = [ctypes.c_int64, ctypes.c_int64]
+        for name in ("sage_oracle_f32_to_bf16_n", "sage_oracle_f32_to_f16_n",
+                     "sage_oracle_f32_to_e4m3_n", "sage_oracle_e4m3_to_f32_n"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+        for name in ("sage_oracle_sdpa_f32", "sage_oracle_sdpa_online_f32"):
+            getattr(L, name).restype = ctypes.c_int
+            getattr(L, name).argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 4
+        L.sage_oracle_quant_q.restype = ctypes.c_int
+        L.sage_oracle_quant_q.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_float,
+                                          ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_kmean.restype = ctypes.c_int
+        L.sage_oracle_kmean.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p]
+        L.sage_oracle_quant_k.restype = ctypes.c_int
+        L.sage_oracle_quant_k.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p,
+                                          ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_quant_v_f16.restype = ctypes.c_int
+        L.sage_oracle_quant_v_f16.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_int, ctypes.c_void_p]
+        L.sage_oracle_quant_v_fp8.restype = ctypes.c_int
+        L.sage_oracle_quant_v_fp8.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_int,
+                                              ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_attn.restype = ctypes.c_int
+        L.sage_oracle_attn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
+                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
+                                       ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int] + [ctypes.c_int] * 5 + [
+                                       ctypes.c_void_p, ctypes.c_void_p, _i64p]
+        L.sage_oracle_sdpa_bf16.restype = ctypes.c_int
+        L.sage_oracle_sdpa_bf16.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [
+                                            ctypes.c_int] * 4
+        L.sage_oracle_num_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+# ---------------------------------------------------------------------------
+# layout helpers
+# ---------------------------------------------------------------------------
+
+def strides_bshd(S, H, D):
+    """[B,S,H,D] contiguous memory seen as logical [B,H,N,D]
+    (serenitymojo/ops/attention_flash.mojo:46-54)."""
+    return (ctypes.c_int64 * 4)(S * H * D, D, H * D, 1)
+
+
+def strides_bhsd(H, S, D):
+    return (ctypes.c_int64 * 4)(H * S * D, S * D, D, 1)
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _chk(rc, what):
+    if rc != 0:
+        raise RuntimeError("%s: oracle rc=%d" % (what, rc))
+
+
+def pad(n, mult):
+    return (n + mult - 1) // mult * mult
+
+
+# ---------------------------------------------------------------------------
+# codecs (vector forms)
+# ---------------------------------------------------------------------------
+
+def f32_to_bf16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty(x.shape, np.uint16)
+    lib().sage_oracle_f32_to_bf16_n(_p(x), _p(y), x.size)
+    return y
+
+
+def bf16_to_f32(b):
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_f16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty(x.shape, np.uint16)
+    lib().sage_oracle_f32_to_f16_n(_p(x), _p(y), x.size)
+    return y
+
+
+def f32_to_e4m3(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty(x.shape, np.uint8)
+    lib().sage_oracle_f32_to_e4m3_n(_p(x), _p(y), x.size)
+    return y
+
+
+def e4m3_to_f32(b):
+    b = np.ascontiguousarray(b, dtype=np.uint8)
+    y = np.empty(b.shape, np.float32)
+    lib().sage_oracle_e4m3_to_f32_n(_p(b), _p(y), b.size)
+    return y
+
+
+# ---------------------------------------------------------------------------
+# SDPA on [B,S,H,D] arrays (the reference's physical layout)
+# ---------------------------------------------------------------------------
+
+def _dims_bshd(q, k):
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    return B, H, Sq, Skv, D
+
+
+def sdpa_f32(q, k, v, scale, online=False):
+    """fp32 inputs [B,S,H,D] -> fp32 output [B,Sq,H,D]."""
+    q, k, v = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v))
+    B, H, Sq, Skv, D = _dims_bshd(q, k)
+    o = np.empty_like(q)
+    fn = lib().sage_oracle_sdpa_online_f32 if online else lib().sage_oracle_sdpa_f32
+    _chk(fn(_p(q), _p(k), _p(v), _p(o), B, H, Sq, Skv, D, scale,
+            strides_bshd(Sq, H, D), strides_bshd(Skv, H, D), strides_bshd(Skv, H, D),
+            strides_bshd(Sq, H, D)), "sdpa_f32")
+    return o
+
+
+def quant_q(q_bf16, scale, blkq, npad_mult=None):
+    """q_bf16: uint16 [B,S,H,D].  Returns (q8 [B,H,Spad,D] int8, qscale [B,H,nblk] f32)."""
+    q = np.ascontiguousarray(q_bf16, dtype=np.uint16)
+    B, S, H, D = q.shape
+    mult = npad_mult or blkq
+    q8 = np.empty((B, H, pad(S, mult), D), np.int8)
+    sc = np.empty((B, H, (S + blkq - 1) // blkq), np.float32)
+    _chk(lib().sage_oracle_quant_q(_p(q), B, H, S, D, strides_bshd(S, H, D), scale, blkq, mult,
+                                   _p(q8), _p(sc)), "quant_q")
+    return q8, sc
+
+
+def kmean(k_bf16):
+    k = np.ascontiguousarray(k_bf16, dtype=np.uint16)
+    B, S, H, D = k.shape
+    mu = np.empty((B, H, D), np.float32)
+    _chk(lib().sage_oracle_kmean(_p(k), B, H, S, D, strides_bshd(S, H, D), _p(mu)), "kmean")
+    return mu
+
+
+def quant_k(k_bf16, mu, blkk, npad_mult=None):
+    k = np.ascontiguousarray(k_bf16, dtype=np.uint16)
+    B, S, H, D = k.shape
+    mult = npad_mult or blkk
+    k8 = np.empty((B, H, pad(S, mult), D), np.int8)
+    sc = np.empty((B, H, (S + blkk - 1) // blkk), np.float32)
+    if mu is not None:
+        mu = np.ascontiguousarray(mu, dtype=np.float32)
+    _chk(lib().sage_oracle_quant_k(_p(k), B, H, S, D, strides_bshd(S, H, D), _p(mu), blkk, mult,
+                                   _p(k8), _p(sc)), "quant_k")
+    return k8, sc
+
+
+def quant_v_f16(v_bf16, npad_mult):
+    v = np.ascontiguousarray(v_bf16, dtype=np.uint16)
+    B, S, H, D = v.shape
+    v16 = np.empty((B, H, pad(S, npad_mult), D), np.uint16)
+    _chk(lib().sage_oracle_quant_v_f16(_p(v), B, H, S, D, strides_bshd(S, H, D), npad_mult, _p(v16)),
+         "quant_v_f16")
+    return v16
+
+
+def quant_v_fp8(v_bf16, npad_mult):
+    v = np.ascontiguousarray(v_bf16, dtype=np.uint16)
+    B, S, H, D = v.shape
+    v8 = np.empty((B, H, pad(S, npad_mult), D), np.uint8)
+    vs = np.empty((B, H, D), np.float32)
+    _chk(lib().sage_oracle_quant_v_fp8(_p(v), B, H, S, D, strides_bshd(S, H, D), npad_mult,
+                                       _p(v8), _p(vs)), "quant_v_fp8")
+    return v8, vs
+
+
+def attn(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv):
+    """Quantized tensors in the oracle's plain [B,H,Npad,D] layout.
+    Returns (o_bf16 uint16 [B,Sq,H,D], o_f32 [B,Sq,H,D])."""
+    B, H, NqPad, D = q8.shape
+    NkvPad = k8.shape[2]
+    o16 = np.empty((B, Sq, H, D), np.uint16)
+    o32 = np.empty((B, Sq, H, D), np.float32)
+    _chk(lib().sage_oracle_attn(_p(q8), _p(qscale), blkq, NqPad, _p(k8), _p(kscale), blkk, NkvPad,
+                                _p(vq), _p(vscale), variant, B, H, Sq, Skv, D,
+                                _p(o16), _p(o32), strides_bshd(Sq, H, D)), "attn")
+    return o16, o32
+
+
+def sdpa_bf16(q, k, v, scale, variant=0, blkq=128, blkk=64, smooth_k=True):
+    """Whole quantized path on bf16 (uint16) [B,S,H,D] inputs.
+    Returns (o_bf16 uint16, o_f32)."""
+    q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
+    B, H, Sq, Skv, D = _dims_bshd(q, k)
+    o16 = np.empty((B, Sq, H, D), np.uint16)
+    o32 = np.empty((B, Sq, H, D), np.float32)
+    _chk(lib().sage_oracle_sdpa_bf16(_p(q), _p(k), _p(v), _p(o16), _p(o32), B, H, Sq, Skv, D, scale,
+                                     strides_bshd(Sq, H, D), strides_bshd(Skv, H, D),
+                                     strides_bshd(Skv, H, D), strides_bshd(Sq, H, D),
+                                     variant, blkq, blkk, 1 if smooth_k else 0), "sdpa_bf16")
+    return o16, o32
+
+
+def num_threads():
+    return lib().sage_oracle_num_threads()

@@ -1,0 +1,119 @@
+"""Independent numpy restatement of the quantizers and the quantized attention,
+written from the prose rules (not from the C oracle's code) so that the two can
+check each other.  numpy's float32 divide is correctly rounded and np.rint is
+round-half-to-even, which is what the rules require.
+
+Quantization rules restated:
+  Q:  x = f32(bf16) * c,  c = float32(float64(scale) * log2(e))
+  K:  x = f32(bf16) - mean32[b,h,d]          (when smoothing)
+  per block of `blk` tokens of one (b,h): amax = max|x|; sc = amax/127 (1 if 0);
+      code = clip(rint(x / sc), -127, 127)
+  V0: fp16(v);  V1: per (b,h,d) amax over tokens; sc = amax/448 (1 if 0); e4m3(v/sc)
+"""
+import math
+
+import numpy as np
+import torch
+
+LOG2E = 1.4426950408889634074
+
+
+def bf16_to_f32(b):
+    return (b.astype(np.uint32) << 16).view(np.float32)
+
+
+def quant_blocks(x_bhsd, blk, npad_mult):
+    """x: fp32 [B,H,S,D] already transformed.  Returns codes [B,H,Spad,D], scales [B,H,nblk]."""
+    B, H, S, D = x_bhsd.shape
+    nblk = (S + blk - 1) // blk
+    spad = (S + npad_mult - 1) // npad_mult * npad_mult
+    codes = np.zeros((B, H, spad, D), np.int8)
+    scales = np.zeros((B, H, nblk), np.float32)
+    for t in range(nblk):
+        tile = x_bhsd[:, :, t * blk:(t + 1) * blk, :]
+        amax = np.abs(tile).max(axis=(2, 3)).astype(np.float32)
+        sc = np.where(amax > 0, amax / np.float32(127.0), np.float32(1.0)).astype(np.float32)
+        c = np.clip(np.rint(tile / sc[:, :, None, None]), -127, 127).astype(np.int8)
+        codes[:, :, t * blk:t * blk + tile.shape[2], :] = c
+        scales[:, :, t] = sc
+    return codes, scales
+
+
+def quant_q(q_bits_bshd, scale, blkq, npad_mult):
+    c = np.float32(np.float64(np.float32(scale)) * LOG2E)
+    x = bf16_to_f32(q_bits_bshd).transpose(0, 2, 1, 3) * c
+    return quant_blocks(x.astype(np.float32), blkq, npad_mult)
+
+
+def kmean_exact(k_bits_bshd):
+    """Exactly rounded mean: math.fsum is an exact sum."""
+    x = bf16_to_f32(k_bits_bshd).transpose(0, 2, 1, 3).astype(np.float64)
+    B, H, S, D = x.shape
+    mu = np.empty((B, H, D), np.float32)
+    for b in range(B):
+        for h in range(H):
+            for d in range(D):
+                mu[b, h, d] = np.float32(math.fsum(x[b, h, :, d]) / S)
+    return mu
+
+
+def kmean_blocked(k_bits_bshd):
+    """The normative order: 64-token partials (ascending), partials ascending."""
+    x = bf16_to_f32(k_bits_bshd).transpose(0, 2, 1, 3).astype(np.float64)
+    B, H, S, D = x.shape
+    total = np.zeros((B, H, D))
+    for t0 in range(0, S, 64):
+        part = np.zeros((B, H, D))
+        for s in range(t0, min(S, t0 + 64)):
+            part = part + x[:, :, s, :]
+        total = total + part
+    return (total / float(S)).astype(np.float32)
+
+
+def quant_k(k_bits_bshd, mu, blkk, npad_mult):
+    x = bf16_to_f32(k_bits_bshd).transpose(0, 2, 1, 3)
+    if mu is not None:
+        x = x - mu[:, :, None, :]
+    return quant_blocks(x.astype(np.float32), blkk, npad_mult)
+
+
+def _pad_tokens(x, npad_mult):
+    B, H, S, D = x.shape
+    spad = (S + npad_mult - 1) // npad_mult * npad_mult
+    out = np.zeros((B, H, spad, D), x.dtype)
+    out[:, :, :S] = x
+    return out
+
+
+def quant_v_f16(v_bits_bshd, npad_mult):
+    x = bf16_to_f32(v_bits_bshd).transpose(0, 2, 1, 3)
+    with np.errstate(over="ignore"):
+        h = np.clip(x, -65504.0, 65504.0).astype(np.float16)
+    return _pad_tokens(h.view(np.uint16), npad_mult)
+
+
+def quant_v_fp8(v_bits_bshd, npad_mult):
+    x = bf16_to_f32(v_bits_bshd).transpose(0, 2, 1, 3)
+    amax = np.abs(x).max(axis=2).astype(np.float32)
+    sc = np.where(amax > 0, amax / np.float32(448.0), np.float32(1.0)).astype(np.float32)
+    y = (x / sc[:, :, None, :]).astype(np.float32)
+    b = torch.from_numpy(np.ascontiguousarray(y)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    return _pad_tokens(b, npad_mult), sc
+
+
+def attn_float64(q8, qs, blkq, k8, ks, blkk, v_f32, Sq, Skv, p_codec):
+    """Quantized attention in float64 from the quantized tensors.
+    v_f32: decoded V [B,H,Skv_pad,D] (already multiplied by any per-channel scale).
+    p_codec: function rounding p (float32 array in [0,1]) to the P*V operand grid."""
+    B, H, _, D = q8.shape
+    out = np.zeros((B, Sq, H, D))
+    for b in range(B):
+        for h in range(H):
+            acc = q8[b, h, :Sq].astype(np.int64) @ k8[b, h, :Skv].astype(np.int64).T
+            sq = np.repeat(qs[b, h], blkq)[:Sq]
+            sk = np.repeat(ks[b, h], blkk)[:Skv]
+            s = acc.astype(np.float32) * (sq[:, None] * sk[None, :]).astype(np.float32)
+            p = np.exp2((s - s.max(axis=1, keepdims=True)).astype(np.float32)).astype(np.float32)
+            l = p.astype(np.float64).sum(axis=1, keepdims=True)
+            out[b, :, h, :] = (p_codec(p).astype(np.float64) @ v_f32[b, h, :Skv].astype(np.float64)) / l
+    return out
