@@ -1,0 +1,176 @@
+/*
+ * mi355_sage.h — C ABI of libmi355_sage.so: SageAttention-style quantized
+ * scaled-dot-product attention for AMD MI355X (gfx950), hand-written HIP.
+ *
+ * The library sits behind the same seam as the reference's native attention
+ * shim: raw device pointers, dims, four ELEMENT strides per tensor describing
+ * the memory as logical [B, H, N, D], element offsets, a stream, an int return
+ * code.  Work is enqueued on the caller's stream; no call synchronizes.
+ *
+ * Conventions shared by every entry point
+ *   - tensors are caller-allocated device memory; stride arrays are host
+ *     memory read during the call only
+ *     (serenitymojo/ops/attention_flash.mojo:177-193);
+ *   - q/k/v/o are bf16; the innermost (D) stride must be 1 and every row start
+ *     must be 16-byte aligned (callers hand out 16-byte-aligned scratch views,
+ *     serenitymojo/scratch_ring.mojo:49);
+ *   - D is 64 or 128; attention is full, non-causal, unmasked; N_q may differ
+ *     from N_kv;
+ *   - return 0 on success; -1 for a null pointer, a non-positive dimension or
+ *     null strides (serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393); -2 for an
+ *     unsupported configuration; -3 for a workspace that is too small; a
+ *     positive value is a hipError_t.  Diagnostics go to stderr tagged
+ *     [mi355_sage].
+ */
+#ifndef MI355_SAGE_H
+#define MI355_SAGE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_SAGE_OK            0
+#define MI355_SAGE_EINVAL      (-1)
+#define MI355_SAGE_EUNSUPPORTED (-2)
+#define MI355_SAGE_EWORKSPACE  (-3)
+
+/* P*V arithmetic. */
+#define MI355_SAGE_PV_FP16 0   /* INT8 QK^T, FP16 P*V              */
+#define MI355_SAGE_PV_FP8  1   /* INT8 QK^T, FP8-e4m3 P*V, per-channel V scales */
+
+/* ------------------------------------------------------------------------
+ * One-shot drop-in.
+ * Replaces flame_cudnn_sdpa_bf16 (serenitymojo/ops/cshim/cudnn_sdpa.cpp:375-387):
+ * the parameter list up to `stream` is identical; `variant`, `workspace` and
+ * `workspace_bytes` are appended.  Quantizes Q/K (K mean-smoothed, Q in
+ * 128-token blocks for variant 0 and 32-token blocks for variant 1, K in
+ * 64-token blocks), repacks or quantizes V, runs the attention kernel and
+ * writes bf16 O in the caller's strides.
+ *
+ * workspace == NULL: the library keeps one internal device buffer per device,
+ * grown on demand (the counterpart of the reference shim's lazily allocated,
+ * never-freed workspace, cudnn_sdpa.cpp:218-231); a call that does not grow it
+ * allocates nothing.  Otherwise workspace_bytes must be at least
+ * mi355_sage_workspace_bytes(...) and the pointer 256-byte aligned.
+ * `causal` must be 0.
+ * ---------------------------------------------------------------------- */
+int mi355_sage_sdpa_bf16(
+    const void* Q, const void* K, const void* V, void* O,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems,
+    int causal,
+    void* stream,
+    int variant, void* workspace, size_t workspace_bytes);
+
+/* Same with the quantization recipe spelled out: blkq / blkk = tokens per Q / K
+ * scale block (32, 64 or 128 each), smooth_k 0/1. */
+int mi355_sage_sdpa_bf16_ex(
+    const void* Q, const void* K, const void* V, void* O,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems,
+    int causal,
+    void* stream,
+    int variant, int blkq, int blkk, int smooth_k,
+    void* workspace, size_t workspace_bytes);
+
+/* Replaces flame_cudnn_sdpa_bf16_train_fwd (cudnn_sdpa.cpp:470-484), the symbol
+ * every Mojo caller binds (serenitymojo/ops/attention_flash.mojo:182-192): same
+ * parameter list plus the three trailing arguments.  Stats receives the fp32
+ * natural-log log-sum-exp of the scaled scores, layout [B,H,N_q,1] with strides
+ * {H*N_q, N_q, 1, 1} (cudnn_sdpa.cpp:304-312).  real_N_kv in (0, N_kv) masks
+ * the keys at and beyond it (the padding mask of attention_flash.mojo:275-287);
+ * query rows at and beyond real_N_q are computed but carry no meaning. */
+int mi355_sage_sdpa_bf16_train_fwd(
+    const void* Q, const void* K, const void* V, void* O, void* Stats,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems,
+    int64_t stats_offset_elems,
+    int causal,
+    int real_N_q, int real_N_kv,
+    void* stream,
+    int variant, void* workspace, size_t workspace_bytes);
+
+/* Bytes of workspace the one-shot calls need for this problem (0 on bad
+ * arguments).  No counterpart in the reference, whose shim sizes its own. */
+size_t mi355_sage_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int variant);
+
+/* ------------------------------------------------------------------------
+ * Stage entry points (no counterpart in the reference, which has no quantized
+ * attention): each kernel of the path in isolation, so that the INT8 codes and
+ * fp32 scales can be compared bit-for-bit with a CPU restatement.
+ *
+ * Quantized tensor layouts (device memory, caller-allocated):
+ *   q8      int8  [B, H, pad_q(N_q),  D]   pad rows are 0
+ *   qscale  fp32  [B, H, pad_q(N_q)/blkq]  pad blocks are 1.0
+ *   k8      int8  [B, H, pad_kv(N_kv), D]
+ *   kscale  fp32  [B, H, pad_kv(N_kv)/blkk]
+ *   kmean   fp32  [B, H, D]
+ *   v16     fp16  [B, H, pad_kv/64, D, 64]  64-key tiles, channel-major inside a
+ *                                           tile, key k of a tile stored at slot
+ *                                           mi355_sage_v_slot(k, PV_FP16)
+ *   v8      e4m3  [B, H, pad_kv/64, D, 64]  same with mi355_sage_v_slot(k, PV_FP8)
+ *   vscale  fp32  [B, H, D]
+ * ---------------------------------------------------------------------- */
+int64_t mi355_sage_pad_q(int64_t n);    /* query tokens round up to the query tile  */
+int64_t mi355_sage_pad_kv(int64_t n);   /* key tokens round up to the key tile      */
+int     mi355_sage_v_slot(int key_in_tile, int variant);
+
+/* Bytes of scratch mi355_sage_quant_qk_bf16 / _quant_v_fp8 need (partial sums). */
+size_t mi355_sage_quant_scratch_bytes(int B, int H, int N_kv, int D);
+
+/* Q: x = f32(q) * fp32(scale*log2(e));  K: x = f32(k) - kmean (if smooth_k).
+ * Per block: amax -> s = amax/127 (1.0 when 0) -> code = clamp(rne(x/s), +-127).
+ * kmean is written when smooth_k != 0 (pass NULL otherwise). */
+int mi355_sage_quant_qk_bf16(
+    const void* Q, const void* K,
+    int B, int H, int N_q, int N_kv, int D, float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int blkq, int blkk, int smooth_k,
+    void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+    void* scratch, size_t scratch_bytes, void* stream);
+
+/* V -> fp16 (round-to-nearest-even, finite overflow saturates), tiled layout. */
+int mi355_sage_quant_v_f16(
+    const void* V, int B, int H, int N_kv, int D,
+    const int64_t* v_strides, int64_t v_offset_elems,
+    void* v16, void* stream);
+
+/* V -> e4m3 with per-(b,h,channel) scale amax/448 (1.0 when 0), tiled layout. */
+int mi355_sage_quant_v_fp8(
+    const void* V, int B, int H, int N_kv, int D,
+    const int64_t* v_strides, int64_t v_offset_elems,
+    void* v8, void* vscale, void* stream);
+
+/* Attention on the quantized tensors.  stats may be NULL.  kv_valid = number of
+ * real keys (<= N_kv); keys beyond it are masked. */
+int mi355_sage_attn_fwd(
+    const void* q8, const void* qscale, int blkq,
+    const void* k8, const void* kscale, int blkk,
+    const void* vq, const void* vscale, int variant,
+    int B, int H, int N_q, int N_kv, int kv_valid, int D,
+    void* O, const int64_t* o_strides, int64_t o_offset_elems,
+    void* stats, void* stream);
+
+/* Library identification: "mi355_sage <version> gfx950". */
+const char* mi355_sage_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,178 @@
+"""Host side of the quantized-SDPA path: the serenitymojo attention call surface
+bound to libmi355_sage.so.
+
+Function names, argument meaning and error behaviour follow
+serenitymojo/ops/attention_flash.mojo (sdpa_flash_train_fwd :149-202, _rect
+:205-264, sdpa_flash_fwd_padmask :267-342, sdpa_flash_train_fwd_f32 :457-475) and
+serenitymojo/ops/attention.mojo (sdpa_nomask :1690-1718, sdpa_nomask_tiled
+:1762-1787, sdpa_cross_nomask :1860-1894).  Tensors are [B, S, H, Dh]; torch is
+used only to own device memory and the stream.  What differs from the cuDNN path:
+no 128-padding copies are needed (ragged S is handled in the kernels), so the
+`*_pad` members of the result alias the caller's tensors.
+"""
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+PV_FP16 = 0
+PV_FP8 = 1
+
+
+class Error(RuntimeError):
+    """Counterpart of Mojo's `raise Error(...)`."""
+
+
+@dataclass
+class SdpaFlashFwd:
+    """serenitymojo/ops/attention_flash.mojo:108-135."""
+    o: torch.Tensor
+    o_pad: torch.Tensor
+    q_pad: torch.Tensor
+    k_pad: torch.Tensor
+    v_pad: torch.Tensor
+    stats: torch.Tensor
+
+
+_workspaces = {}
+
+
+def _workspace(nbytes, device):
+    """Caller-side workspace reuse: one growing buffer per device, so steady-state
+    calls allocate nothing."""
+    key = (device.type, device.index)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _require_bf16(name, *ts):
+    for t in ts:
+        if t.dtype != torch.bfloat16:
+            raise Error("%s: q/k/v must be BF16" % name)
+
+
+def _require_cuda(name, *ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise Error("%s: tensors must live on the GPU (no CPU fallback exists)" % name)
+        if not t.is_contiguous():
+            raise Error("%s: tensors must be contiguous [B,S,H,Dh]" % name)
+
+
+def _call_train_fwd(name, q, k, v, scale, real_q, real_kv, variant, want_stats):
+    B, Sq, H, Dh = q.shape
+    Skv = k.shape[1]
+    L = _lib.lib()
+    o = torch.empty_like(q)
+    stats = torch.empty((B, H, Sq, 1), dtype=torch.float32, device=q.device) if want_stats else None
+    nbytes = L.mi355_sage_workspace_bytes(B, H, Sq, Skv, Dh, variant)
+    ws = _workspace(max(nbytes, 256), q.device)
+    qs = _lib.strides_bhnd(Sq, H, Dh)
+    ks = _lib.strides_bhnd(Skv, H, Dh)
+    stream = torch.cuda.current_stream(q.device).cuda_stream
+    if want_stats:
+        rc = L.mi355_sage_sdpa_bf16_train_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), stats.data_ptr(),
+            B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, 0, 0, 0, 0, 0,
+            0, real_q, real_kv, stream, variant, ws.data_ptr(), ws.numel())
+    else:
+        rc = L.mi355_sage_sdpa_bf16(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+            B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, 0, 0, 0, 0,
+            0, stream, variant, ws.data_ptr(), ws.numel())
+    if rc != 0:
+        raise Error("%s: shim rc=%d (B=%d Sq=%d Skv=%d H=%d Dh=%d)" % (name, rc, B, Sq, Skv, H, Dh))
+    return o, stats
+
+
+def _check_shapes(name, q, k, v, square):
+    if q.dim() != 4:
+        raise Error("%s: q must be rank-4 [B,S,H,Dh]" % name)
+    if k.shape != v.shape or k.dim() != 4:
+        raise Error("%s: k/v shape mismatch" % name)
+    if q.shape[0] != k.shape[0] or q.shape[2] != k.shape[2] or q.shape[3] != k.shape[3]:
+        raise Error("%s: q and k/v disagree on B/H/Dh" % name)
+    if square and q.shape[1] != k.shape[1]:
+        raise Error("%s: k/v shape does not match q [B,S,H,Dh]" % name)
+
+
+def sdpa_flash_train_fwd(q, k, v, scale, variant=PV_FP16):
+    """Forward on [B,S,H,Dh] BF16 (no mask, non-causal); returns O and the
+    log-sum-exp Stats [B,H,S,1].  Fails loudly on any non-zero return code."""
+    _require_bf16("sdpa_flash_train_fwd", q, k, v)
+    _check_shapes("sdpa_flash_train_fwd", q, k, v, True)
+    _require_cuda("sdpa_flash_train_fwd", q, k, v)
+    o, stats = _call_train_fwd("sdpa_flash_train_fwd", q, k, v, scale, q.shape[1], k.shape[1], variant, True)
+    return SdpaFlashFwd(o, o, q, k, v, stats)
+
+
+def sdpa_flash_train_fwd_rect(q, k, v, scale, variant=PV_FP16):
+    """Rectangular no-mask attention: q [B,Sq,H,Dh], k/v [B,Skv,H,Dh]."""
+    _require_bf16("sdpa_flash_train_fwd_rect", q, k, v)
+    _check_shapes("sdpa_flash_train_fwd_rect", q, k, v, False)
+    _require_cuda("sdpa_flash_train_fwd_rect", q, k, v)
+    o, stats = _call_train_fwd("sdpa_flash_train_fwd_rect", q, k, v, scale, q.shape[1], k.shape[1], variant, True)
+    return SdpaFlashFwd(o, o, q, k, v, stats)
+
+
+def sdpa_flash_fwd_padmask(q, k, v, real_len, scale, variant=PV_FP16):
+    """Pre-padded [B,S_BUF,H,Dh] buffers whose first real_len positions are real:
+    keys at and beyond real_len are excluded from every query; query rows there
+    are garbage the caller discards."""
+    _require_bf16("sdpa_flash_fwd_padmask", q, k, v)
+    _check_shapes("sdpa_flash_fwd_padmask", q, k, v, True)
+    s_buf = q.shape[1]
+    if s_buf % 128 != 0:
+        raise Error("sdpa_flash_fwd_padmask: S_BUF must be 128-aligned")
+    if real_len < 1 or real_len > s_buf:
+        raise Error("sdpa_flash_fwd_padmask: real_len out of [1, S_BUF]")
+    _require_cuda("sdpa_flash_fwd_padmask", q, k, v)
+    o, stats = _call_train_fwd("sdpa_flash_fwd_padmask", q, k, v, scale, real_len, real_len, variant, True)
+    return SdpaFlashFwd(o, o, q, k, v, stats)
+
+
+def sdpa_flash_train_fwd_f32(q, k, v, scale, variant=PV_FP16):
+    """F32 activations: cast to BF16 at the boundary, attend, cast back
+    (attention_flash.mojo:457-475).  Returns (att_f32, SdpaFlashFwd of the bf16 run)."""
+    fwd = sdpa_flash_train_fwd(q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16), scale, variant)
+    return fwd.o.to(torch.float32), fwd
+
+
+def sdpa_nomask(q, k, v, scale, variant=PV_FP16):
+    """Full attention without a mask tensor (attention.mojo:1690-1718): the entry
+    every DiT sampler uses.  Output has q's dtype; F32/F16 storage is cast to
+    BF16 at the boundary as the reference's per-model dispatchers do
+    (models/zimage/lora_block.mojo:99-123)."""
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise Error("sdpa_nomask: q/k/v dtype mismatch")
+    _check_shapes("sdpa_nomask", q, k, v, True)
+    _require_cuda("sdpa_nomask", q, k, v)
+    if q.dtype == torch.bfloat16:
+        o, _ = _call_train_fwd("sdpa_nomask", q, k, v, scale, q.shape[1], k.shape[1], variant, False)
+        return o
+    o, _ = _call_train_fwd("sdpa_nomask", q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16),
+                           scale, q.shape[1], k.shape[1], variant, False)
+    return o.to(q.dtype)
+
+
+def sdpa_nomask_tiled(q, k, v, scale, variant=PV_FP16):
+    """attention.mojo:1762-1787: the long-sequence entry (video DiTs).  The
+    quantized kernel never materialises scores, so it is the same call."""
+    return sdpa_nomask(q, k, v, scale, variant)
+
+
+def sdpa_cross_nomask(q, k, v, scale, variant=PV_FP16):
+    """attention.mojo:1860-1894: rectangular Sq != Skv, no mask."""
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise Error("sdpa_cross_nomask: q/k/v dtype mismatch")
+    _check_shapes("sdpa_cross_nomask", q, k, v, False)
+    _require_cuda("sdpa_cross_nomask", q, k, v)
+    if q.dtype == torch.bfloat16:
+        return _call_train_fwd("sdpa_cross_nomask", q, k, v, scale, q.shape[1], k.shape[1], variant, False)[0]
+    o = _call_train_fwd("sdpa_cross_nomask", q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16),
+                        scale, q.shape[1], k.shape[1], variant, False)[0]
+    return o.to(q.dtype)

@@ -1,0 +1,422 @@
+// sage_quant.hip — HBM-bound kernels of the quantized-SDPA path (gfx950):
+//   * per-block INT8 quantization of Q (pre-scaled) and K (mean-smoothed),
+//   * the K mean over tokens (deterministic summation tree in fp64),
+//   * V repack to tiled fp16, V quantization to tiled e4m3 with per-channel scales.
+//
+// Every fp32 step that decides a code is a single IEEE operation (true divide,
+// round-half-to-even), so the codes and scales are reproducible bit-for-bit.
+// All kernels read bf16 rows with 16-byte loads (8 channels per lane).
+#include "sage_internal.h"
+
+#include <hip/hip_fp16.h>
+
+namespace sage {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+
+__device__ __forceinline__ void unpack8(const u32x4& w, float* x) {
+    x[0] = bf16_lo(w.x); x[1] = bf16_hi(w.x);
+    x[2] = bf16_lo(w.y); x[3] = bf16_hi(w.y);
+    x[4] = bf16_lo(w.z); x[5] = bf16_hi(w.z);
+    x[6] = bf16_lo(w.w); x[7] = bf16_hi(w.w);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// Per-block INT8 quantization.  One workgroup (256 threads) per (block, h, b);
+// the block's BLK x D tile lives in registers between the absmax pass and the
+// encode pass, so HBM sees one read of bf16 and one write of int8.
+// ---------------------------------------------------------------------------
+template <int D, int BLK, bool IS_K>
+__global__ __launch_bounds__(256) void quant_i8_kernel(
+    const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
+    int8_t* __restrict__ codes, float* __restrict__ scales) {
+    constexpr int CPR = D / 8;                 // 16-byte chunks per row
+    constexpr int NCH = BLK * CPR / 256;       // chunks per thread
+    static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
+    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int r0 = t * BLK;
+    const int64_t bh = (int64_t)b * H + h;
+    const uint16_t* src = x + b * sb + h * sh;
+
+    float v[NCH][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = i * 256 + tid;
+        const int row = r0 + c / CPR, col = (c % CPR) * 8;
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (row < N) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+        unpack8(w, v[i]);
+        if (IS_K) {
+            if (mean != nullptr) {
+                const float4 m0 = *reinterpret_cast<const float4*>(mean + bh * D + col);
+                const float4 m1 = *reinterpret_cast<const float4*>(mean + bh * D + col + 4);
+                v[i][0] -= m0.x; v[i][1] -= m0.y; v[i][2] -= m0.z; v[i][3] -= m0.w;
+                v[i][4] -= m1.x; v[i][5] -= m1.y; v[i][6] -= m1.z; v[i][7] -= m1.w;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[i][e] *= cmul;
+        }
+        if (row < N) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[i][e]));
+        }
+    }
+
+    __shared__ float red[4];
+    amax = wave_max(amax);
+    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+
+    const bool real_block = r0 < N;
+    const float sc = (real_block && amax > 0.0f) ? amax / 127.0f : 1.0f;
+    if (tid == 0) scales[bh * (n_pad / BLK) + t] = sc;
+
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = i * 256 + tid;
+        const int row = r0 + c / CPR, col = (c % CPR) * 8;
+        uint32_t pk[2] = {0u, 0u};
+        if (row < N) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                float r = rintf(v[i][e] / sc);
+                r = fminf(fmaxf(r, -127.0f), 127.0f);
+                pk[e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
+            }
+        }
+        u32x2 o = {pk[0], pk[1]};
+        *reinterpret_cast<u32x2*>(codes + (bh * n_pad + row) * D + col) = o;
+    }
+}
+
+template <int D, bool IS_K>
+static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t n_pad, int blk,
+                                    float cmul, const float* mean, int8_t* codes, float* scales,
+                                    hipStream_t st) {
+    dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
+#define SAGE_LAUNCH_Q(BLK)                                                                    \
+    hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K>), grid, block, 0, st, x.p, x.sb, x.sh,   \
+                       x.sn, N, H, n_pad, cmul, mean, codes, scales)
+    switch (blk) {
+        case 32: SAGE_LAUNCH_Q(32); break;
+        case 64: SAGE_LAUNCH_Q(64); break;
+        case 128: SAGE_LAUNCH_Q(128); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef SAGE_LAUNCH_Q
+    return hipGetLastError();
+}
+
+hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad, int blk,
+                           bool is_k, float cmul, const float* mean, int8_t* codes,
+                           float* scales, hipStream_t st) {
+    if (n_pad % blk != 0) return hipErrorInvalidValue;
+    if (D == 128)
+        return is_k ? launch_quant_i8_d<128, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st)
+                    : launch_quant_i8_d<128, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st);
+    if (D == 64)
+        return is_k ? launch_quant_i8_d<64, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st)
+                    : launch_quant_i8_d<64, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st);
+    return hipErrorInvalidValue;
+}
+
+// ---------------------------------------------------------------------------
+// K mean.  Summation tree (all in fp64, every order fixed):
+//   leaf  = 16 consecutive tokens, added in ascending order by one lane
+//   group = 16 consecutive leaves, added in ascending order
+//   total = groups added in ascending order;  mean = fp32(total / N)
+// Kernel 1: one workgroup per (group, h, b); lane (leaf, 8-channel chunk).
+// Kernel 2: one thread per (b, h, channel).
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
+    const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int ngroups, double* __restrict__ partial) {
+    constexpr int CPR = D / 8;
+    const int g = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int leaf = tid / CPR, col = (tid % CPR) * 8;
+    const uint16_t* src = k + b * sb + h * sh + col;
+    const int s0 = g * kGroup + leaf * kLeaf;
+
+    u32x4 w[kLeaf];
+#pragma unroll
+    for (int i = 0; i < kLeaf; i++) {
+        w[i] = u32x4{0u, 0u, 0u, 0u};
+        if (s0 + i < N) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)(s0 + i) * sn);
+    }
+    double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < kLeaf; i++) {
+        float x[8];
+        unpack8(w[i], x);
+        // rows past N contribute +0.0, which leaves a double sum unchanged
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += (double)x[e];
+    }
+
+    __shared__ double leafsum[16][D + 2];
+#pragma unroll
+    for (int e = 0; e < 8; e++) leafsum[leaf][col + e] = acc[e];
+    __syncthreads();
+    if (tid < D) {
+        double gsum = 0.0;
+#pragma unroll
+        for (int u = 0; u < 16; u++) gsum += leafsum[u][tid];
+        partial[(((int64_t)b * H + h) * ngroups + g) * D + tid] = gsum;
+    }
+}
+
+__global__ __launch_bounds__(256) void kmean_final_kernel(
+    const double* __restrict__ partial, int ngroups, int D, int N, int64_t total,
+    float* __restrict__ kmean) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;      // (bh, d)
+    if (i >= total) return;
+    const int64_t bh = i / D;
+    const int d = (int)(i % D);
+    const double* p = partial + bh * ngroups * D + d;
+    double sum = 0.0;
+    for (int g = 0; g < ngroups; g++) sum += p[(int64_t)g * D];
+    kmean[i] = (float)(sum / (double)N);
+}
+
+hipError_t launch_kmean(const View& k, int B, int H, int N, int D, double* partial,
+                        float* kmean, hipStream_t st) {
+    const int ngroups = (N + kGroup - 1) / kGroup;
+    dim3 grid((unsigned)ngroups, (unsigned)H, (unsigned)B);
+    if (D == 128)
+        hipLaunchKernelGGL((kmean_group_kernel<128>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
+                           N, H, ngroups, partial);
+    else if (D == 64)
+        hipLaunchKernelGGL((kmean_group_kernel<64>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
+                           N, H, ngroups, partial);
+    else
+        return hipErrorInvalidValue;
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t total = (int64_t)B * H * D;
+    hipLaunchKernelGGL(kmean_final_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       partial, ngroups, D, N, total, kmean);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// V repack: bf16 [.., N, D] -> fp16 tiles [.., N/64, D, 64]; key k of a tile
+// goes to slot v_slot_f16(k).  One workgroup per (tile, h, b): rows are read
+// coalesced, staged in LDS and written back channel-major in 16-byte runs.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint16_t f32_to_f16_sat(float x) {
+    x = fminf(fmaxf(x, -65504.0f), 65504.0f);
+    return __half_as_ushort(__float2half_rn(x));
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void quant_v_f16_kernel(
+    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, uint16_t* __restrict__ out) {
+    constexpr int CPR = D / 8;
+    constexpr int LD = D + 8;                              // padded row (halves), keeps 16-byte alignment
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * LD];
+    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const uint16_t* src = v + b * sb + h * sh;
+#pragma unroll
+    for (int i = 0; i < 64 * CPR / 256; i++) {
+        const int c = i * 256 + tid;
+        const int key = c / CPR, col = (c % CPR) * 8;
+        const int row = t * 64 + key;
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (row < N) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+        float x[8];
+        unpack8(w, x);
+        u32x4 o;
+        o.x = f32_to_f16_sat(x[0]) | ((uint32_t)f32_to_f16_sat(x[1]) << 16);
+        o.y = f32_to_f16_sat(x[2]) | ((uint32_t)f32_to_f16_sat(x[3]) << 16);
+        o.z = f32_to_f16_sat(x[4]) | ((uint32_t)f32_to_f16_sat(x[5]) << 16);
+        o.w = f32_to_f16_sat(x[6]) | ((uint32_t)f32_to_f16_sat(x[7]) << 16);
+        *reinterpret_cast<u32x4*>(&tile[v_slot_f16(key) * LD + col]) = o;
+    }
+    __syncthreads();
+    uint16_t* dst = out + ((((int64_t)b * H + h) * (n_pad / 64)) + t) * (int64_t)(D * 64);
+    // output chunk = (channel d, 8 consecutive slots)
+#pragma unroll
+    for (int i = 0; i < D * 8 / 256; i++) {
+        const int c = i * 256 + tid;
+        const int d = c >> 3, s0 = (c & 7) * 8;
+        uint32_t pk[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            pk[e] = tile[(s0 + 2 * e) * LD + d] | ((uint32_t)tile[(s0 + 2 * e + 1) * LD + d] << 16);
+        *reinterpret_cast<u32x4*>(dst + d * 64 + s0) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+    }
+}
+
+hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t n_pad,
+                              uint16_t* v16, hipStream_t st) {
+    dim3 grid((unsigned)(n_pad / 64), (unsigned)H, (unsigned)B);
+    if (D == 128)
+        hipLaunchKernelGGL((quant_v_f16_kernel<128>), grid, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, v16);
+    else if (D == 64)
+        hipLaunchKernelGGL((quant_v_f16_kernel<64>), grid, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, v16);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// V e4m3 quantization with one scale per (b, h, channel).
+// Kernel 1: channel absmax over tokens (max is order-free; fp32 bit patterns of
+//           non-negative values order like unsigned integers, so atomicMax on
+//           the bits is exact).  vscale holds the amax bits until kernel 2.
+// Kernel 2: amax -> scale in place.  Kernel 3: encode into the tiled layout.
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void v_absmax_kernel(
+    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, uint32_t* __restrict__ amax_bits) {
+    constexpr int CPR = D / 8;
+    constexpr int ROWS = 256 / CPR;                        // rows covered per step
+    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int col = (tid % CPR) * 8, r = tid / CPR;
+    const uint16_t* src = v + b * sb + h * sh + col;
+    float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    // 256 tokens per workgroup
+#pragma unroll 4
+    for (int i = 0; i < 256 / ROWS; i++) {
+        const int row = t * 256 + i * ROWS + r;
+        if (row < N) {
+            u32x4 w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn);
+            float x[8];
+            unpack8(w, x);
+#pragma unroll
+            for (int e = 0; e < 8; e++) m[e] = fmaxf(m[e], fabsf(x[e]));
+        }
+    }
+    __shared__ float red[ROWS][D + 1];
+#pragma unroll
+    for (int e = 0; e < 8; e++) red[r][col + e] = m[e];
+    __syncthreads();
+    if (tid < D) {
+        float mm = 0.0f;
+        for (int i = 0; i < ROWS; i++) mm = fmaxf(mm, red[i][tid]);
+        atomicMax(amax_bits + ((int64_t)b * H + h) * D + tid, __float_as_uint(mm));
+    }
+}
+
+// Clears the amax accumulator with a kernel (not hipMemsetAsync) so that a caller can
+// capture the whole sequence into a HIP graph.
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* __restrict__ p, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) p[i] = 0u;
+}
+
+__global__ __launch_bounds__(256) void v_scale_kernel(float* __restrict__ vscale, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const float amax = vscale[i];                          // bits written by atomicMax
+    vscale[i] = amax > 0.0f ? amax / 448.0f : 1.0f;
+}
+
+// fp32 -> e4m3fn, round-to-nearest-even, saturating at +-448, NaN -> +-0.
+__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    float a = fabsf(x);
+    if (!(a == a)) return sign;
+    a = fminf(a, 448.0f);
+    uint32_t byte;
+    if (a < 0.015625f) {                                   // below 2^-6: quantum 2^-9
+        byte = (uint32_t)(int)rintf(a * 512.0f);           // 0..8; 8 is exactly code 0x08
+    } else {
+        const uint32_t au = __float_as_uint(a);
+        // keep 3 mantissa bits, round half to even on the 20 dropped bits
+        uint32_t r = au + 0x7FFFFu + ((au >> 20) & 1u);
+        r >>= 20;                                          // (biased exp << 3) | mant3, carry included
+        byte = r - ((127u - 7u) << 3);
+        if (byte > 0x7Eu) byte = 0x7Eu;
+    }
+    return byte | sign;
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void quant_v_fp8_kernel(
+    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, const float* __restrict__ vscale, uint8_t* __restrict__ out) {
+    constexpr int CPR = D / 8;
+    constexpr int LD = D + 16;                             // padded row (bytes)
+    __shared__ __attribute__((aligned(16))) uint8_t tile[64 * LD];
+    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int64_t bh = (int64_t)b * H + h;
+    const uint16_t* src = v + b * sb + h * sh;
+#pragma unroll
+    for (int i = 0; i < 64 * CPR / 256; i++) {
+        const int c = i * 256 + tid;
+        const int key = c / CPR, col = (c % CPR) * 8;
+        const int row = t * 64 + key;
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (row < N) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+        float x[8];
+        unpack8(w, x);
+        const float4 s0 = *reinterpret_cast<const float4*>(vscale + bh * D + col);
+        const float4 s1 = *reinterpret_cast<const float4*>(vscale + bh * D + col + 4);
+        const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 8; e++) pk[e >> 2] |= f32_to_e4m3(x[e] / sc[e]) << ((e & 3) * 8);
+        *reinterpret_cast<u32x2*>(&tile[v_slot_fp8(key) * LD + col]) = u32x2{pk[0], pk[1]};
+    }
+    __syncthreads();
+    uint8_t* dst = out + ((bh * (n_pad / 64)) + t) * (int64_t)(D * 64);
+    // output chunk = (channel d, 16 consecutive slots)
+#pragma unroll
+    for (int i = 0; i < D * 4 / 256; i++) {
+        const int c = i * 256 + tid;
+        const int d = c >> 2, s0 = (c & 3) * 16;
+        uint32_t pk[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 16; e++) pk[e >> 2] |= (uint32_t)tile[(s0 + e) * LD + d] << ((e & 3) * 8);
+        *reinterpret_cast<u32x4*>(dst + d * 64 + s0) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+    }
+}
+
+hipError_t launch_quant_v_fp8(const View& v, int B, int H, int N, int D, int64_t n_pad,
+                              uint8_t* v8, float* vscale, hipStream_t st) {
+    const int64_t total = (int64_t)B * H * D;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       reinterpret_cast<uint32_t*>(vscale), total);
+    dim3 g1((unsigned)((N + 255) / 256), (unsigned)H, (unsigned)B);
+    dim3 g3((unsigned)(n_pad / 64), (unsigned)H, (unsigned)B);
+    if (D == 128) {
+        hipLaunchKernelGGL((v_absmax_kernel<128>), g1, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H,
+                           reinterpret_cast<uint32_t*>(vscale));
+        hipLaunchKernelGGL(v_scale_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, vscale, total);
+        hipLaunchKernelGGL((quant_v_fp8_kernel<128>), g3, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, vscale, v8);
+    } else if (D == 64) {
+        hipLaunchKernelGGL((v_absmax_kernel<64>), g1, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H,
+                           reinterpret_cast<uint32_t*>(vscale));
+        hipLaunchKernelGGL(v_scale_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, vscale, total);
+        hipLaunchKernelGGL((quant_v_fp8_kernel<64>), g3, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, vscale, v8);
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace sage

@@ -312,13 +312,19 @@ int sage_oracle_kmean(const uint16_t* k, int B, int H, int N, int D,
         int h = (int)(w % H);
         int b = (int)(w / H);
         for (int d = 0; d < D; d++) {
+            /* fixed summation tree: 16-token leaves (tokens ascending), 16-leaf
+             * groups (leaves ascending), groups ascending */
             double sum = 0.0;
-            for (int t0 = 0; t0 < N; t0 += 64) {
-                int t1 = (t0 + 64 < N) ? t0 + 64 : N;
-                double part = 0.0;
-                for (int s = t0; s < t1; s++)
-                    part += (double)sage_oracle_bf16_to_f32(k[b * st[0] + h * st[1] + (int64_t)s * st[2] + d * st[3]]);
-                sum += part;
+            for (int g0 = 0; g0 < N; g0 += 256) {
+                double group = 0.0;
+                for (int u0 = g0; u0 < g0 + 256 && u0 < N; u0 += 16) {
+                    int u1 = (u0 + 16 < N) ? u0 + 16 : N;
+                    double leaf = 0.0;
+                    for (int s = u0; s < u1; s++)
+                        leaf += (double)sage_oracle_bf16_to_f32(k[b * st[0] + h * st[1] + (int64_t)s * st[2] + d * st[3]]);
+                    group += leaf;
+                }
+                sum += group;
             }
             kmean[w * D + d] = (float)(sum / (double)N);
         }

@@ -73,9 +73,12 @@ int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
                         const int64_t* strides, float scale, int blkq, int npad_mult,
                         int8_t* q8, float* qscale);
 
-/* K mean over tokens per (b,h,d): 64-token partial sums in double (tokens
- * ascending), partials added in ascending order, divided by N in double,
- * rounded once to fp32.  kmean: [B,H,D]. */
+/* K mean over tokens per (b,h,d) with a fixed summation tree in double:
+ * 16-token leaves (tokens ascending), groups of 16 leaves (ascending), groups
+ * ascending; the total is divided by N in double and rounded once to fp32.
+ * (Sums of bf16 values in double are exact unless one column spans more than
+ * ~2^40 in magnitude, so in practice any order gives these bits; the tree is
+ * what holds when it does not.)  kmean: [B,H,D]. */
 int sage_oracle_kmean(const uint16_t* k, int B, int H, int N, int D,
                       const int64_t* strides, float* kmean);
 

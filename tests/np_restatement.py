@@ -58,15 +58,18 @@ def kmean_exact(k_bits_bshd):
 
 
 def kmean_blocked(k_bits_bshd):
-    """The normative order: 64-token partials (ascending), partials ascending."""
+    """The normative order: 16-token leaves (ascending), 16-leaf groups, groups ascending."""
     x = bf16_to_f32(k_bits_bshd).transpose(0, 2, 1, 3).astype(np.float64)
     B, H, S, D = x.shape
     total = np.zeros((B, H, D))
-    for t0 in range(0, S, 64):
-        part = np.zeros((B, H, D))
-        for s in range(t0, min(S, t0 + 64)):
-            part = part + x[:, :, s, :]
-        total = total + part
+    for g0 in range(0, S, 256):
+        group = np.zeros((B, H, D))
+        for u0 in range(g0, min(S, g0 + 256), 16):
+            leaf = np.zeros((B, H, D))
+            for s in range(u0, min(S, u0 + 16)):
+                leaf = leaf + x[:, :, s, :]
+            group = group + leaf
+        total = total + group
     return (total / float(S)).astype(np.float32)
 
 

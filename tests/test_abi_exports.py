@@ -1,0 +1,93 @@
+"""CPU-side checks of the C ABI: the shared library loads without a GPU and
+exports every function include/mi355_sage.h declares; argument validation that
+needs no device returns the documented codes."""
+import ctypes
+import os
+import re
+
+from mojodiffusion_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "mi355_sage.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_sage_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = _declared_functions()
+    assert len(names) >= 12
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), "library does not export %s" % n
+    assert sorted(_lib.SIGNATURES) == names        # the Python binding covers the whole header
+
+
+def test_no_gpu_helpers():
+    L = _lib.lib()
+    assert L.mi355_sage_version().startswith(b"mi355_sage")
+    assert L.mi355_sage_pad_q(1) == 128 and L.mi355_sage_pad_q(4608) == 4608
+    assert L.mi355_sage_pad_kv(32760) == 32768
+    for variant in (0, 1):
+        slots = sorted(L.mi355_sage_v_slot(k, variant) for k in range(64))
+        assert slots == list(range(64))            # a permutation of the tile
+    assert L.mi355_sage_v_slot(64, 0) == -1
+    assert L.mi355_sage_workspace_bytes(1, 24, 4608, 4608, 128, 0) > 3 * 24 * 4608 * 128
+    assert L.mi355_sage_workspace_bytes(1, 24, 4608, 4608, 96, 0) == 0
+    assert L.mi355_sage_workspace_bytes(0, 24, 4608, 4608, 128, 0) == 0
+
+
+def test_argument_validation_without_device():
+    """Order and codes of serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393: null
+    pointers, non-positive dims, null strides -> -1 before anything touches a GPU."""
+    L = _lib.lib()
+    st = _lib.strides_bhnd(128, 2, 128)
+    fake = ctypes.c_void_p(4096)
+    ok_dims = (1, 2, 128, 128, 128)
+    call = lambda q, k, v, o, dims, s0: L.mi355_sage_sdpa_bf16(
+        q, k, v, o, *dims, 0.1, s0, st, st, st, 0, 0, 0, 0, 0, None, 0, None, 0)
+    assert call(None, fake, fake, fake, ok_dims, st) == -1
+    assert call(fake, fake, fake, None, ok_dims, st) == -1
+    assert call(fake, fake, fake, fake, (1, 0, 128, 128, 128), st) == -1
+    assert call(fake, fake, fake, fake, (1, 2, 128, -4, 128), st) == -1
+    assert call(fake, fake, fake, fake, ok_dims, None) == -1
+    # unsupported configurations -> -2
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
+                                  0, 0, 0, 0, 1, None, 0, None, 0) == -2          # causal
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 96, 0.1, st, st, st, st,
+                                  0, 0, 0, 0, 0, None, 0, None, 0) == -2          # head dim
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
+                                  0, 0, 0, 0, 0, None, 7, None, 0) == -2          # variant
+    bad = (ctypes.c_int64 * 4)(128 * 2 * 128, 128, 2 * 128, 2)
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, bad, st, st, st,
+                                  0, 0, 0, 0, 0, None, 0, None, 0) == -2          # strided head dim
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
+                                  3, 0, 0, 0, 0, None, 0, None, 0) == -2          # misaligned offset
+    # workspace too small -> -3 (checked before any launch)
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
+                                  0, 0, 0, 0, 0, None, 0, ctypes.c_void_p(256 * 64), 1024) == -3
+    assert L.mi355_sage_sdpa_bf16_train_fwd(fake, fake, fake, fake, None, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
+                                            0, 0, 0, 0, 0, 0, 128, 128, None, 0, None, 0) == -1   # Stats null
+
+
+def test_host_mirror_error_strings():
+    import pytest
+    import torch
+    from mojodiffusion_amd import attention_sage as A
+    q = torch.zeros((1, 128, 2, 64), dtype=torch.float32)
+    with pytest.raises(A.Error, match="q/k/v must be BF16"):
+        A.sdpa_flash_train_fwd(q, q, q, 0.1)
+    with pytest.raises(A.Error, match="sdpa_nomask: q/k/v dtype mismatch"):
+        A.sdpa_nomask(q, q.to(torch.bfloat16), q, 0.1)
+    with pytest.raises(A.Error, match=r"sdpa_nomask: q must be rank-4 \[B,S,H,Dh\]"):
+        A.sdpa_nomask(q[0], q[0], q[0], 0.1)
+    qb = torch.zeros((1, 100, 2, 64), dtype=torch.bfloat16)
+    with pytest.raises(A.Error, match="S_BUF must be 128-aligned"):
+        A.sdpa_flash_fwd_padmask(qb, qb, qb, 50, 0.1)
+    qb = torch.zeros((1, 128, 2, 64), dtype=torch.bfloat16)
+    with pytest.raises(A.Error, match=r"real_len out of \[1, S_BUF\]"):
+        A.sdpa_flash_fwd_padmask(qb, qb, qb, 0, 0.1)
+    with pytest.raises(A.Error, match="no CPU fallback"):
+        A.sdpa_nomask(qb, qb, qb, 0.1)

@@ -1,0 +1,128 @@
+"""GPU parity of the quantize kernels, through the C ABI, against the CPU
+checker: INT8 codes, fp32 scales, the K mean, fp16 / e4m3 V and V scales must
+be bit-identical."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from mojodiffusion_amd import _lib
+from mojodiffusion_amd.workloads import WORKLOADS, make_inputs, f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_qk(oracle, H, q, k, scale, blkq, blkk, smooth):
+    g = H.quant_qk(q, k, scale, blkq, blkk, smooth)
+    Sq, Skv = q.shape[1], k.shape[1]
+    q8, qs = oracle.quant_q(q, scale, blkq, 128)
+    mu = oracle.kmean(k) if smooth else None
+    k8, ks = oracle.quant_k(k, mu, blkk, 64)
+    if smooth:
+        np.testing.assert_array_equal(g["kmean"].view(np.uint32), mu.view(np.uint32))
+    nqb, nkb = qs.shape[2], ks.shape[2]
+    np.testing.assert_array_equal(g["qscale"][:, :, :nqb].view(np.uint32), qs.view(np.uint32))
+    np.testing.assert_array_equal(g["kscale"][:, :, :nkb].view(np.uint32), ks.view(np.uint32))
+    assert np.all(g["qscale"][:, :, nqb:] == 1.0) and np.all(g["kscale"][:, :, nkb:] == 1.0)
+    np.testing.assert_array_equal(g["q8"], q8)           # includes the zero pad rows
+    np.testing.assert_array_equal(g["k8"], k8)
+    return g
+
+
+@pytest.mark.parametrize("wid", [1, 2, 3, 4])
+def test_quant_qk_bit_exact_workload_stats(oracle, wid):
+    import gpu_harness as H
+    w = WORKLOADS[wid]
+    w = w if wid == 1 else w.scaled(B=w.B, H=3, S=1100)      # ragged: 1100 = 8*128 + 76 = 17*64 + 12
+    q, k, _ = make_inputs(w)
+    _check_qk(oracle, H, q, k, w.scale, w.blkq, w.blkk, True)
+
+
+@pytest.mark.parametrize("D,blkq,blkk,S,smooth", [
+    (64, 32, 32, 96, True), (64, 128, 128, 300, False), (128, 32, 64, 1, True),
+    (128, 64, 32, 65, True), (128, 128, 64, 257, False), (64, 64, 64, 1024, True)])
+def test_quant_qk_bit_exact_shapes(oracle, D, blkq, blkk, S, smooth):
+    import gpu_harness as H
+    rng = np.random.default_rng(S * 7 + D)
+    q = f32_to_bf16_bits(rng.standard_normal((2, S, 2, D)).astype(np.float32))
+    k = f32_to_bf16_bits((rng.standard_normal((2, S, 2, D)) * 3 + rng.standard_normal((2, 1, 2, D)) * 5).astype(np.float32))
+    _check_qk(oracle, H, q, k, 0.2, blkq, blkk, smooth)
+
+
+def test_quant_qk_ties_zero_blocks_and_extremes(oracle):
+    """Adversarial inputs: exact .5 ties (absmax 127 -> scale 1), an all-zero
+    block, subnormal-scale blocks and bf16 extremes."""
+    import gpu_harness as H
+    D, S = 64, 256
+    x = np.zeros((1, S, 1, D), np.float32)
+    ties = np.float32([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, 64.5, -126.5, 126.5, 0.25, 0.75, -0.75])
+    x[0, 0, 0, :len(ties)] = ties                         # block 0: ties
+    # block 1 (rows 64..127): all zero
+    x[0, 128:192] = np.random.default_rng(5).standard_normal((64, 1, D)) * 1e-30      # block 2: tiny values
+    x[0, 192:256] = np.random.default_rng(6).standard_normal((64, 1, D)) * 1e30       # block 3: huge values
+    k = f32_to_bf16_bits(x)
+    q = f32_to_bf16_bits(np.random.default_rng(7).standard_normal((1, S, 1, D)).astype(np.float32))
+    g = _check_qk(oracle, H, q, k, 1.0, 64, 64, False)
+    assert g["kscale"][0, 0, 0] == 1.0 and g["kscale"][0, 0, 1] == 1.0
+    np.testing.assert_array_equal(g["k8"][0, 0, 0, :len(ties)],
+                                  np.int8([127, 0, 2, 2, 0, -2, -2, 64, 64, -126, 126, 0, 1, -1]))
+
+
+def test_quant_qk_bhsd_strides_and_offsets(oracle):
+    """The same logical tensor presented head-major ([B,H,S,D] memory) and at a
+    non-zero element offset inside a larger buffer gives identical codes."""
+    import gpu_harness as H
+    rng = np.random.default_rng(21)
+    B, S, Hh, D = 2, 200, 3, 128
+    q = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32))
+    k = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32) + 2.0)
+    ref = H.quant_qk(q, k, 0.1, 128, 64, True)
+    off = 64
+    def bhsd_buf(x):
+        flat = np.zeros(off + x.size, np.uint16)
+        flat[off:] = np.ascontiguousarray(x.transpose(0, 2, 1, 3)).reshape(-1)
+        return flat
+    st = (ctypes.c_int64 * 4)(Hh * S * D, S * D, D, 1)
+    got = H.quant_qk(bhsd_buf(q), bhsd_buf(k), 0.1, 128, 64, True, strides_q=st, strides_k=st,
+                     q_off=off, k_off=off, shape=(B, Hh, S, S, D))
+    for name in ("q8", "qscale", "k8", "kscale", "kmean"):
+        np.testing.assert_array_equal(got[name], ref[name])
+
+
+@pytest.mark.parametrize("D,S", [(128, 1100), (64, 1024), (128, 64), (64, 7)])
+def test_quant_v_bit_exact(oracle, D, S):
+    import gpu_harness as H
+    rng = np.random.default_rng(S + D)
+    x = rng.standard_normal((2, S, 3, D)).astype(np.float32) * np.exp(rng.uniform(-3, 3, (1, 1, 3, D))).astype(np.float32)
+    x[:, :, 1, 5] = 0.0                                    # all-zero channel -> scale 1.0
+    if S > 10:
+        x[0, 3, 0, 0] = 1e6                                # beyond fp16 range: saturates
+    v = f32_to_bf16_bits(x)
+    g0 = H.quant_v(v, 0)
+    np.testing.assert_array_equal(H.untile_v(g0["vq"], 0), oracle.quant_v_f16(v, 64))
+    g1 = H.quant_v(v, 1)
+    v8, vs = oracle.quant_v_fp8(v, 64)
+    np.testing.assert_array_equal(g1["vscale"].view(np.uint32), vs.view(np.uint32))
+    np.testing.assert_array_equal(H.untile_v(g1["vq"], 1), v8)
+
+
+def test_quant_full_size_properties():
+    """Workload 2 at full size: size-independent properties of the device output
+    (no CPU pass over 14 M elements per tensor needed)."""
+    import torch
+    import gpu_harness as H
+    w = WORKLOADS[2]
+    q, k, _ = make_inputs(w)
+    g = H.quant_qk(q, k, w.scale, w.blkq, w.blkk, True)
+    q8, k8 = g["q8"].astype(np.int32), g["k8"].astype(np.int32)
+    # every block's absmax code is exactly 127 and -128 never appears
+    assert np.all(np.abs(q8).reshape(w.B, w.H, -1, w.blkq * w.D).max(-1) == 127)
+    assert np.all(np.abs(k8).reshape(w.B, w.H, -1, w.blkk * w.D).max(-1) == 127)
+    assert q8.min() >= -127 and k8.min() >= -127
+    # dequantised K + mean reproduces K within half a step per element
+    kf = (k.astype(np.uint32) << 16).view(np.float32).transpose(0, 2, 1, 3)
+    deq = k8 * np.repeat(g["kscale"], w.blkk, axis=2)[..., None] + g["kmean"][:, :, None, :]
+    step = np.repeat(g["kscale"], w.blkk, axis=2)[..., None]
+    assert np.all(np.abs(deq - kf) <= 0.5 * step * (1 + 1e-5) + 1e-6)
+    # the mean is the column mean
+    np.testing.assert_allclose(g["kmean"], kf.astype(np.float64).mean(2), rtol=0, atol=1e-6)

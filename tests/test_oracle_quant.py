@@ -69,16 +69,16 @@ def test_kmean_exact_and_blocked(oracle, S):
 
 def test_kmean_order_is_the_blocked_one(oracle):
     """With a magnitude spread beyond 2^53 the order matters; the oracle must
-    follow the 64-token-partials order, not a straight running sum."""
-    S, D = 192, 1
+    follow the leaf/group tree, not a straight running sum."""
+    S, D = 48, 1
     x = np.zeros((1, S, 1, D), np.float32)
     x[0, 0] = 2.0 ** 60
-    x[0, 1:64] = 1.0                                  # lost inside block 0 (absorbed by 2^60)
-    x[0, 64] = -(2.0 ** 60)
-    x[0, 65:192] = 1.0                                # block 1: absorbed; block 2: 64 survives
+    x[0, 1:16] = 1.0                                  # leaf 0: absorbed by 2^60
+    x[0, 16] = -(2.0 ** 60)
+    x[0, 17:48] = 1.0                                 # leaf 1: absorbed; leaf 2: 16 survives
     mu = oracle.kmean(f32_to_bf16_bits(x))
     np.testing.assert_array_equal(mu, R.kmean_blocked(f32_to_bf16_bits(x)))
-    assert mu[0, 0, 0] == np.float32(64.0 / S)
+    assert mu[0, 0, 0] == np.float32(16.0 / S)
 
 
 @pytest.mark.parametrize("wid", [1, 2, 3])
