@@ -127,7 +127,7 @@ size_t mi355_sage_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int va
  *   vscale  fp32  [B, H, D]
  * ---------------------------------------------------------------------- */
 int64_t mi355_sage_pad_q(int64_t n);    /* query tokens round up to the query tile  */
-int64_t mi355_sage_pad_kv(int64_t n);   /* key tokens round up to the key tile      */
+int64_t mi355_sage_pad_kv(int64_t n);   /* key tokens round up to 128               */
 int     mi355_sage_v_slot(int key_in_tile, int variant);
 
 /* Bytes of scratch mi355_sage_quant_qk_bf16 / _quant_v_fp8 need (partial sums). */

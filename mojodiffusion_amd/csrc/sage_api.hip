@@ -58,7 +58,7 @@ struct Carve {
 
 Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     const size_t bh = (size_t)B * H;
-    const size_t nqp = (size_t)pad_to(Nq, kTileQ), nkp = (size_t)pad_to(Nkv, kTileKV);
+    const size_t nqp = (size_t)pad_to(Nq, kTileQ), nkp = (size_t)pad_to(Nkv, kPadKV);
     Carve c{};
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
@@ -107,7 +107,7 @@ int quant_qk(const View& q, const View& k, int B, int H, int Nq, int Nkv, int D,
     const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
     SAGE_HIP(launch_quant_i8(q, B, H, Nq, D, pad_to(Nq, kTileQ), blkq, false, cmul, nullptr, q8, qscale, st));
     if (smooth_k) SAGE_HIP(launch_kmean(k, B, H, Nkv, D, partial, kmean, st));
-    SAGE_HIP(launch_quant_i8(k, B, H, Nkv, D, pad_to(Nkv, kTileKV), blkk, true, 0.0f,
+    SAGE_HIP(launch_quant_i8(k, B, H, Nkv, D, pad_to(Nkv, kPadKV), blkk, true, 0.0f,
                              smooth_k ? kmean : nullptr, k8, kscale, st));
     return 0;
 }
@@ -161,7 +161,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if ((rc = quant_qk(q, k, B, H, N_q, kv, D, scale, blkq, blkk, smooth_k, q8, qscale, k8, kscale,
                        kmean, partial, st)))
         return rc;
-    const int64_t nkp = pad_to(kv, kTileKV);
+    const int64_t nkp = pad_to(kv, kPadKV);
     if (variant == MI355_SAGE_PV_FP16)
         SAGE_HIP(launch_quant_v_f16(v, B, H, kv, D, nkp, static_cast<uint16_t*>(vq), st));
     else
@@ -187,7 +187,7 @@ extern "C" {
 const char* mi355_sage_version(void) { return "mi355_sage 0.1 gfx950"; }
 
 int64_t mi355_sage_pad_q(int64_t n) { return pad_to(n, kTileQ); }
-int64_t mi355_sage_pad_kv(int64_t n) { return pad_to(n, kTileKV); }
+int64_t mi355_sage_pad_kv(int64_t n) { return pad_to(n, kPadKV); }
 
 int mi355_sage_v_slot(int key_in_tile, int variant) {
     if (key_in_tile < 0 || key_in_tile >= kTileKV) return -1;
@@ -272,7 +272,7 @@ int mi355_sage_quant_v_f16(const void* V, int B, int H, int N_kv, int D, const i
     if (!dims_ok(D)) return MI355_SAGE_EUNSUPPORTED;
     int rc;
     if ((rc = check_view("V", V, v_strides, v_off))) return rc;
-    SAGE_HIP(launch_quant_v_f16(make_view(V, v_strides, v_off), B, H, N_kv, D, pad_to(N_kv, kTileKV),
+    SAGE_HIP(launch_quant_v_f16(make_view(V, v_strides, v_off), B, H, N_kv, D, pad_to(N_kv, kPadKV),
                                 static_cast<uint16_t*>(v16), static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
 }
@@ -284,7 +284,7 @@ int mi355_sage_quant_v_fp8(const void* V, int B, int H, int N_kv, int D, const i
     if (!dims_ok(D)) return MI355_SAGE_EUNSUPPORTED;
     int rc;
     if ((rc = check_view("V", V, v_strides, v_off))) return rc;
-    SAGE_HIP(launch_quant_v_fp8(make_view(V, v_strides, v_off), B, H, N_kv, D, pad_to(N_kv, kTileKV),
+    SAGE_HIP(launch_quant_v_fp8(make_view(V, v_strides, v_off), B, H, N_kv, D, pad_to(N_kv, kPadKV),
                                 static_cast<uint8_t*>(v8), static_cast<float*>(vscale),
                                 static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
@@ -308,7 +308,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     a.vq = vq; a.vscale = static_cast<const float*>(vscale); a.kmean = nullptr;
     a.variant = variant;
     a.B = B; a.H = H; a.Nq = N_q; a.Nkv = N_kv; a.kv_valid = kv_valid; a.D = D;
-    a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(N_kv, kTileKV);
+    a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(N_kv, kPadKV);
     a.o = static_cast<uint16_t*>(O) + o_off; a.osb = o_strides[0]; a.osh = o_strides[1]; a.osn = o_strides[2];
     a.stats = static_cast<float*>(stats);
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));

@@ -10,6 +10,7 @@ namespace sage {
 // Tile geometry of the attention kernel; the quantized layouts are padded to it.
 constexpr int kTileQ  = 128;   // query rows per workgroup
 constexpr int kTileKV = 64;    // keys per main-loop iteration
+constexpr int kPadKV  = 128;   // key tokens are padded to this (every scale-block size divides it)
 constexpr int kLeaf   = 16;    // tokens per leaf of the K-mean summation tree
 constexpr int kGroup  = 256;   // tokens per group (16 leaves)
 

@@ -15,11 +15,11 @@ COS = 0.999
 
 def _oracle_quantized(oracle, q, k, v, w, variant):
     q8, qs = oracle.quant_q(q, w.scale, w.blkq, 128)
-    k8, ks = oracle.quant_k(k, oracle.kmean(k), w.blkk, 64)
+    k8, ks = oracle.quant_k(k, oracle.kmean(k), w.blkk, 128)
     if variant == 0:
-        vq, vs = oracle.quant_v_f16(v, 64), None
+        vq, vs = oracle.quant_v_f16(v, 128), None
     else:
-        vq, vs = oracle.quant_v_fp8(v, 64)
+        vq, vs = oracle.quant_v_fp8(v, 128)
     return q8, qs, k8, ks, vq, vs
 
 

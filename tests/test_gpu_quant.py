@@ -17,7 +17,7 @@ def _check_qk(oracle, H, q, k, scale, blkq, blkk, smooth):
     Sq, Skv = q.shape[1], k.shape[1]
     q8, qs = oracle.quant_q(q, scale, blkq, 128)
     mu = oracle.kmean(k) if smooth else None
-    k8, ks = oracle.quant_k(k, mu, blkk, 64)
+    k8, ks = oracle.quant_k(k, mu, blkk, 128)
     if smooth:
         np.testing.assert_array_equal(g["kmean"].view(np.uint32), mu.view(np.uint32))
     nqb, nkb = qs.shape[2], ks.shape[2]
@@ -99,9 +99,9 @@ def test_quant_v_bit_exact(oracle, D, S):
         x[0, 3, 0, 0] = 1e6                                # beyond fp16 range: saturates
     v = f32_to_bf16_bits(x)
     g0 = H.quant_v(v, 0)
-    np.testing.assert_array_equal(H.untile_v(g0["vq"], 0), oracle.quant_v_f16(v, 64))
+    np.testing.assert_array_equal(H.untile_v(g0["vq"], 0), oracle.quant_v_f16(v, 128))
     g1 = H.quant_v(v, 1)
-    v8, vs = oracle.quant_v_fp8(v, 64)
+    v8, vs = oracle.quant_v_fp8(v, 128)
     np.testing.assert_array_equal(g1["vscale"].view(np.uint32), vs.view(np.uint32))
     np.testing.assert_array_equal(H.untile_v(g1["vq"], 1), v8)
 
