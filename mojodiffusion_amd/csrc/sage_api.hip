@@ -53,7 +53,7 @@ bool blk_ok(int blk) { return blk == 32 || blk == 64 || blk == 128; }
 
 // Workspace layout of the one-shot calls.
 struct Carve {
-    size_t q8, k8, vq, qscale, kscale, kmean, vscale, partial, total;
+    size_t q8, k8, vq, qscale, kscale, kmean, vscale, partial, qshift, total;
 };
 
 Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
@@ -70,6 +70,7 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.kmean = take(bh * D * sizeof(float));
     c.vscale = take(bh * D * sizeof(float));
     c.partial = take(bh * ((Nkv + kGroup - 1) / kGroup) * D * sizeof(double));
+    c.qshift = take(bh * nqp * sizeof(float));
     c.total = off;
     return c;
 }
@@ -103,12 +104,13 @@ int internal_workspace(size_t need, void** out) {
 
 int quant_qk(const View& q, const View& k, int B, int H, int Nq, int Nkv, int D, float scale,
              int blkq, int blkk, int smooth_k, int8_t* q8, float* qscale, int8_t* k8, float* kscale,
-             float* kmean, double* partial, hipStream_t st) {
+             float* kmean, double* partial, float* qshift, hipStream_t st) {
     const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
-    SAGE_HIP(launch_quant_i8(q, B, H, Nq, D, pad_to(Nq, kTileQ), blkq, false, cmul, nullptr, q8, qscale, st));
     if (smooth_k) SAGE_HIP(launch_kmean(k, B, H, Nkv, D, partial, kmean, st));
+    SAGE_HIP(launch_quant_i8(q, B, H, Nq, D, pad_to(Nq, kTileQ), blkq, false, cmul, kmean, q8, qscale,
+                             smooth_k ? qshift : nullptr, st));
     SAGE_HIP(launch_quant_i8(k, B, H, Nkv, D, pad_to(Nkv, kPadKV), blkk, true, 0.0f,
-                             smooth_k ? kmean : nullptr, k8, kscale, st));
+                             smooth_k ? kmean : nullptr, k8, kscale, nullptr, st));
     return 0;
 }
 
@@ -156,10 +158,11 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     float* kmean = reinterpret_cast<float*>(ws + c.kmean);
     float* vscale = reinterpret_cast<float*>(ws + c.vscale);
     double* partial = reinterpret_cast<double*>(ws + c.partial);
+    float* qshift = Stats ? reinterpret_cast<float*>(ws + c.qshift) : nullptr;
 
     const View q = make_view(Q, qs, q_off), k = make_view(K, ks, k_off), v = make_view(V, vs, v_off);
     if ((rc = quant_qk(q, k, B, H, N_q, kv, D, scale, blkq, blkk, smooth_k, q8, qscale, k8, kscale,
-                       kmean, partial, st)))
+                       kmean, partial, qshift, st)))
         return rc;
     const int64_t nkp = pad_to(kv, kPadKV);
     if (variant == MI355_SAGE_PV_FP16)
@@ -170,7 +173,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     AttnArgs a{};
     a.q8 = q8; a.qscale = qscale; a.blkq = blkq;
     a.k8 = k8; a.kscale = kscale; a.blkk = blkk;
-    a.vq = vq; a.vscale = vscale; a.kmean = smooth_k ? kmean : nullptr;
+    a.vq = vq; a.vscale = vscale; a.qshift = smooth_k ? qshift : nullptr;
     a.variant = variant;
     a.B = B; a.H = H; a.Nq = N_q; a.Nkv = kv; a.kv_valid = kv; a.D = D;
     a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = nkp;
@@ -262,7 +265,7 @@ int mi355_sage_quant_qk_bf16(const void* Q, const void* K, int B, int H, int N_q
     return quant_qk(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), B, H, N_q, N_kv, D,
                     scale, blkq, blkk, smooth_k, static_cast<int8_t*>(q8), static_cast<float*>(qscale),
                     static_cast<int8_t*>(k8), static_cast<float*>(kscale), static_cast<float*>(kmean),
-                    static_cast<double*>(scratch), static_cast<hipStream_t>(stream));
+                    static_cast<double*>(scratch), nullptr, static_cast<hipStream_t>(stream));
 }
 
 int mi355_sage_quant_v_f16(const void* V, int B, int H, int N_kv, int D, const int64_t* v_strides,
@@ -305,7 +308,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     AttnArgs a{};
     a.q8 = static_cast<const int8_t*>(q8); a.qscale = static_cast<const float*>(qscale); a.blkq = blkq;
     a.k8 = static_cast<const int8_t*>(k8); a.kscale = static_cast<const float*>(kscale); a.blkk = blkk;
-    a.vq = vq; a.vscale = static_cast<const float*>(vscale); a.kmean = nullptr;
+    a.vq = vq; a.vscale = static_cast<const float*>(vscale); a.qshift = nullptr;
     a.variant = variant;
     a.B = B; a.H = H; a.Nq = N_q; a.Nkv = N_kv; a.kv_valid = kv_valid; a.D = D;
     a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(N_kv, kPadKV);

@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
-    const float* __restrict__ kmean,
+    const float* __restrict__ qshift,
     int H, int Nq, int kv_valid, int64_t nq_pad, int64_t nkv_pad,
     uint16_t* __restrict__ o, int64_t osb, int64_t osh, int64_t osn,
     float* __restrict__ stats, int n_qtiles, int total_wg) {
@@ -248,13 +248,8 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
             }
         if (STATS && half == 0) {
             // natural-log log-sum-exp of the scaled scores.  With K smoothing every score
-            // of a row was lowered by q.mean, which is added back from the int8 query.
-            float shift = 0.0f;
-            if (kmean != nullptr) {
-                const int8_t* qp = q8 + (bh * nq_pad + qrow) * D;
-                for (int d = 0; d < D; d++) shift += (float)qp[d] * kmean[bh * D + d];
-                shift *= sq;
-            }
+            // of a row was lowered by <q, mean>, which the Q quantizer recorded per row.
+            const float shift = qshift != nullptr ? qshift[bh * nq_pad + qrow] : 0.0f;
             stats[bh * Nq + qrow] = (m_run + __builtin_amdgcn_logf(l_tot) + shift) * 0.6931471805599453f;
         }
     }
@@ -268,11 +263,11 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     dim3 grid((unsigned)total), block(256);
     if (a.stats != nullptr)
         hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, true>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
-                           a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.kmean, a.H, a.Nq,
+                           a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
                            a.kv_valid, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
     else
         hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, false>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
-                           a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.kmean, a.H, a.Nq,
+                           a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
                            a.kv_valid, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
     return hipGetLastError();
 }

@@ -24,9 +24,11 @@ struct View {
 
 // ---- quantize kernels (sage_quant.hip) -------------------------------------
 // Q (is_k = false): x = f32(q)*cmul.  K (is_k = true): x = f32(k) - mean (mean may be null).
+// rowdot (Q only, may be null): [B,H,n_pad] <pre-scaled q row, mean>, needed for the
+// log-sum-exp output when K is smoothed.
 hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad,
                            int blk, bool is_k, float cmul, const float* mean,
-                           int8_t* codes, float* scales, hipStream_t st);
+                           int8_t* codes, float* scales, float* rowdot, hipStream_t st);
 
 // K mean: group partials (double, [B,H,ngroups,D]) then the final mean.
 hipError_t launch_kmean(const View& k, int B, int H, int N, int D,
@@ -42,7 +44,7 @@ hipError_t launch_quant_v_fp8(const View& v, int B, int H, int N, int D, int64_t
 struct AttnArgs {
     const int8_t* q8;  const float* qscale;  int blkq;
     const int8_t* k8;  const float* kscale;  int blkk;
-    const void* vq;    const float* vscale;  const float* kmean;   // kmean only for stats
+    const void* vq;    const float* vscale;  const float* qshift;  // qshift [B,H,nq_pad], stats only
     int variant;
     int B, H, Nq, Nkv, kv_valid, D;
     int64_t nq_pad, nkv_pad;

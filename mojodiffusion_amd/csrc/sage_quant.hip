@@ -40,7 +40,7 @@ template <int D, int BLK, bool IS_K>
 __global__ __launch_bounds__(256) void quant_i8_kernel(
     const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
-    int8_t* __restrict__ codes, float* __restrict__ scales) {
+    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot) {
     constexpr int CPR = D / 8;                 // 16-byte chunks per row
     constexpr int NCH = BLK * CPR / 256;       // chunks per thread
     static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
@@ -69,6 +69,17 @@ __global__ __launch_bounds__(256) void quant_i8_kernel(
         } else {
 #pragma unroll
             for (int e = 0; e < 8; e++) v[i][e] *= cmul;
+            if (rowdot != nullptr) {
+                // <pre-scaled query row, K mean>: the amount K smoothing lowers every score
+                // of this row by; the CPR lanes that share a row are adjacent in the wave.
+                const float4 m0 = *reinterpret_cast<const float4*>(mean + bh * D + col);
+                const float4 m1 = *reinterpret_cast<const float4*>(mean + bh * D + col + 4);
+                float dot = v[i][0] * m0.x + v[i][1] * m0.y + v[i][2] * m0.z + v[i][3] * m0.w +
+                            v[i][4] * m1.x + v[i][5] * m1.y + v[i][6] * m1.z + v[i][7] * m1.w;
+#pragma unroll
+                for (int off = CPR / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+                if ((tid % CPR) == 0) rowdot[bh * n_pad + row] = dot;
+            }
         }
         if (row < N) {
 #pragma unroll
@@ -107,11 +118,11 @@ __global__ __launch_bounds__(256) void quant_i8_kernel(
 template <int D, bool IS_K>
 static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t n_pad, int blk,
                                     float cmul, const float* mean, int8_t* codes, float* scales,
-                                    hipStream_t st) {
+                                    float* rowdot, hipStream_t st) {
     dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
 #define SAGE_LAUNCH_Q(BLK)                                                                    \
     hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K>), grid, block, 0, st, x.p, x.sb, x.sh,   \
-                       x.sn, N, H, n_pad, cmul, mean, codes, scales)
+                       x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot)
     switch (blk) {
         case 32: SAGE_LAUNCH_Q(32); break;
         case 64: SAGE_LAUNCH_Q(64); break;
@@ -124,14 +135,14 @@ static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t 
 
 hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad, int blk,
                            bool is_k, float cmul, const float* mean, int8_t* codes,
-                           float* scales, hipStream_t st) {
+                           float* scales, float* rowdot, hipStream_t st) {
     if (n_pad % blk != 0) return hipErrorInvalidValue;
     if (D == 128)
-        return is_k ? launch_quant_i8_d<128, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st)
-                    : launch_quant_i8_d<128, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st);
+        return is_k ? launch_quant_i8_d<128, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st)
+                    : launch_quant_i8_d<128, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st);
     if (D == 64)
-        return is_k ? launch_quant_i8_d<64, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st)
-                    : launch_quant_i8_d<64, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, st);
+        return is_k ? launch_quant_i8_d<64, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st)
+                    : launch_quant_i8_d<64, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st);
     return hipErrorInvalidValue;
 }
 
