@@ -15,13 +15,20 @@
 // B-operand fragment of the second product once V^T is stored with its keys in
 // the matching slot order (v_slot_f16 / v_slot_fp8).
 //
-// K and V^T tiles of 64 keys are double-buffered in LDS with a 16-byte-chunk
-// XOR swizzle; the next tile's global loads are issued before the current
-// tile's math.  Scores are in the log2 domain (scale*log2(e) is folded into the
-// Q quantizer), so the exponential is a bare v_exp_f32.
+// Pipeline.  K and V^T tiles of 64 keys travel global -> LDS with register-
+// bypassing copies (global_load_lds_dwordx4) into 3-deep rings; the 16-byte-chunk
+// XOR swizzle is applied on the source side of the copy.  Iteration t computes
+// the scores of tile t, then interleaves — one matrix instruction, then the
+// exponentials of two scores, in program order — the softmax of tile t with
+// P.V of tile t-1, so the matrix pipe and the vector ALU of a SIMD run
+// together inside one wave; the second wave on the SIMD covers what is left.
+// Scores are in the log2 domain (scale*log2(e) is folded into the Q
+// quantizer), so the exponential is a bare v_exp_f32.
 #include "sage_internal.h"
 
 #include <hip/hip_fp16.h>
+
+#include <type_traits>
 
 namespace sage {
 
@@ -32,10 +39,13 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 
-// Byte offset of 16-byte chunk L of a tile whose rows are grouped into 128-byte
-// super-rows: chunk position inside the super-row is XORed with the super-row index.
-__device__ __forceinline__ int swz(int L) { return (((L >> 3) << 3) | ((L & 7) ^ ((L >> 3) & 7))) << 4; }
+// Byte offset of 16-byte chunk L of a tile.  Chunks are grouped into 128-byte super-rows
+// (8 chunks); the chunk position inside a super-row is XORed with bits of the index of
+// the PAIR of super-rows it belongs to, so that the 16 lanes the 64-bank LDS serves per
+// cycle (16 consecutive rows, one logical column) land in 16 different 16-byte bank groups.
+__device__ __forceinline__ int swz(int L) { return (((L >> 3) << 3) | ((L & 7) ^ ((L >> 4) & 7))) << 4; }
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     uint32_t u = __float_as_uint(f);
@@ -43,6 +53,42 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     u += 0x7FFFu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
 }
+
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave lands at
+// lds_base + 16*l.  Written as assembly on purpose: the compiler then keeps no record of
+// an outstanding LDS write and does not put a full vector-memory wait in front of every
+// later LDS read; completion is awaited explicitly (dma_wait) before the workgroup
+// barrier that publishes the tile.
+__device__ __forceinline__ void dma16(const void* gbase_uniform, uint32_t goff, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base_uniform), "v"(goff), "s"(gbase_uniform)
+                 : "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+// The int32 score accumulators start at the bit pattern of 1.5*2^23 instead of 0, so a
+// finished accumulator, read as fp32, IS the float 12582912 + dot (exact while
+// |dot| < 2^22; the largest possible |dot| is 128*127*127 < 2^21): no int->float
+// conversion is needed and dequantisation, max subtraction and the exponent argument
+// collapse into one FMA per score.
+constexpr int kMagicI = 0x4B400000;
+constexpr float kMagicF = 12582912.0f;
+
+// A row's reference maximum is only refreshed (and the accumulators rescaled) when a tile
+// exceeds it by more than tau powers of two; until then p = exp2(s - m_used) may reach
+// 2^tau.  fp16 P holds 2^8 without loss.  The e4m3 variant maps p = 2^tau to the format
+// maximum 448, i.e. it stores e4m3(p * 448 / 2^tau); the factor cancels against the
+// normaliser, which sums the same scaled values.  tau = 1 keeps all but one binade of the
+// e4m3 range below p = 1.
+template <int VARIANT> struct Lazy {
+    static constexpr float tau = VARIANT == 0 ? 8.0f : 1.0f;
+    static constexpr float log2_pscale = VARIANT == 0 ? 0.0f : 7.807354922057604f;     // log2(448 / 2)
+};
 
 template <int D, int VARIANT, bool STATS>
 __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
@@ -62,9 +108,19 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     constexpr int V_CH = V_BYTES / 16 / 256;
     constexpr int K_CPR = D / 16;                       // chunks per K row
     constexpr int V_CPR = kTileKV * VB / 16;            // chunks per V^T row
+    constexpr int VROW = kTileKV * VB;                  // bytes per V^T row
+    constexpr int NS = 3;                               // LDS ring depth
+    constexpr int JS = VARIANT == 0 ? 4 : 1;            // PV steps over the 64 keys of a tile
+    constexpr int NUNIT = JS * DB;                      // PV matrix instructions per tile
+    constexpr int EPU = 32 / NUNIT;                     // scores exponentiated per PV instruction
+    constexpr int FPU = VARIANT == 0 ? 1 : 2;           // 16-byte V fragments per PV instruction
+    constexpr int PD = VARIANT == 0 ? 2 : 1;            // V fragment prefetch distance (units)
+    constexpr int PW = VARIANT == 0 ? 16 : 8;           // dwords of packed P per tile
+    static_assert(32 % NUNIT == 0 && EPU % 2 == 0, "unit split");
 
-    __shared__ __attribute__((aligned(16))) uint8_t lds_k[2][K_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_v[2][V_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NS][K_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NS][V_BYTES];
+    __shared__ float lds_ks[1024];
 
     // Workgroup -> (q tile, b*h).  Hardware hands consecutive workgroup ids to the 8
     // XCDs round-robin; give each XCD a contiguous range of (head, q tile) work so the
@@ -80,7 +136,8 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     const int64_t bh = wg / n_qtiles;
     const int b = (int)(bh / H), h = (int)(bh % H);
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
     const int qrow = qt * kTileQ + wave * 32 + l32;     // this lane's query (padded index)
 
@@ -92,141 +149,301 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
         for (int s = 0; s < KSTEPS; s++) qf[s] = *reinterpret_cast<const v4i*>(qp + s * 32);
     }
     const float sq = qscale[bh * (nq_pad / blkq) + qrow / blkq];
-    const float* ksc = kscale + bh * (nkv_pad / blkk);
 
-    const int8_t* kg = k8 + bh * nkv_pad * D;
+    // K scales of this head are staged in LDS once: a global load inside the main loop
+    // would make the compiler wait for ALL outstanding vector-memory operations, i.e. for the
+    // tile copies that are meant to stay in flight.
+    const float* ksc = kscale + bh * (nkv_pad / blkk);
+    const int nks = (int)(nkv_pad / blkk);
+    const int ush = blkk == 32 ? 0 : (blkk == 64 ? 1 : 2);      // log2(32-key blocks per scale block)
+    for (int i = tid; i < nks; i += 256) lds_ks[i] = ksc[i];
+    auto kscale_of = [&](int u32blk) -> float { return lds_ks[u32blk >> ush]; };
+
+    const uint8_t* kg = reinterpret_cast<const uint8_t*>(k8) + bh * nkv_pad * D;
     const uint8_t* vg = vq + bh * nkv_pad * D * VB;
     const int ntiles = (kv_valid + kTileKV - 1) / kTileKV;
+    const int last = ntiles - 1;
 
-    v4i kreg[K_CH], vreg[V_CH];
-    auto load_tile = [&](int t) {
-        const v4i* kp = reinterpret_cast<const v4i*>(kg + (int64_t)t * K_BYTES);
-        const v4i* vp = reinterpret_cast<const v4i*>(vg + (int64_t)t * V_BYTES);
+    // Tile-relative LDS byte offsets of this lane's MFMA A-operand fragments.  Rows
+    // 32 apart keep the same swizzle, so the 32-row blocks are plain constant offsets.
+    int koff[KSTEPS], voff[JS * FPU];
 #pragma unroll
-        for (int i = 0; i < K_CH; i++) kreg[i] = kp[i * 256 + tid];
+    for (int s = 0; s < KSTEPS; s++) koff[s] = swz(l32 * K_CPR + s * 2 + half);
+    if constexpr (VARIANT == 0) {
 #pragma unroll
-        for (int i = 0; i < V_CH; i++) vreg[i] = vp[i * 256 + tid];
+        for (int j = 0; j < JS; j++) voff[j] = swz(l32 * V_CPR + j * 2 + half);
+    } else {
+        voff[0] = swz(l32 * V_CPR + half * 2);
+        voff[1] = swz(l32 * V_CPR + half * 2 + 1);
+    }
+
+    // Copy i of wave w fills physical chunks (i*4 + w)*64 .. +63 of a tile; the lane that
+    // fills physical chunk P fetches logical chunk swz^-1(P) (the XOR is its own inverse).
+    int src_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) src_off[i] = swz((i * 4 + wave) * 64 + lane);
+    const uint32_t ldsk0 = lds_addr(&lds_k[0][0]) + wave * 1024;
+    const uint32_t ldsv0 = lds_addr(&lds_v[0][0]) + wave * 1024;
+    auto dma_k = [&](int t, int slot) {
+        const uint8_t* g = kg + (int64_t)t * K_BYTES;
+#pragma unroll
+        for (int i = 0; i < K_CH; i++)
+            dma16(g, src_off[i], __builtin_amdgcn_readfirstlane(ldsk0 + slot * K_BYTES + i * 4096));
     };
-    auto store_tile = [&](int buf) {
+    auto dma_v = [&](int t, int slot) {
+        const uint8_t* g = vg + (int64_t)t * V_BYTES;
 #pragma unroll
-        for (int i = 0; i < K_CH; i++) *reinterpret_cast<v4i*>(&lds_k[buf][swz(i * 256 + tid)]) = kreg[i];
-#pragma unroll
-        for (int i = 0; i < V_CH; i++) *reinterpret_cast<v4i*>(&lds_v[buf][swz(i * 256 + tid)]) = vreg[i];
+        for (int i = 0; i < V_CH; i++)
+            dma16(g, src_off[i], __builtin_amdgcn_readfirstlane(ldsv0 + slot * V_BYTES + i * 4096));
     };
+
+    v16i magic;
+#pragma unroll
+    for (int i = 0; i < 16; i++) magic[i] = kMagicI;
 
     v16f oacc[DB];
 #pragma unroll
     for (int d = 0; d < DB; d++)
 #pragma unroll
         for (int i = 0; i < 16; i++) oacc[d][i] = 0.0f;
-    float m_run = -INFINITY;       // running row max (log2 domain)
-    float l_run = 0.0f;            // this lane's share of the row sum
+    float m_used = -INFINITY;      // reference maximum the exponentials are taken against (log2 domain)
+    float l_run = 0.0f;            // this lane's share of the row sum (times pscale)
 
-    load_tile(0);
-    store_tile(0);
+    // Loop-carried fragments: K of the tile whose scores come next, the first PD units of
+    // V^T of the tile whose P.V comes next, and the packed probabilities of two tiles (parity).
+    v4i kf[2][KSTEPS];
+    v4i vf[NUNIT][FPU];
+    uint32_t p[2][PW];
+
+    auto read_kf = [&](int slot, int kb) {
+#pragma unroll
+        for (int st = 0; st < KSTEPS; st++)
+            kf[kb][st] = *reinterpret_cast<const v4i*>(&lds_k[slot][koff[st] + kb * 32 * D]);
+    };
+    auto read_vf = [&](int slot, int u) {               // unit u = (key step j, channel block d)
+        const int j = u / DB, d = u % DB;
+#pragma unroll
+        for (int x = 0; x < FPU; x++)
+            vf[u][x] = *reinterpret_cast<const v4i*>(&lds_v[slot][voff[j * FPU + x] + d * 32 * VROW]);
+    };
+    auto pv_unit = [&](int pb, int u) {
+        const int j = u / DB, d = u % DB;
+        if constexpr (VARIANT == 0) {
+            const v4i pw = {(int)p[pb][j * 4], (int)p[pb][j * 4 + 1], (int)p[pb][j * 4 + 2], (int)p[pb][j * 4 + 3]};
+            oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vf[u][0]),
+                                                             __builtin_bit_cast(v8h, pw), oacc[d], 0, 0, 0);
+        } else {
+            const v8i a = {vf[u][0].x, vf[u][0].y, vf[u][0].z, vf[u][0].w, vf[u][1].x, vf[u][1].y, vf[u][1].z, vf[u][1].w};
+            const v8i pw = {(int)p[pb][0], (int)p[pb][1], (int)p[pb][2], (int)p[pb][3],
+                            (int)p[pb][4], (int)p[pb][5], (int)p[pb][6], (int)p[pb][7]};
+            oacc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pw, oacc[d], 0, 0, 0, 0, 0, 0);
+        }
+    };
+
+    // ---- prologue: K(0), V(0), K(1) into the rings --------------------------------------
+    // (tile indices past the end are clamped: the extra copies are in bounds and unused)
+    dma_k(0, 0);
+    dma_v(0, 0);
+    dma_k(min(1, last), 1);
+    dma_wait_all();
     __syncthreads();
+    read_kf(0, 0);
+    read_kf(0, 1);
 
-    for (int t = 0; t < ntiles; t++) {
-        const int buf = t & 1;
-        if (t + 1 < ntiles) load_tile(t + 1);
+    // Iteration t (X = t & 1).  On entry: kf = K(t) fragments; (t > 0) p[X^1] = P(t-1),
+    // vf[0..PD) = V(t-1) fragments; K(t+1) and V(t) are in flight, started at the midpoint of
+    // iteration t-1.
+    //
+    // OPT (fp16 variant, interior tiles): the exponentials are taken against the reference
+    // maximum as it stands, without looking for the tile maximum first — that removes the
+    // max / compare / cross-lane chain from the common path.  A reference that has become too
+    // low shows up as a large tile sum (every p is non-negative, so sum <= 2^12 bounds each
+    // p, far inside fp16 range); then the tile is redone the careful way.
+    auto iteration = [&](int t, auto x_tag, auto first_tag, auto mask_tag, auto opt_tag) {
+        constexpr int X = decltype(x_tag)::value;
+        constexpr bool FIRST = decltype(first_tag)::value;
+        constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr bool OPT = decltype(opt_tag)::value;
+        const int slot_vprev = (t + NS - 1) % NS, slot_next = (t + 1) % NS, slot_k2 = (t + 2) % NS;
 
-        // ---- S^T = K . Q^T : two 32-key blocks ---------------------------------
-        v16i sacc[2];
+        // ---- S^T = K(t) . Q^T : two 32-key blocks
+        v16i s[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) sacc[kb][i] = 0;
-#pragma unroll
-            for (int s = 0; s < KSTEPS; s++) {
-                const int L = (kb * 32 + l32) * K_CPR + s * 2 + half;
-                const v4i a = *reinterpret_cast<const v4i*>(&lds_k[buf][swz(L)]);
-                sacc[kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[s], sacc[kb], 0, 0, 0);
-            }
-        }
+            for (int st = 0; st < KSTEPS; st++)
+                s[kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], st == 0 ? magic : s[kb], 0, 0, 0);
 
-        // ---- online softmax ------------------------------------------------------
-        float sf[2][16];
-        float mx = -INFINITY;
+        float f[2], c0[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            const float f = sq * ksc[(t * kTileKV + kb * 32) / blkk];
-#pragma unroll
-            for (int i = 0; i < 16; i++) sf[kb][i] = (float)sacc[kb][i] * f;
-        }
-        if (t == ntiles - 1 && (kv_valid & (kTileKV - 1)) != 0) {
+        for (int kb = 0; kb < 2; kb++) f[kb] = sq * kscale_of(t * 2 + kb);
+        if (MASK) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int key = t * kTileKV + kb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                    if (key >= kv_valid) sf[kb][i] = -INFINITY;
+                    if (key >= kv_valid) s[kb][i] = (int)0xFF800000;     // -inf as fp32, below every real accumulator
                 }
         }
+        float corr = 1.0f;
+        bool refresh = false;
+        // tile maximum on the raw accumulators (monotone in the score since f > 0), refresh decision
+        auto decide = [&](float tau) {
+            float mt = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < 2; kb++) {
+                int ma = max(max(s[kb][0], s[kb][1]), s[kb][2]);
+                int mb = max(max(s[kb][3], s[kb][4]), s[kb][5]);
 #pragma unroll
-            for (int i = 0; i < 16; i++) mx = fmaxf(mx, sf[kb][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.0f;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                sf[kb][i] = __builtin_amdgcn_exp2f(sf[kb][i] - m_new);
-                psum += sf[kb][i];
+                for (int i = 6; i < 14; i += 4) {
+                    ma = max(max(ma, s[kb][i]), s[kb][i + 1]);
+                    mb = max(max(mb, s[kb][i + 2]), s[kb][i + 3]);
+                }
+                const int mi = max(max(ma, mb), max(s[kb][14], s[kb][15]));
+                const float mk = MASK && mi < 0 ? -INFINITY : (float)(mi - kMagicI) * f[kb];
+                mt = fmaxf(mt, mk);
             }
-        l_run = l_run * corr + psum;
-        if (__any(corr != 1.0f)) {
+            const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);
+            mt = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
+            refresh = __any(mt > m_used + tau);
+            const float m_new = refresh ? fmaxf(m_used, mt) : m_used;
+            corr = __builtin_amdgcn_exp2f(m_used - m_new);           // 1 when nothing changed
+            m_used = m_new;
+            l_run *= corr;             // already includes tile t-1's probabilities
+        };
+        if (!OPT) decide(Lazy<VARIANT>::tau);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(kMagicF, f[kb], m_used);
+        const float l_before = l_run;
+
+        // Exponentials of scores n, n+1 of this lane (n counts through kb, then i).
+        auto exp_pair = [&](int n) {
+            const int kb = n >> 4, i = n & 15;
+            float p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
+            float p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
+            if (MASK) {
+                if (s[kb][i] < 0) p0 = 0.0f;
+                if (s[kb][i + 1] < 0) p1 = 0.0f;
+            }
+            if constexpr (VARIANT == 0) {
+                const v2h pr = {(_Float16)p0, (_Float16)p1};
+                const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+                // the normaliser sums the rounded probabilities the product actually uses
+                l_run = __builtin_amdgcn_fdot2(pr, ones, l_run, false);
+                p[X][n >> 1] = __builtin_bit_cast(uint32_t, pr);
+            } else {
+                l_run += p0 + p1;
+                const int w = n >> 2;
+                if (n & 2) p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, (int)p[X][w], true);
+                else p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
+            }
+        };
+        auto exp_group = [&](int g) {                  // the EPU scores that go with PV unit g
+#pragma unroll
+            for (int e = 0; e < EPU; e += 2) exp_pair(g * EPU + e);
+            // Pin the group here: an empty volatile statement that consumes the results keeps the
+            // compiler from sinking the exponentials below the matrix instructions they are meant
+            // to overlap with.
+            asm volatile("" : "+v"(l_run), "+v"(p[X][VARIANT == 0 ? (g * EPU) >> 1 : (g * EPU) >> 2]));
+        };
+
+        // At the midpoint every wave has finished iteration t-1 completely, so the ring slots
+        // it read are free: publish K(t+1)/V(t), start the copies of K(t+2) and V(t+1), and
+        // fetch the fragments of K(t+1).
+        auto midpoint = [&]() {
+            dma_wait_all();
+            __syncthreads();
+            dma_k(min(t + 2, last), slot_k2);
+            dma_v(min(t + 1, last), slot_next);
+            read_kf(slot_next, 0);
+        };
+
+        // ---- softmax(t) interleaved with O^T += V^T(t-1) . P^T(t-1)
+#pragma unroll
+        for (int u = 0; u < NUNIT; u++) {
+            if (!FIRST) {
+                if (u + PD < NUNIT) read_vf(slot_vprev, u + PD);
+                pv_unit(X ^ 1, u);
+            }
+            exp_group(u);
+            if (u == NUNIT / 2 - 1) midpoint();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (OPT) {
+            // !(x <= bound) also catches an infinite or NaN sum
+            if (__any(!(l_run - l_before <= 4096.0f))) {
+                l_run = l_before;
+                decide(0.0f);
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(kMagicF, f[kb], m_used);
+#pragma unroll
+                for (int n = 0; n < 32; n += 2) exp_pair(n);
+            }
+        }
+        if (!FIRST && refresh) {
+            // the accumulators include tile t-1 at the old reference; move them to the new one
+            // (the empty volatile statement keeps this rare block a real branch)
+            asm volatile("" ::: "memory");
 #pragma unroll
             for (int d = 0; d < DB; d++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) oacc[d][i] *= corr;
         }
+        // first V^T fragments of tile t for the next iteration (published by this iteration's midpoint)
+#pragma unroll
+        for (int u = 0; u < PD; u++) read_vf(t % NS, u);
+        read_kf(slot_next, 1);
+    };
 
-        // ---- O^T += V^T . P^T ----------------------------------------------------
-        if (VARIANT == 0) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {                 // 16 key slots per step
-                v8h p;
-#pragma unroll
-                for (int e = 0; e < 8; e++) p[e] = (_Float16)sf[j >> 1][(j & 1) * 8 + e];
-#pragma unroll
-                for (int d = 0; d < DB; d++) {
-                    const int L = (d * 32 + l32) * V_CPR + j * 2 + half;
-                    const v8h a = *reinterpret_cast<const v8h*>(&lds_v[buf][swz(L)]);
-                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, p, oacc[d], 0, 0, 0);
-                }
-            }
-        } else {
-            // P8 = e4m3(p * 448); 32 key slots of this half-wave in 8 dwords
-            v8i p;
-#pragma unroll
-            for (int w = 0; w < 8; w++) {
-                const float* s4 = &sf[w >> 2][(w & 3) * 4];
-                int pk = __builtin_amdgcn_cvt_pk_fp8_f32(s4[0] * 448.0f, s4[1] * 448.0f, 0, false);
-                pk = __builtin_amdgcn_cvt_pk_fp8_f32(s4[2] * 448.0f, s4[3] * 448.0f, pk, true);
-                p[w] = pk;
-            }
-#pragma unroll
-            for (int d = 0; d < DB; d++) {
-                const int L0 = (d * 32 + l32) * V_CPR + half * 2;
-                const v4i a0 = *reinterpret_cast<const v4i*>(&lds_v[buf][swz(L0)]);
-                const v4i a1 = *reinterpret_cast<const v4i*>(&lds_v[buf][swz(L0 + 1)]);
-                const v8i a = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-                oacc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, p, oacc[d], 0, 0, 0, 0, 0, 0);
-            }
+    const bool ragged = (kv_valid & (kTileKV - 1)) != 0;
+    using T = std::true_type;
+    using F = std::false_type;
+    using X0 = std::integral_constant<int, 0>;
+    using X1 = std::integral_constant<int, 1>;
+    using OPT = std::integral_constant<bool, VARIANT == 0>;
+    if (last == 0) {
+        if (ragged) iteration(0, X0{}, T{}, T{}, F{});
+        else iteration(0, X0{}, T{}, F{}, F{});
+    } else {
+        iteration(0, X0{}, T{}, F{}, F{});
+        int t = 1;
+        for (; t + 1 < last; t += 2) {
+            iteration(t, X1{}, F{}, F{}, OPT{});
+            iteration(t + 1, X0{}, F{}, F{}, OPT{});
         }
-
-        if (t + 1 < ntiles) store_tile(buf ^ 1);
-        __syncthreads();
+        if (t < last) {
+            iteration(t, X1{}, F{}, F{}, OPT{});
+            t++;
+        }
+        // t == last
+        if (t & 1) {
+            if (ragged) iteration(t, X1{}, F{}, T{}, F{});
+            else iteration(t, X1{}, F{}, F{}, F{});
+        } else {
+            if (ragged) iteration(t, X0{}, F{}, T{}, F{});
+            else iteration(t, X0{}, F{}, F{}, F{});
+        }
     }
+    // ---- drain: P.V of the last tile ------------------------------------------------------
+    auto drain = [&](auto x_tag) {
+        constexpr int X = decltype(x_tag)::value;
+#pragma unroll
+        for (int u = 0; u < NUNIT; u++) {
+            if (u + PD < NUNIT) read_vf(last % NS, u + PD);
+            pv_unit(X, u);
+        }
+    };
+    if (last & 1) drain(X1{});
+    else drain(X0{});
 
     // ---- epilogue: normalise, bf16 round-to-nearest-even, caller's strides ---------
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / l_tot;
+    float l_tot;
+    {
+        const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+        l_tot = __uint_as_float(r.x) + __uint_as_float(r.y);
+    }
+    const float inv = 1.0f / l_tot;      // l carries pscale, which cancels the pscale in P
     if (qrow < Nq) {
         uint16_t* op = o + b * osb + h * osh + (int64_t)qrow * osn;
 #pragma unroll
@@ -238,7 +455,7 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     x[e] = oacc[d][g * 4 + e];
-                    if (VARIANT == 1) x[e] = x[e] * vscale[bh * D + ch + e] * (1.0f / 448.0f);
+                    if (VARIANT == 1) x[e] = x[e] * vscale[bh * D + ch + e];
                     x[e] *= inv;
                 }
                 u32x2 pk;
@@ -250,7 +467,7 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
             // natural-log log-sum-exp of the scaled scores.  With K smoothing every score
             // of a row was lowered by <q, mean>, which the Q quantizer recorded per row.
             const float shift = qshift != nullptr ? qshift[bh * nq_pad + qrow] : 0.0f;
-            stats[bh * Nq + qrow] = (m_run + __builtin_amdgcn_logf(l_tot) + shift) * 0.6931471805599453f;
+            stats[bh * Nq + qrow] = (m_used + __builtin_amdgcn_logf(l_tot) - Lazy<VARIANT>::log2_pscale + shift) * 0.6931471805599453f;
         }
     }
 }
