@@ -51,6 +51,15 @@ View make_view(const void* p, const int64_t* s, int64_t off) {
 
 bool blk_ok(int blk) { return blk == 32 || blk == 64 || blk == 128; }
 
+// The attention kernel keeps one head's K scales in LDS.
+int check_kv_len(int N_kv, int blkk) {
+    if (pad_to(N_kv, kPadKV) / blkk > kMaxKScales) {
+        SAGE_LOG("N_kv=%d with %d-token K blocks exceeds %d scale blocks per head", N_kv, blkk, kMaxKScales);
+        return MI355_SAGE_EUNSUPPORTED;
+    }
+    return 0;
+}
+
 // Workspace layout of the one-shot calls.
 struct Carve {
     size_t q8, k8, vq, qscale, kscale, kmean, vscale, partial, qshift, total;
@@ -129,6 +138,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
     if (!blk_ok(blkq) || !blk_ok(blkk)) { SAGE_LOG("block sizes must be 32, 64 or 128"); return MI355_SAGE_EUNSUPPORTED; }
     int rc;
+    if ((rc = check_kv_len(N_kv, blkk))) return rc;
     if ((rc = check_view("Q", Q, qs, q_off)) || (rc = check_view("K", K, ks, k_off)) ||
         (rc = check_view("V", V, vs, v_off)) || (rc = check_view("O", O, os, o_off)))
         return rc;
@@ -304,6 +314,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
     if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk)) return MI355_SAGE_EUNSUPPORTED;
     int rc;
+    if ((rc = check_kv_len(N_kv, blkk))) return rc;
     if ((rc = check_view("O", O, o_strides, o_off))) return rc;
     AttnArgs a{};
     a.q8 = static_cast<const int8_t*>(q8); a.qscale = static_cast<const float*>(qscale); a.blkq = blkq;

@@ -65,7 +65,11 @@ __device__ __forceinline__ void dma16(const void* gbase_uniform, uint32_t goff, 
                  : "s"(lds_base_uniform), "v"(goff), "s"(gbase_uniform)
                  : "memory");
 }
-__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Wait until at most N of this wave's copies are still in flight (they complete in order).
+template <int N> __device__ __forceinline__ void dma_wait() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
@@ -91,7 +95,7 @@ template <int VARIANT> struct Lazy {
 };
 
 template <int D, int VARIANT, bool STATS>
-__global__ __launch_bounds__(256, 2) void sage_attn_kernel(
+__global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
@@ -104,12 +108,15 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     constexpr int DB = D / 32;                          // 32-channel output blocks
     constexpr int K_BYTES = kTileKV * D;                // K tile
     constexpr int V_BYTES = D * kTileKV * VB;           // V^T tile
-    constexpr int K_CH = K_BYTES / 16 / 256;            // 16-byte chunks per thread
-    constexpr int V_CH = V_BYTES / 16 / 256;
+    constexpr int NW = 8;                               // waves per workgroup
+    constexpr int K_NCH = K_BYTES / 1024, V_NCH = V_BYTES / 1024;      // 1 KiB copies per tile
+    constexpr int K_CH = (K_NCH + NW - 1) / NW;         // copies per wave (short tiles: some waves repeat a copy)
+    constexpr int V_CH = (V_NCH + NW - 1) / NW;
+    constexpr int LEAD = 2;                             // tile copies run this many iterations ahead
+    constexpr int NSK = LEAD + 1, NSV = LEAD + 2;       // ring depths
     constexpr int K_CPR = D / 16;                       // chunks per K row
     constexpr int V_CPR = kTileKV * VB / 16;            // chunks per V^T row
     constexpr int VROW = kTileKV * VB;                  // bytes per V^T row
-    constexpr int NS = 3;                               // LDS ring depth
     constexpr int JS = VARIANT == 0 ? 4 : 1;            // PV steps over the 64 keys of a tile
     constexpr int NUNIT = JS * DB;                      // PV matrix instructions per tile
     constexpr int EPU = 32 / NUNIT;                     // scores exponentiated per PV instruction
@@ -118,9 +125,9 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     constexpr int PW = VARIANT == 0 ? 16 : 8;           // dwords of packed P per tile
     static_assert(32 % NUNIT == 0 && EPU % 2 == 0, "unit split");
 
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NS][K_BYTES];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NS][V_BYTES];
-    __shared__ float lds_ks[1024];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NSK][K_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][V_BYTES];
+    __shared__ float lds_ks[kMaxKScales];
 
     // Workgroup -> (q tile, b*h).  Hardware hands consecutive workgroup ids to the 8
     // XCDs round-robin; give each XCD a contiguous range of (head, q tile) work so the
@@ -156,7 +163,7 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     const float* ksc = kscale + bh * (nkv_pad / blkk);
     const int nks = (int)(nkv_pad / blkk);
     const int ush = blkk == 32 ? 0 : (blkk == 64 ? 1 : 2);      // log2(32-key blocks per scale block)
-    for (int i = tid; i < nks; i += 256) lds_ks[i] = ksc[i];
+    for (int i = tid; i < nks; i += 64 * NW) lds_ks[i] = ksc[i];
     auto kscale_of = [&](int u32blk) -> float { return lds_ks[u32blk >> ush]; };
 
     const uint8_t* kg = reinterpret_cast<const uint8_t*>(k8) + bh * nkv_pad * D;
@@ -177,24 +184,33 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
         voff[1] = swz(l32 * V_CPR + half * 2 + 1);
     }
 
-    // Copy i of wave w fills physical chunks (i*4 + w)*64 .. +63 of a tile; the lane that
-    // fills physical chunk P fetches logical chunk swz^-1(P) (the XOR is its own inverse).
-    int src_off[4];
+    // Copy i of wave w fills the 1 KiB run c = (i*8 + w) mod (copies per tile) of a tile (short
+    // tiles are covered twice with identical data, which keeps every wave's copy count equal);
+    // the lane that fills physical chunk P fetches logical chunk swz^-1(P) (the XOR is its own
+    // inverse).
+    int ksrc[K_CH], vsrc[V_CH];
+    uint32_t kdst[K_CH], vdst[V_CH];
 #pragma unroll
-    for (int i = 0; i < 4; i++) src_off[i] = swz((i * 4 + wave) * 64 + lane);
-    const uint32_t ldsk0 = lds_addr(&lds_k[0][0]) + wave * 1024;
-    const uint32_t ldsv0 = lds_addr(&lds_v[0][0]) + wave * 1024;
+    for (int i = 0; i < K_CH; i++) {
+        const int c = (i * NW + wave) % K_NCH;
+        ksrc[i] = swz(c * 64 + lane);
+        kdst[i] = lds_addr(&lds_k[0][0]) + c * 1024;
+    }
+#pragma unroll
+    for (int i = 0; i < V_CH; i++) {
+        const int c = (i * NW + wave) % V_NCH;
+        vsrc[i] = swz(c * 64 + lane);
+        vdst[i] = lds_addr(&lds_v[0][0]) + c * 1024;
+    }
     auto dma_k = [&](int t, int slot) {
         const uint8_t* g = kg + (int64_t)t * K_BYTES;
 #pragma unroll
-        for (int i = 0; i < K_CH; i++)
-            dma16(g, src_off[i], __builtin_amdgcn_readfirstlane(ldsk0 + slot * K_BYTES + i * 4096));
+        for (int i = 0; i < K_CH; i++) dma16(g, ksrc[i], __builtin_amdgcn_readfirstlane(kdst[i] + slot * K_BYTES));
     };
     auto dma_v = [&](int t, int slot) {
         const uint8_t* g = vg + (int64_t)t * V_BYTES;
 #pragma unroll
-        for (int i = 0; i < V_CH; i++)
-            dma16(g, src_off[i], __builtin_amdgcn_readfirstlane(ldsv0 + slot * V_BYTES + i * 4096));
+        for (int i = 0; i < V_CH; i++) dma16(g, vsrc[i], __builtin_amdgcn_readfirstlane(vdst[i] + slot * V_BYTES));
     };
 
     v16i magic;
@@ -243,9 +259,12 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
     // ---- prologue: K(0), V(0), K(1) into the rings --------------------------------------
     // (tile indices past the end are clamped: the extra copies are in bounds and unused)
     dma_k(0, 0);
-    dma_v(0, 0);
-    dma_k(min(1, last), 1);
-    dma_wait_all();
+#pragma unroll
+    for (int x = 0; x < LEAD; x++) {
+        dma_k(min(x + 1, last), (x + 1) % NSK);
+        dma_v(min(x, last), x % NSV);
+    }
+    dma_wait<0>();
     __syncthreads();
     read_kf(0, 0);
     read_kf(0, 1);
@@ -264,7 +283,7 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
         constexpr bool FIRST = decltype(first_tag)::value;
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr bool OPT = decltype(opt_tag)::value;
-        const int slot_vprev = (t + NS - 1) % NS, slot_next = (t + 1) % NS, slot_k2 = (t + 2) % NS;
+        const int slot_vprev = (t + NSV - 1) % NSV, slot_knext = (t + 1) % NSK;
 
         // ---- S^T = K(t) . Q^T : two 32-key blocks
         v16i s[2];
@@ -352,11 +371,11 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
         // it read are free: publish K(t+1)/V(t), start the copies of K(t+2) and V(t+1), and
         // fetch the fragments of K(t+1).
         auto midpoint = [&]() {
-            dma_wait_all();
+            dma_wait<(LEAD - 1) * (K_CH + V_CH)>();
             __syncthreads();
-            dma_k(min(t + 2, last), slot_k2);
-            dma_v(min(t + 1, last), slot_next);
-            read_kf(slot_next, 0);
+            dma_k(min(t + LEAD + 1, last), (t + LEAD + 1) % NSK);
+            dma_v(min(t + LEAD, last), (t + LEAD) % NSV);
+            read_kf(slot_knext, 0);
         };
 
         // ---- softmax(t) interleaved with O^T += V^T(t-1) . P^T(t-1)
@@ -392,8 +411,8 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
         }
         // first V^T fragments of tile t for the next iteration (published by this iteration's midpoint)
 #pragma unroll
-        for (int u = 0; u < PD; u++) read_vf(t % NS, u);
-        read_kf(slot_next, 1);
+        for (int u = 0; u < PD; u++) read_vf(t % NSV, u);
+        read_kf(slot_knext, 1);
     };
 
     const bool ragged = (kv_valid & (kTileKV - 1)) != 0;
@@ -430,7 +449,7 @@ __global__ __launch_bounds__(256, 2) void sage_attn_kernel(
         constexpr int X = decltype(x_tag)::value;
 #pragma unroll
         for (int u = 0; u < NUNIT; u++) {
-            if (u + PD < NUNIT) read_vf(last % NS, u + PD);
+            if (u + PD < NUNIT) read_vf(last % NSV, u + PD);
             pv_unit(X, u);
         }
     };
@@ -477,7 +496,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     const int n_qtiles = (int)(a.nq_pad / kTileQ);
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    dim3 grid((unsigned)total), block(256);
+    dim3 grid((unsigned)total), block(512);
     if (a.stats != nullptr)
         hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, true>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
                            a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
@@ -490,6 +509,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
 }
 
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st) {
+    if (a.nkv_pad / a.blkk > kMaxKScales) return hipErrorInvalidValue;      // K scales would not fit the LDS staging
     if (a.D == 128) return a.variant == 0 ? launch_attn_dv<128, 0>(a, st) : launch_attn_dv<128, 1>(a, st);
     if (a.D == 64) return a.variant == 0 ? launch_attn_dv<64, 0>(a, st) : launch_attn_dv<64, 1>(a, st);
     return hipErrorInvalidValue;

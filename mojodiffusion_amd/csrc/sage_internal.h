@@ -8,11 +8,12 @@
 namespace sage {
 
 // Tile geometry of the attention kernel; the quantized layouts are padded to it.
-constexpr int kTileQ  = 128;   // query rows per workgroup
+constexpr int kTileQ  = 256;   // query rows per workgroup (8 waves x 32 rows)
 constexpr int kTileKV = 64;    // keys per main-loop iteration
 constexpr int kPadKV  = 128;   // key tokens are padded to this (every scale-block size divides it)
 constexpr int kLeaf   = 16;    // tokens per leaf of the K-mean summation tree
 constexpr int kGroup  = 256;   // tokens per group (16 leaves)
+constexpr int kMaxKScales = 1024;   // K scale blocks per head the attention kernel stages in LDS
 
 inline int64_t pad_to(int64_t n, int64_t m) { return (n + m - 1) / m * m; }
 

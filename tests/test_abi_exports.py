@@ -28,7 +28,7 @@ def test_every_declared_symbol_is_exported_and_bound():
 def test_no_gpu_helpers():
     L = _lib.lib()
     assert L.mi355_sage_version().startswith(b"mi355_sage")
-    assert L.mi355_sage_pad_q(1) == 128 and L.mi355_sage_pad_q(4608) == 4608
+    assert L.mi355_sage_pad_q(1) in (128, 256) and L.mi355_sage_pad_q(4608) == 4608
     assert L.mi355_sage_pad_kv(32760) == 32768
     for variant in (0, 1):
         slots = sorted(L.mi355_sage_v_slot(k, variant) for k in range(64))
@@ -65,6 +65,9 @@ def test_argument_validation_without_device():
                                   0, 0, 0, 0, 0, None, 0, None, 0) == -2          # strided head dim
     assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
                                   3, 0, 0, 0, 0, None, 0, None, 0) == -2          # misaligned offset
+    st_long = _lib.strides_bhnd(70000, 2, 128)
+    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 70000, 128, 0.1, st, st_long, st_long, st,
+                                  0, 0, 0, 0, 0, None, 0, None, 0) == -2          # more K scale blocks than the kernel stages
     # workspace too small -> -3 (checked before any launch)
     assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
                                   0, 0, 0, 0, 0, None, 0, ctypes.c_void_p(256 * 64), 1024) == -3

@@ -14,7 +14,7 @@ COS = 0.999
 
 
 def _oracle_quantized(oracle, q, k, v, w, variant):
-    q8, qs = oracle.quant_q(q, w.scale, w.blkq, 128)
+    q8, qs = oracle.quant_q(q, w.scale, w.blkq, int(_lib.lib().mi355_sage_pad_q(1)))
     k8, ks = oracle.quant_k(k, oracle.kmean(k), w.blkk, 128)
     if variant == 0:
         vq, vs = oracle.quant_v_f16(v, 128), None

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 def _check_qk(oracle, H, q, k, scale, blkq, blkk, smooth):
     g = H.quant_qk(q, k, scale, blkq, blkk, smooth)
     Sq, Skv = q.shape[1], k.shape[1]
-    q8, qs = oracle.quant_q(q, scale, blkq, 128)
+    q8, qs = oracle.quant_q(q, scale, blkq, int(_lib.lib().mi355_sage_pad_q(1)))
     mu = oracle.kmean(k) if smooth else None
     k8, ks = oracle.quant_k(k, mu, blkk, 128)
     if smooth:
