@@ -171,14 +171,24 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     float* qshift = Stats ? reinterpret_cast<float*>(ws + c.qshift) : nullptr;
 
     const View q = make_view(Q, qs, q_off), k = make_view(K, ks, k_off), v = make_view(V, vs, v_off);
-    if ((rc = quant_qk(q, k, B, H, N_q, kv, D, scale, blkq, blkk, smooth_k, q8, qscale, k8, kscale,
-                       kmean, partial, qshift, st)))
-        return rc;
     const int64_t nkp = pad_to(kv, kPadKV);
-    if (variant == MI355_SAGE_PV_FP16)
-        SAGE_HIP(launch_quant_v_f16(v, B, H, kv, D, nkp, static_cast<uint16_t*>(vq), st));
-    else
-        SAGE_HIP(launch_quant_v_fp8(v, B, H, kv, D, nkp, static_cast<uint8_t*>(vq), vscale, st));
+    if (variant == MI355_SAGE_PV_FP16 && !Stats) {
+        // two launches: {Q quantize, V repack, K-mean group sums} then {K mean + K quantize}
+        const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
+        SAGE_HIP(launch_prep_fused(q, k, v, B, H, N_q, kv, D, pad_to(N_q, kTileQ), nkp, cmul, blkq, smooth_k != 0,
+                                   q8, qscale, static_cast<uint16_t*>(vq), partial, st));
+        SAGE_HIP(launch_kquant_fused(k, B, H, kv, D, nkp, blkk, smooth_k ? partial : nullptr, kmean, k8, kscale, st));
+    } else {
+        // Stats needs <q, kmean> per row, i.e. the mean before the Q quantizer; the e4m3 V path
+        // has its own three launches
+        if ((rc = quant_qk(q, k, B, H, N_q, kv, D, scale, blkq, blkk, smooth_k, q8, qscale, k8, kscale,
+                           kmean, partial, qshift, st)))
+            return rc;
+        if (variant == MI355_SAGE_PV_FP16)
+            SAGE_HIP(launch_quant_v_f16(v, B, H, kv, D, nkp, static_cast<uint16_t*>(vq), st));
+        else
+            SAGE_HIP(launch_quant_v_fp8(v, B, H, kv, D, nkp, static_cast<uint8_t*>(vq), vscale, st));
+    }
 
     AttnArgs a{};
     a.q8 = q8; a.qscale = qscale; a.blkq = blkq;

@@ -35,6 +35,15 @@ hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_
 hipError_t launch_kmean(const View& k, int B, int H, int N, int D,
                         double* group_partials, float* kmean, hipStream_t st);
 
+// One-shot path: Q quantizer + V fp16 repack + K-mean group sums in one launch, then the
+// K quantizer that finishes the mean from the group partials itself (partial == null: no
+// smoothing).  Same arithmetic, bit for bit, as the separate launches above.
+hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B, int H, int Nq, int Nkv, int D,
+                             int64_t nq_pad, int64_t nkv_pad, float cmul, int blkq, bool smooth_k,
+                             int8_t* q8, float* qscale, uint16_t* v16, double* partial, hipStream_t st);
+hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
+                               const double* partial, float* kmean, int8_t* codes, float* scales, hipStream_t st);
+
 hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t n_pad,
                               uint16_t* v16, hipStream_t st);
 

@@ -36,15 +36,15 @@ __device__ __forceinline__ float wave_max(float v) {
 // the block's BLK x D tile lives in registers between the absmax pass and the
 // encode pass, so HBM sees one read of bf16 and one write of int8.
 // ---------------------------------------------------------------------------
+// `mean` points at the D means of this (b,h) (global or LDS), or is null.
 template <int D, int BLK, bool IS_K>
-__global__ __launch_bounds__(256) void quant_i8_kernel(
-    const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
-    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot) {
+__device__ __forceinline__ void quant_i8_block(
+    int t, int h, int b, const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, float cmul, const float* mean,
+    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, float* red) {
     constexpr int CPR = D / 8;                 // 16-byte chunks per row
     constexpr int NCH = BLK * CPR / 256;       // chunks per thread
     static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
-    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x;
     const int r0 = t * BLK;
     const int64_t bh = (int64_t)b * H + h;
@@ -61,8 +61,8 @@ __global__ __launch_bounds__(256) void quant_i8_kernel(
         unpack8(w, v[i]);
         if (IS_K) {
             if (mean != nullptr) {
-                const float4 m0 = *reinterpret_cast<const float4*>(mean + bh * D + col);
-                const float4 m1 = *reinterpret_cast<const float4*>(mean + bh * D + col + 4);
+                const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
+                const float4 m1 = *reinterpret_cast<const float4*>(mean + col + 4);
                 v[i][0] -= m0.x; v[i][1] -= m0.y; v[i][2] -= m0.z; v[i][3] -= m0.w;
                 v[i][4] -= m1.x; v[i][5] -= m1.y; v[i][6] -= m1.z; v[i][7] -= m1.w;
             }
@@ -72,8 +72,8 @@ __global__ __launch_bounds__(256) void quant_i8_kernel(
             if (rowdot != nullptr) {
                 // <pre-scaled query row, K mean>: the amount K smoothing lowers every score
                 // of this row by; the CPR lanes that share a row are adjacent in the wave.
-                const float4 m0 = *reinterpret_cast<const float4*>(mean + bh * D + col);
-                const float4 m1 = *reinterpret_cast<const float4*>(mean + bh * D + col + 4);
+                const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
+                const float4 m1 = *reinterpret_cast<const float4*>(mean + col + 4);
                 float dot = v[i][0] * m0.x + v[i][1] * m0.y + v[i][2] * m0.z + v[i][3] * m0.w +
                             v[i][4] * m1.x + v[i][5] * m1.y + v[i][6] * m1.z + v[i][7] * m1.w;
 #pragma unroll
@@ -87,7 +87,6 @@ __global__ __launch_bounds__(256) void quant_i8_kernel(
         }
     }
 
-    __shared__ float red[4];
     amax = wave_max(amax);
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
@@ -113,6 +112,17 @@ __global__ __launch_bounds__(256) void quant_i8_kernel(
         u32x2 o = {pk[0], pk[1]};
         *reinterpret_cast<u32x2*>(codes + (bh * n_pad + row) * D + col) = o;
     }
+}
+
+template <int D, int BLK, bool IS_K>
+__global__ __launch_bounds__(256) void quant_i8_kernel(
+    const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
+    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot) {
+    __shared__ float red[4];
+    const int h = blockIdx.y, b = blockIdx.z;
+    quant_i8_block<D, BLK, IS_K>(blockIdx.x, h, b, x, sb, sh, sn, N, H, n_pad, cmul,
+                                 mean ? mean + ((int64_t)b * H + h) * D : nullptr, codes, scales, rowdot, red);
 }
 
 template <int D, bool IS_K>
@@ -154,13 +164,12 @@ hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_
 // Kernel 1: one workgroup per (group, h, b); lane (leaf, 8-channel chunk).
 // Kernel 2: one thread per (b, h, channel).
 // ---------------------------------------------------------------------------
+// Executed by 16*(D/8) consecutive threads; `tid` is the index among them.
 template <int D>
-__global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
-    const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int ngroups, double* __restrict__ partial) {
+__device__ __forceinline__ void kmean_group_body(
+    int g, int h, int b, int tid, const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int ngroups, double* __restrict__ partial, double (*leafsum)[D + 2]) {
     constexpr int CPR = D / 8;
-    const int g = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int tid = threadIdx.x;
     const int leaf = tid / CPR, col = (tid % CPR) * 8;
     const uint16_t* src = k + b * sb + h * sh + col;
     const int s0 = g * kGroup + leaf * kLeaf;
@@ -169,7 +178,7 @@ __global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
 #pragma unroll
     for (int i = 0; i < kLeaf; i++) {
         w[i] = u32x4{0u, 0u, 0u, 0u};
-        if (s0 + i < N) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)(s0 + i) * sn);
+        if (g >= 0 && s0 + i < N) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)(s0 + i) * sn);
     }
     double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -181,16 +190,23 @@ __global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
         for (int e = 0; e < 8; e++) acc[e] += (double)x[e];
     }
 
-    __shared__ double leafsum[16][D + 2];
 #pragma unroll
     for (int e = 0; e < 8; e++) leafsum[leaf][col + e] = acc[e];
     __syncthreads();
-    if (tid < D) {
+    if (tid < D && g >= 0) {
         double gsum = 0.0;
 #pragma unroll
         for (int u = 0; u < 16; u++) gsum += leafsum[u][tid];
         partial[(((int64_t)b * H + h) * ngroups + g) * D + tid] = gsum;
     }
+}
+
+template <int D>
+__global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
+    const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int ngroups, double* __restrict__ partial) {
+    __shared__ double leafsum[16][D + 2];
+    kmean_group_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x, k, sb, sh, sn, N, H, ngroups, partial, leafsum);
 }
 
 __global__ __launch_bounds__(256) void kmean_final_kernel(
@@ -237,13 +253,11 @@ __device__ __forceinline__ uint16_t f32_to_f16_sat(float x) {
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void quant_v_f16_kernel(
-    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, uint16_t* __restrict__ out) {
+__device__ __forceinline__ void quant_v_f16_body(
+    int t, int h, int b, const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, uint16_t* __restrict__ out, uint16_t* tile) {
     constexpr int CPR = D / 8;
     constexpr int LD = D + 8;                              // padded row (halves), keeps 16-byte alignment
-    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * LD];
-    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x;
     const uint16_t* src = v + b * sb + h * sh;
 #pragma unroll
@@ -277,6 +291,14 @@ __global__ __launch_bounds__(256) void quant_v_f16_kernel(
     }
 }
 
+template <int D>
+__global__ __launch_bounds__(256) void quant_v_f16_kernel(
+    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, uint16_t* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * (D + 8)];
+    quant_v_f16_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, v, sb, sh, sn, N, H, n_pad, out, tile);
+}
+
 hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t n_pad,
                               uint16_t* v16, hipStream_t st) {
     dim3 grid((unsigned)(n_pad / 64), (unsigned)H, (unsigned)B);
@@ -286,6 +308,135 @@ hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t
         hipLaunchKernelGGL((quant_v_f16_kernel<64>), grid, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, v16);
     else
         return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Fused launches of the one-shot path.  The Q quantizer, the V repack and the K-mean
+// group sums are independent of each other: one launch runs all three as workgroup roles
+// (saves two launch gaps and fills the chip while each role alone is too short to).  The
+// K quantizer then takes its mean straight from the group partials (added in group
+// order, the same arithmetic as kmean_final_kernel) and covers a whole 256-token group
+// per workgroup, which also removes the separate final-mean launch.
+// ---------------------------------------------------------------------------
+struct PrepArgs {
+    View q, k, v;
+    int H, Nq, Nkv;
+    int64_t nq_pad, nkv_pad;
+    float cmul;
+    int8_t* q8; float* qscale; uint16_t* v16; double* partial;
+    int nq_blk, nv_tile, nk_wg, ngroups;      // per (b,h): Q blocks, V tiles, K-mean workgroups; K groups
+};
+
+template <int D, int BLKQ>
+__global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
+    constexpr int GPW = 256 / (16 * (D / 8));             // K-mean groups per workgroup
+    union Smem {
+        float red[4];
+        uint16_t tile[64 * (D + 8)];
+        double leafsum[GPW][16][D + 2];
+    };
+    __shared__ __attribute__((aligned(16))) Smem sm;
+    const int per_bh = a.nq_blk + a.nv_tile + a.nk_wg;
+    const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
+    const int b = bh / a.H, h = bh % a.H;
+    if (r < a.nq_blk) {
+        quant_i8_block<D, BLKQ, false>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, a.cmul, nullptr,
+                                       a.q8, a.qscale, nullptr, sm.red);
+    } else if (r < a.nq_blk + a.nv_tile) {
+        quant_v_f16_body<D>(r - a.nq_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.v16, sm.tile);
+    } else {
+        const int sub = threadIdx.x / (16 * (D / 8));
+        const int g = (r - a.nq_blk - a.nv_tile) * GPW + sub;
+        // groups past the end still take part in the barrier inside; they read nothing and
+        // their sum is not stored
+        kmean_group_body<D>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh, a.k.sn,
+                            a.Nkv, a.H, a.ngroups, a.partial, sm.leafsum[sub]);
+    }
+}
+
+template <int D, int BLK>
+__global__ __launch_bounds__(256) void kquant_group_kernel(
+    const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, const double* __restrict__ partial, int ngroups,
+    float* __restrict__ kmean, int8_t* __restrict__ codes, float* __restrict__ scales) {
+    __shared__ float mean_s[D];
+    __shared__ float red[4];
+    const int grp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int64_t bh = (int64_t)b * H + h;
+    const bool smooth = partial != nullptr;
+    if (smooth && threadIdx.x < D) {
+        const double* p = partial + bh * ngroups * D + threadIdx.x;
+        double sum = 0.0;
+        for (int g = 0; g < ngroups; g++) sum += p[(int64_t)g * D];
+        const float m = (float)(sum / (double)N);
+        mean_s[threadIdx.x] = m;
+        if (grp == 0) kmean[bh * D + threadIdx.x] = m;
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int i = 0; i < kGroup / BLK; i++) {
+        const int t = grp * (kGroup / BLK) + i;
+        if ((int64_t)t * BLK >= n_pad) break;
+        quant_i8_block<D, BLK, true>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
+                                     codes, scales, nullptr, red);
+        __syncthreads();                                   // `red` is reused by the next block
+    }
+}
+
+template <int D>
+static hipError_t launch_prep_d(const PrepArgs& a, int B, int blkq, hipStream_t st) {
+    dim3 grid((unsigned)((int64_t)B * a.H * (a.nq_blk + a.nv_tile + a.nk_wg))), block(256);
+    switch (blkq) {
+        case 32: hipLaunchKernelGGL((prep_kernel<D, 32>), grid, block, 0, st, a); break;
+        case 64: hipLaunchKernelGGL((prep_kernel<D, 64>), grid, block, 0, st, a); break;
+        case 128: hipLaunchKernelGGL((prep_kernel<D, 128>), grid, block, 0, st, a); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B, int H, int Nq, int Nkv, int D,
+                             int64_t nq_pad, int64_t nkv_pad, float cmul, int blkq, bool smooth_k,
+                             int8_t* q8, float* qscale, uint16_t* v16, double* partial, hipStream_t st) {
+    PrepArgs a{};
+    a.q = q; a.k = k; a.v = v; a.H = H; a.Nq = Nq; a.Nkv = Nkv; a.nq_pad = nq_pad; a.nkv_pad = nkv_pad;
+    a.cmul = cmul; a.q8 = q8; a.qscale = qscale; a.v16 = v16; a.partial = partial;
+    a.nq_blk = (int)(nq_pad / blkq);
+    a.nv_tile = (int)(nkv_pad / 64);
+    a.ngroups = (Nkv + kGroup - 1) / kGroup;
+    const int gpw = D == 128 ? 1 : 2;
+    a.nk_wg = smooth_k ? (a.ngroups + gpw - 1) / gpw : 0;
+    if (D == 128) return launch_prep_d<128>(a, B, blkq, st);
+    if (D == 64) return launch_prep_d<64>(a, B, blkq, st);
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
+                               const double* partial, float* kmean, int8_t* codes, float* scales, hipStream_t st) {
+    const int ngroups = (N + kGroup - 1) / kGroup;
+    dim3 grid((unsigned)((n_pad + kGroup - 1) / kGroup), (unsigned)H, (unsigned)B), block(256);
+#define SAGE_LAUNCH_KQ(DD, BLK)                                                                          \
+    hipLaunchKernelGGL((kquant_group_kernel<DD, BLK>), grid, block, 0, st, k.p, k.sb, k.sh, k.sn, N, H, \
+                       n_pad, partial, ngroups, kmean, codes, scales)
+    if (D == 128) {
+        switch (blk) {
+            case 32: SAGE_LAUNCH_KQ(128, 32); break;
+            case 64: SAGE_LAUNCH_KQ(128, 64); break;
+            case 128: SAGE_LAUNCH_KQ(128, 128); break;
+            default: return hipErrorInvalidValue;
+        }
+    } else if (D == 64) {
+        switch (blk) {
+            case 32: SAGE_LAUNCH_KQ(64, 32); break;
+            case 64: SAGE_LAUNCH_KQ(64, 64); break;
+            case 128: SAGE_LAUNCH_KQ(64, 128); break;
+            default: return hipErrorInvalidValue;
+        }
+    } else {
+        return hipErrorInvalidValue;
+    }
+#undef SAGE_LAUNCH_KQ
     return hipGetLastError();
 }
 

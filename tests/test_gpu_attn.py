@@ -91,6 +91,24 @@ def test_one_shot_matches_checker_and_referee(oracle, wid, S):
     assert cos_ref >= (0.998 if wid == 3 else COS), (cos_ref, mx_ref)
 
 
+@pytest.mark.parametrize("wid,S,smooth", [(2, 1100, True), (1, 1024, True), (3, 333, False), (1, 77, True)])
+def test_one_shot_equals_stage_pipeline(wid, S, smooth):
+    """The one-shot call runs fused launches (Q quantize + V repack + K-mean sums in one kernel,
+    K mean + K quantize in another); the stage entry points run them separately.  The stage
+    outputs are proven bit-exact against the CPU checker, so bit-equal O from both routes
+    carries that proof over to the fused kernels."""
+    import torch
+    import gpu_harness as H
+    w = WORKLOADS[wid]
+    w = w.scaled(B=2, H=3, S=S)
+    q, k, v = make_inputs(w)
+    got = _one_shot(q, k, v, w.scale, 0, w.blkq, w.blkk, smooth)
+    g = H.quant_qk(q, k, w.scale, w.blkq, w.blkk, smooth)["dev"]
+    gv = H.quant_v(v, 0)["dev"]
+    staged, _ = H.attn_fwd(g["q8"], g["qscale"], w.blkq, g["k8"], g["kscale"], w.blkk, gv["vq"], None, 0, S, S)
+    np.testing.assert_array_equal(got, staged)
+
+
 def test_default_recipe_entry_point(oracle):
     """mi355_sage_sdpa_bf16 without the recipe arguments: blkq 128 / blkk 64 / smoothing on."""
     import gpu_harness as H
