@@ -36,12 +36,31 @@ __device__ __forceinline__ float wave_max(float v) {
 // the block's BLK x D tile lives in registers between the absmax pass and the
 // encode pass, so HBM sees one read of bf16 and one write of int8.
 // ---------------------------------------------------------------------------
-// `mean` points at the D means of this (b,h) (global or LDS), or is null.
-template <int D, int BLK, bool IS_K>
+// rint(x / sc) for |x / sc| <= ~127 without paying a full IEEE divide per element: x * (1/sc)
+// is within 2^-15 of the correctly rounded quotient (both below 128), so whenever it lies at
+// least 2^-12 away from a rounding tie it rounds to the same integer; the few elements near
+// a tie (and any non-finite case) take the true divide.  `fast` is false when sc is so small
+// or large that 1/sc is not a normal number.
+__device__ __forceinline__ float rint_quotient(float x, float sc, float rinv, bool fast) {
+    const float q = x * rinv;
+    float n = rintf(q);
+    if (!fast || !(fabsf(q - n) <= 0.5f - 0x1p-12f)) n = rintf(x / sc);
+    return n;
+}
+
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// `mean` points at the D means of this (b,h) (global or LDS), or is null.  `hook` runs after
+// the tile's loads are issued and before anything reads `mean` (it may compute the mean into
+// LDS; it must end with a barrier if it does).
+template <int D, int BLK, bool IS_K, typename Hook = NoHook>
 __device__ __forceinline__ void quant_i8_block(
     int t, int h, int b, const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, float cmul, const float* mean,
-    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, float* red) {
+    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, float* red,
+    Hook hook = Hook()) {
     constexpr int CPR = D / 8;                 // 16-byte chunks per row
     constexpr int NCH = BLK * CPR / 256;       // chunks per thread
     static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
@@ -50,15 +69,23 @@ __device__ __forceinline__ void quant_i8_block(
     const int64_t bh = (int64_t)b * H + h;
     const uint16_t* src = x + b * sb + h * sh;
 
+    u32x4 raw[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = i * 256 + tid;
+        const int row = r0 + c / CPR, col = (c % CPR) * 8;
+        raw[i] = u32x4{0u, 0u, 0u, 0u};
+        if (row < N) raw[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+    }
+    hook();
+
     float v[NCH][8];
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
         const int c = i * 256 + tid;
         const int row = r0 + c / CPR, col = (c % CPR) * 8;
-        u32x4 w = {0u, 0u, 0u, 0u};
-        if (row < N) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
-        unpack8(w, v[i]);
+        unpack8(raw[i], v[i]);
         if (IS_K) {
             if (mean != nullptr) {
                 const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
@@ -95,6 +122,8 @@ __device__ __forceinline__ void quant_i8_block(
     const bool real_block = r0 < N;
     const float sc = (real_block && amax > 0.0f) ? amax / 127.0f : 1.0f;
     if (tid == 0) scales[bh * (n_pad / BLK) + t] = sc;
+    const bool fast = sc >= 0x1p-100f && sc <= 0x1p100f;
+    const float rinv = 1.0f / sc;
 
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -104,7 +133,7 @@ __device__ __forceinline__ void quant_i8_block(
         if (row < N) {
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                float r = rintf(v[i][e] / sc);
+                float r = rint_quotient(v[i][e], sc, rinv, fast);
                 r = fminf(fmaxf(r, -127.0f), 127.0f);
                 pk[e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
             }
@@ -218,7 +247,14 @@ __global__ __launch_bounds__(256) void kmean_final_kernel(
     const int d = (int)(i % D);
     const double* p = partial + bh * ngroups * D + d;
     double sum = 0.0;
-    for (int g = 0; g < ngroups; g++) sum += p[(int64_t)g * D];
+    for (int g0 = 0; g0 < ngroups; g0 += 8) {
+        double v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = p[(int64_t)(g0 + j < ngroups ? g0 + j : ngroups - 1) * D];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (g0 + j < ngroups) sum += v[j];
+    }
     kmean[i] = (float)(sum / (double)N);
 }
 
@@ -252,42 +288,63 @@ __device__ __forceinline__ uint16_t f32_to_f16_sat(float x) {
     return __half_as_ushort(__float2half_rn(x));
 }
 
+// LDS tile: 64 slots x D halves, unpadded; the 16-byte chunk index of a row is XORed with
+// 2*(slot/8) so that both the row-wise 16-byte writes and the column-wise dword reads below
+// touch every bank once (D = 128: 16 chunks; D = 64: 8 chunks, XOR with slot/8 instead).
+template <int D>
+__device__ __forceinline__ int v_tile_chunk(int slot, int chunk) {
+    return D == 128 ? (chunk ^ (((slot >> 3) & 7) << 1)) : (chunk ^ ((slot >> 3) & 7));
+}
+
 template <int D>
 __device__ __forceinline__ void quant_v_f16_body(
     int t, int h, int b, const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, uint16_t* __restrict__ out, uint16_t* tile) {
     constexpr int CPR = D / 8;
-    constexpr int LD = D + 8;                              // padded row (halves), keeps 16-byte alignment
     const int tid = threadIdx.x;
     const uint16_t* src = v + b * sb + h * sh;
+    u32x4 raw[64 * CPR / 256];
 #pragma unroll
     for (int i = 0; i < 64 * CPR / 256; i++) {
         const int c = i * 256 + tid;
         const int key = c / CPR, col = (c % CPR) * 8;
         const int row = t * 64 + key;
-        u32x4 w = {0u, 0u, 0u, 0u};
-        if (row < N) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+        raw[i] = u32x4{0u, 0u, 0u, 0u};
+        if (row < N) raw[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+    }
+#pragma unroll
+    for (int i = 0; i < 64 * CPR / 256; i++) {
+        const int c = i * 256 + tid;
+        const int key = c / CPR, chunk = c % CPR;
         float x[8];
-        unpack8(w, x);
+        unpack8(raw[i], x);
         u32x4 o;
         o.x = f32_to_f16_sat(x[0]) | ((uint32_t)f32_to_f16_sat(x[1]) << 16);
         o.y = f32_to_f16_sat(x[2]) | ((uint32_t)f32_to_f16_sat(x[3]) << 16);
         o.z = f32_to_f16_sat(x[4]) | ((uint32_t)f32_to_f16_sat(x[5]) << 16);
         o.w = f32_to_f16_sat(x[6]) | ((uint32_t)f32_to_f16_sat(x[7]) << 16);
-        *reinterpret_cast<u32x4*>(&tile[v_slot_f16(key) * LD + col]) = o;
+        const int slot = v_slot_f16(key);
+        *reinterpret_cast<u32x4*>(&tile[slot * D + v_tile_chunk<D>(slot, chunk) * 8]) = o;
     }
     __syncthreads();
     uint16_t* dst = out + ((((int64_t)b * H + h) * (n_pad / 64)) + t) * (int64_t)(D * 64);
-    // output chunk = (channel d, 8 consecutive slots)
+    // work item = (channel pair, 8 consecutive slots): eight dword reads, two 16-byte stores
+    const uint32_t* tile32 = reinterpret_cast<const uint32_t*>(tile);
 #pragma unroll
-    for (int i = 0; i < D * 8 / 256; i++) {
+    for (int i = 0; i < (D / 2) * 8 / 256; i++) {
         const int c = i * 256 + tid;
-        const int d = c >> 3, s0 = (c & 7) * 8;
-        uint32_t pk[4];
+        const int dp = c >> 3, s0 = (c & 7) * 8;            // channels 2*dp, 2*dp+1
+        uint32_t w[8];
 #pragma unroll
-        for (int e = 0; e < 4; e++)
-            pk[e] = tile[(s0 + 2 * e) * LD + d] | ((uint32_t)tile[(s0 + 2 * e + 1) * LD + d] << 16);
-        *reinterpret_cast<u32x4*>(dst + d * 64 + s0) = u32x4{pk[0], pk[1], pk[2], pk[3]};
+        for (int e = 0; e < 8; e++)
+            w[e] = tile32[(s0 + e) * (D / 2) + v_tile_chunk<D>(s0 + e, dp >> 2) * 4 + (dp & 3)];
+        u32x4 lo, hi;
+        lo.x = __builtin_amdgcn_perm(w[1], w[0], 0x05040100u); hi.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+        lo.y = __builtin_amdgcn_perm(w[3], w[2], 0x05040100u); hi.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+        lo.z = __builtin_amdgcn_perm(w[5], w[4], 0x05040100u); hi.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
+        lo.w = __builtin_amdgcn_perm(w[7], w[6], 0x05040100u); hi.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
+        *reinterpret_cast<u32x4*>(dst + (2 * dp) * 64 + s0) = lo;
+        *reinterpret_cast<u32x4*>(dst + (2 * dp + 1) * 64 + s0) = hi;
     }
 }
 
@@ -295,7 +352,7 @@ template <int D>
 __global__ __launch_bounds__(256) void quant_v_f16_kernel(
     const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, uint16_t* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * (D + 8)];
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * D];
     quant_v_f16_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, v, sb, sh, sn, N, H, n_pad, out, tile);
 }
 
@@ -316,8 +373,8 @@ hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t
 // group sums are independent of each other: one launch runs all three as workgroup roles
 // (saves two launch gaps and fills the chip while each role alone is too short to).  The
 // K quantizer then takes its mean straight from the group partials (added in group
-// order, the same arithmetic as kmean_final_kernel) and covers a whole 256-token group
-// per workgroup, which also removes the separate final-mean launch.
+// order, the same arithmetic as kmean_final_kernel) while its tile loads are in flight,
+// which removes the separate final-mean launch.
 // ---------------------------------------------------------------------------
 struct PrepArgs {
     View q, k, v;
@@ -333,7 +390,7 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
     constexpr int GPW = 256 / (16 * (D / 8));             // K-mean groups per workgroup
     union Smem {
         float red[4];
-        uint16_t tile[64 * (D + 8)];
+        uint16_t tile[64 * D];
         double leafsum[GPW][16][D + 2];
     };
     __shared__ __attribute__((aligned(16))) Smem sm;
@@ -355,33 +412,51 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
     }
 }
 
+template <int D>
+struct MeanFromPartials {
+    const double* partial;      // this (b,h)'s [ngroups][D] group sums, or null
+    int ngroups, N;
+    float* mean_s;              // LDS, D floats
+    float* kmean_out;           // where to publish the mean, or null
+    __device__ __forceinline__ void operator()() const {
+        if (partial == nullptr) return;
+        if (threadIdx.x < D) {
+            // loads eight at a time (independent, all in flight together); adds strictly in
+            // group order
+            double sum = 0.0;
+            for (int g0 = 0; g0 < ngroups; g0 += 8) {
+                double p[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int g = g0 + j < ngroups ? g0 + j : ngroups - 1;
+                    p[j] = partial[(int64_t)g * D + threadIdx.x];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (g0 + j < ngroups) sum += p[j];
+            }
+            const float m = (float)(sum / (double)N);
+            mean_s[threadIdx.x] = m;
+            if (kmean_out != nullptr) kmean_out[threadIdx.x] = m;
+        }
+        __syncthreads();
+    }
+};
+
 template <int D, int BLK>
-__global__ __launch_bounds__(256) void kquant_group_kernel(
+__global__ __launch_bounds__(256) void kquant_fused_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, const double* __restrict__ partial, int ngroups,
     float* __restrict__ kmean, int8_t* __restrict__ codes, float* __restrict__ scales) {
     __shared__ float mean_s[D];
     __shared__ float red[4];
-    const int grp = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int64_t bh = (int64_t)b * H + h;
     const bool smooth = partial != nullptr;
-    if (smooth && threadIdx.x < D) {
-        const double* p = partial + bh * ngroups * D + threadIdx.x;
-        double sum = 0.0;
-        for (int g = 0; g < ngroups; g++) sum += p[(int64_t)g * D];
-        const float m = (float)(sum / (double)N);
-        mean_s[threadIdx.x] = m;
-        if (grp == 0) kmean[bh * D + threadIdx.x] = m;
-    }
-    __syncthreads();
-#pragma unroll 1
-    for (int i = 0; i < kGroup / BLK; i++) {
-        const int t = grp * (kGroup / BLK) + i;
-        if ((int64_t)t * BLK >= n_pad) break;
-        quant_i8_block<D, BLK, true>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
-                                     codes, scales, nullptr, red);
-        __syncthreads();                                   // `red` is reused by the next block
-    }
+    MeanFromPartials<D> hook{smooth ? partial + bh * ngroups * D : nullptr, ngroups, N, mean_s,
+                             (smooth && t == 0) ? kmean + bh * D : nullptr};
+    quant_i8_block<D, BLK, true>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
+                                 codes, scales, nullptr, red, hook);
 }
 
 template <int D>
@@ -415,9 +490,9 @@ hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B,
 hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
                                const double* partial, float* kmean, int8_t* codes, float* scales, hipStream_t st) {
     const int ngroups = (N + kGroup - 1) / kGroup;
-    dim3 grid((unsigned)((n_pad + kGroup - 1) / kGroup), (unsigned)H, (unsigned)B), block(256);
+    dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
 #define SAGE_LAUNCH_KQ(DD, BLK)                                                                          \
-    hipLaunchKernelGGL((kquant_group_kernel<DD, BLK>), grid, block, 0, st, k.p, k.sb, k.sh, k.sn, N, H, \
+    hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK>), grid, block, 0, st, k.p, k.sb, k.sh, k.sn, N, H, \
                        n_pad, partial, ngroups, kmean, codes, scales)
     if (D == 128) {
         switch (blk) {
