@@ -1,6 +1,6 @@
 // sage_attn.hip — flash-style attention on quantized operands for gfx950.
 //
-// One workgroup (4 waves) owns 128 query rows of one (batch, head); wave w owns
+// One workgroup (8 waves) owns 256 query rows of one (batch, head); wave w owns
 // rows 32w..32w+31.  The kernel works on the TRANSPOSED problem so that no
 // cross-lane data movement is needed between the two matrix products:
 //
@@ -16,8 +16,9 @@
 // the matching slot order (v_slot_f16 / v_slot_fp8).
 //
 // Pipeline.  K and V^T tiles of 64 keys travel global -> LDS with register-
-// bypassing copies (global_load_lds_dwordx4) into 3-deep rings; the 16-byte-chunk
-// XOR swizzle is applied on the source side of the copy.  Iteration t computes
+// bypassing copies (global_load_lds_dwordx4) into rings (K: 3 slots, V^T: 4), two
+// iterations ahead of their use; the 16-byte-chunk XOR swizzle is applied on the source
+// side of the copy.  Iteration t computes
 // the scores of tile t, then interleaves — one matrix instruction, then the
 // exponentials of two scores, in program order — the softmax of tile t with
 // P.V of tile t-1, so the matrix pipe and the vector ALU of a SIMD run
@@ -75,13 +76,29 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
-// The int32 score accumulators start at the bit pattern of 1.5*2^23 instead of 0, so a
-// finished accumulator, read as fp32, IS the float 12582912 + dot (exact while
-// |dot| < 2^22; the largest possible |dot| is 128*127*127 < 2^21): no int->float
-// conversion is needed and dequantisation, max subtraction and the exponent argument
-// collapse into one FMA per score.
-constexpr int kMagicI = 0x4B400000;
-constexpr float kMagicF = 12582912.0f;
+// The int32 score accumulators start at the bit pattern of the float 1/(2*pi) instead of 0.
+// That pattern is 2^-3 * (1 + 2292099 * 2^-23), so adding an integer dot with
+// |dot| < 2292099 (the largest possible |dot| is 128*127*127 = 2064512) changes only the
+// mantissa: a finished accumulator, read as fp32, IS the float 1/(2*pi) + dot * 2^-26.  No
+// int->float conversion is needed and dequantisation, max subtraction and the exponent
+// argument collapse into one FMA per score (the scale carries the factor 2^26).  This
+// particular constant is one the matrix instruction takes as an inline operand, so it costs
+// neither registers nor moves.
+constexpr int kMagicI = 0x3E22F983;
+constexpr float kMagicF = 0.15915494309189532f;        // the same 32 bits
+constexpr float kMagicUnit = 67108864.0f;               // 2^26: accumulator-as-float steps per integer
+
+// First matrix instruction of a score chain: accumulator input = the inline constant above.
+// (The compiler keeps a splat constant in 16 registers and copies them into the accumulator
+// for every chain; the instruction itself can take this constant as an immediate.)  The
+// following instructions of the chain are compiler-visible builtins that accumulate in place,
+// so everything that reads the finished scores is ordered against a matrix instruction the
+// compiler knows about.
+__device__ __forceinline__ v16i mfma_i8_from_magic(const v4i& a, const v4i& b) {
+    v16i d;
+    asm("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0.15915494" : "=&v"(d) : "v"(a), "v"(b));
+    return d;
+}
 
 // A row's reference maximum is only refreshed (and the accumulators rescaled) when a tile
 // exceeds it by more than tau powers of two; until then p = exp2(s - m_used) may reach
@@ -155,7 +172,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
 #pragma unroll
         for (int s = 0; s < KSTEPS; s++) qf[s] = *reinterpret_cast<const v4i*>(qp + s * 32);
     }
-    const float sq = qscale[bh * (nq_pad / blkq) + qrow / blkq];
+    const float sq = qscale[bh * (nq_pad / blkq) + qrow / blkq] * kMagicUnit;
 
     // K scales of this head are staged in LDS once: a global load inside the main loop
     // would make the compiler wait for ALL outstanding vector-memory operations, i.e. for the
@@ -212,10 +229,6 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
 #pragma unroll
         for (int i = 0; i < V_CH; i++) dma16(g, vsrc[i], __builtin_amdgcn_readfirstlane(vdst[i] + slot * V_BYTES));
     };
-
-    v16i magic;
-#pragma unroll
-    for (int i = 0; i < 16; i++) magic[i] = kMagicI;
 
     v16f oacc[DB];
 #pragma unroll
@@ -291,7 +304,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int st = 0; st < KSTEPS; st++)
-                s[kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], st == 0 ? magic : s[kb], 0, 0, 0);
+                s[kb] = st == 0 ? mfma_i8_from_magic(kf[kb][0], qf[0])
+                                : __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], s[kb], 0, 0, 0);
 
         float f[2], c0[2];
 #pragma unroll
@@ -320,7 +334,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
                     mb = max(max(mb, s[kb][i + 2]), s[kb][i + 3]);
                 }
                 const int mi = max(max(ma, mb), max(s[kb][14], s[kb][15]));
-                const float mk = MASK && mi < 0 ? -INFINITY : (float)(mi - kMagicI) * f[kb];
+                const float mk = MASK && mi < 0 ? -INFINITY : (float)(mi - kMagicI) * (f[kb] * (1.0f / kMagicUnit));
                 mt = fmaxf(mt, mk);
             }
             const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);

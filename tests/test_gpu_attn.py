@@ -240,5 +240,12 @@ def test_workload2_full_size(oracle):
             assert mx <= MAX_ABS and cos >= 0.9999, (h, r0, cos, mx)
     qd, kd, vd = (H.dev_bf16(x).float().permute(0, 2, 1, 3) for x in (q, k, v))
     ref = torch.nn.functional.scaled_dot_product_attention(qd, kd, vd, scale=w.scale).permute(0, 2, 1, 3)
-    cos, mx = H.cos_maxabs(gotf, ref.cpu().numpy())
+    refn = ref.cpu().numpy()
+    cos, mx = H.cos_maxabs(gotf, refn)
     assert cos >= COS, (cos, mx)
+    # every row on its own
+    num = (gotf.astype(np.float64) * refn).sum(-1)
+    den = np.linalg.norm(gotf.astype(np.float64), axis=-1) * np.linalg.norm(refn.astype(np.float64), axis=-1)
+    rowcos = num / den
+    assert rowcos.min() >= 0.995, rowcos.min()
+    assert np.abs(gotf - refn).max() <= 3e-2, np.abs(gotf - refn).max()
