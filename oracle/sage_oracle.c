@@ -252,6 +252,121 @@ static int bad_quant_args(const void* x, int B, int H, int N, int D, const int64
     return 0;
 }
 
+/* ---- the two ops in front of the path: RMSNorm over D, interleaved RoPE -------------- */
+
+/* serenitymojo/ops/norm.mojo:47-79 (_rms_norm_kernel_f32): out = x * (1/sqrt(mean(x^2)+eps)) * g.
+ * The reference adds the squares in the order of its 256-thread shared-memory tree; an fp32
+ * sum's last bit depends on that order and nothing the reference holds pins it (its vectors
+ * have 6 columns and a 1e-6 bar), so the order here is the one the GPU kernel can afford:
+ * runs of 8 consecutive columns added left to right, then the run sums combined pairwise
+ * (neighbours first: strides 1, 2, 4, ... runs).  Column counts that are not a multiple of 8
+ * are added left to right. */
+static float sumsq_blocked(const float* v, int cols) {
+    int runs = cols / 8;
+    if (cols % 8 == 0 && runs > 0 && runs <= 1024) {
+        float part[1024];
+        for (int r = 0; r < runs; r++) {
+            float a = 0.0f;
+            for (int e = 0; e < 8; e++) {
+                float sq = v[r * 8 + e] * v[r * 8 + e];
+                a = a + sq;
+            }
+            part[r] = a;
+        }
+        /* pairwise, neighbours first; an odd one out moves up unchanged */
+        for (int n = runs; n > 1; n = (n + 1) / 2) {
+            for (int r = 0; r + 1 < n; r += 2) part[r / 2] = part[r] + part[r + 1];
+            if (n & 1) part[n / 2] = part[n - 1];
+        }
+        return part[0];
+    }
+    float a = 0.0f;
+    for (int c = 0; c < cols; c++) {
+        float sq = v[c] * v[c];
+        a = a + sq;
+    }
+    return a;
+}
+
+static float rms_inv(const float* v, int cols, float eps) {
+    float ss = sumsq_blocked(v, cols);
+    float mean = ss / (float)cols;
+    return 1.0f / sqrtf(mean + eps);           /* IEEE sqrt and divide (norm.mojo:73) */
+}
+
+int sage_oracle_rms_norm_f32(const float* x, const float* g, int64_t rows, int cols, float eps, float* out) {
+    if (!x || !g || !out || rows <= 0 || cols <= 0) return -1;
+    for (int64_t r = 0; r < rows; r++) {
+        float inv = rms_inv(x + r * cols, cols, eps);
+        for (int c = 0; c < cols; c++) {
+            float t = x[r * cols + c] * inv;    /* (v * inv) * g, norm.mojo:78 */
+            out[r * cols + c] = t * g[c];
+        }
+    }
+    return 0;
+}
+
+/* serenitymojo/ops/rope.mojo:7-9, :104-122: pairs (x[2i], x[2i+1]); separate multiplies, then
+ * one subtract / add (no fused multiply-add). */
+int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const float* sn,
+                                     int64_t rows, int D, float* out) {
+    if (!x || !cs || !sn || !out || rows <= 0 || D <= 0 || (D & 1)) return -1;
+    int half = D / 2;
+    for (int64_t r = 0; r < rows; r++)
+        for (int i = 0; i < half; i++) {
+            float x0 = x[r * D + 2 * i], x1 = x[r * D + 2 * i + 1];
+            float cv = cs[r * half + i], sv = sn[r * half + i];
+            float a = x0 * cv, b = x1 * sv, c = x0 * sv, d = x1 * cv;
+            out[r * D + 2 * i] = a - b;
+            out[r * D + 2 * i + 1] = c + d;
+        }
+    return 0;
+}
+
+/* bf16 activations: RMSNorm with a bf16 gain, stored as bf16 (norm.mojo:81-114), then
+ * interleaved RoPE with fp32 tables on that bf16 tensor, stored as bf16 (rope.mojo:104-122).
+ * x is logical [B,H,N,D] through strides; tables are [rows_per_batch, D/2] with row n*H + h
+ * (sampling/klein_sampler.mojo:305-307), shared by all batches when table_batch_rows == 0, else
+ * batch b starts at row b*table_batch_rows; cs == NULL skips the rotation.
+ * y: contiguous [B,N,H,D] bf16. */
+int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
+                               const uint16_t* gain, float eps, const float* cs, const float* sn,
+                               int64_t table_batch_rows, uint16_t* y) {
+    if (!x || !st || !gain || !y || B <= 0 || H <= 0 || N <= 0 || D <= 0 || (D & 1) || D > 1024) return -1;
+    if ((cs == NULL) != (sn == NULL)) return -1;
+    int half = D / 2;
+    int64_t work = (int64_t)B * N * H;
+#pragma omp parallel for schedule(static)
+    for (int64_t w = 0; w < work; w++) {
+        int h = (int)(w % H);
+        int n = (int)((w / H) % N);
+        int b = (int)(w / ((int64_t)H * N));
+        float v[1024], t[1024];
+        const uint16_t* src = x + b * st[0] + h * st[1] + (int64_t)n * st[2];
+        for (int d = 0; d < D; d++) v[d] = sage_oracle_bf16_to_f32(src[d * st[3]]);
+        float inv = rms_inv(v, D, eps);
+        for (int d = 0; d < D; d++) {
+            float a = v[d] * inv;
+            float gq = sage_oracle_bf16_to_f32(gain[d]);
+            t[d] = sage_oracle_bf16_to_f32(sage_oracle_f32_to_bf16(a * gq));
+        }
+        uint16_t* dst = y + (((int64_t)b * N + n) * H + h) * D;
+        if (cs) {
+            int64_t row = (int64_t)b * table_batch_rows + (int64_t)n * H + h;
+            for (int i = 0; i < half; i++) {
+                float x0 = t[2 * i], x1 = t[2 * i + 1];
+                float cv = cs[row * half + i], sv = sn[row * half + i];
+                float a = x0 * cv, bb = x1 * sv, c = x0 * sv, dd = x1 * cv;
+                dst[2 * i] = sage_oracle_f32_to_bf16(a - bb);
+                dst[2 * i + 1] = sage_oracle_f32_to_bf16(c + dd);
+            }
+        } else {
+            for (int d = 0; d < D; d++) dst[d] = sage_oracle_f32_to_bf16(t[d]);
+        }
+    }
+    return 0;
+}
+
 /* One block of `rows` tokens by D channels, already transformed to fp32 in
  * `tile` (row-major rows x D): scale and codes. */
 static void quant_block_i8(const float* tile, int rows, int D, int8_t* dst, float* scale_out) {

@@ -16,6 +16,10 @@
  *       (ops/parity/sdpa_math_ref.txt, ops_smoke2.mojo:239-278) + closed forms.
  *   bf16 / fp16 / e4m3 codecs ............. reference KATs
  *       (ops/tests/fp8_quant_smoke.mojo:108-143) + torch / numpy library codecs.
+ *   sage_oracle_rms_norm_f32 / _rope_interleaved_f32 ... reference vectors
+ *       (ops_smoke.mojo:78-96, ops_smoke2.mojo:95-120) + the closed form of
+ *       ops_smoke2.mojo:372-403.  sage_oracle_norm_rope_bf16 composes them with RNE bf16
+ *       stores; its last-bit behaviour (summation order, no FMA) is PARITY UNPINNED.
  *   sage_oracle_quant_q / _kmean / _quant_k / _quant_v_* , sage_oracle_attn:
  *       PARITY UNPINNED by the reference — it holds no INT8 / SageAttention
  *       code, test or vector.  They are pinned only by closed forms, invariants
@@ -60,6 +64,22 @@ int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, 
                                 int B, int H, int Nq, int Nkv, int D, float scale,
                                 const int64_t* qs, const int64_t* ks,
                                 const int64_t* vs, const int64_t* os);
+
+/* ---- the two ops in front of the path (fused into the quantizers by the product) ---- */
+/* RMSNorm rows x cols in fp32: serenitymojo/ops/norm.mojo:47-79.  Pinned by the reference's
+ * vector serenitymojo/ops_smoke.mojo:78-96 and the closed form of ops_smoke2.mojo:372-403
+ * (to their fp32 tolerance; the summation order of the squares is this file's own). */
+int sage_oracle_rms_norm_f32(const float* x, const float* g, int64_t rows, int cols, float eps, float* out);
+/* Interleaved RoPE in fp32: serenitymojo/ops/rope.mojo:7-9.  Pinned by ops_smoke2.mojo:95-120. */
+int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const float* sn,
+                                     int64_t rows, int D, float* out);
+/* The bf16 pipeline rms_norm -> (bf16) -> rope_interleaved -> (bf16) of
+ * serenitymojo/models/klein/single_block.mojo:977-981 on a strided [B,H,N,D] view; output
+ * contiguous [B,N,H,D].  Tables [.., D/2] fp32 with row n*H + h (+ b*table_batch_rows);
+ * cs == NULL: no rotation.  The bf16 roundings are RNE (ops/torch_bf16.mojo:27-60). */
+int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
+                               const uint16_t* gain, float eps, const float* cs, const float* sn,
+                               int64_t table_batch_rows, uint16_t* y);
 
 /* ---- quantizers --------------------------------------------------------- */
 /* Padded token count used by every quantized tensor: N rounded up to `mult`. */

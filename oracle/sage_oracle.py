@@ -76,6 +76,14 @@ def lib():
         L.sage_oracle_sdpa_bf16.restype = ctypes.c_int
         L.sage_oracle_sdpa_bf16.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [
                                             ctypes.c_int] * 4
+        L.sage_oracle_rms_norm_f32.restype = ctypes.c_int
+        L.sage_oracle_rms_norm_f32.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+                                               ctypes.c_float, ctypes.c_void_p]
+        L.sage_oracle_rope_interleaved_f32.restype = ctypes.c_int
+        L.sage_oracle_rope_interleaved_f32.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        L.sage_oracle_norm_rope_bf16.restype = ctypes.c_int
+        L.sage_oracle_norm_rope_bf16.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p, ctypes.c_float,
+                                                 ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         L.sage_oracle_num_threads.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -164,6 +172,43 @@ def sdpa_f32(q, k, v, scale, online=False):
             strides_bshd(Sq, H, D), strides_bshd(Skv, H, D), strides_bshd(Skv, H, D),
             strides_bshd(Sq, H, D)), "sdpa_f32")
     return o
+
+
+def rms_norm_f32(x, g, eps):
+    """x [rows, cols] fp32, g [cols] fp32 -> fp32 (serenitymojo/ops/norm.mojo:47-79)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    g = np.ascontiguousarray(g, dtype=np.float32)
+    out = np.empty_like(x)
+    _chk(lib().sage_oracle_rms_norm_f32(_p(x), _p(g), x.shape[0], x.shape[1], eps, _p(out)), "rms_norm_f32")
+    return out
+
+
+def rope_interleaved_f32(x, cos, sin):
+    """x [rows, D], cos/sin [rows, D/2], all fp32 (serenitymojo/ops/rope.mojo:7-9)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    cos = np.ascontiguousarray(cos, dtype=np.float32)
+    sin = np.ascontiguousarray(sin, dtype=np.float32)
+    out = np.empty_like(x)
+    _chk(lib().sage_oracle_rope_interleaved_f32(_p(x), _p(cos), _p(sin), x.shape[0], x.shape[1], _p(out)),
+         "rope_interleaved_f32")
+    return out
+
+
+def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=0):
+    """x: uint16 [B,S,H,D] bf16 bits; gain: uint16 [D]; cos/sin: fp32 [rows, D/2] with row s*H + h
+    (plus b*table_batch_rows), or None for no rotation.  Returns uint16 [B,S,H,D]."""
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
+    g = np.ascontiguousarray(gain_bf16, dtype=np.uint16)
+    B, S, H, D = x.shape
+    y = np.empty_like(x)
+    if cos is not None:
+        cos = np.ascontiguousarray(cos, dtype=np.float32)
+        sin = np.ascontiguousarray(sin, dtype=np.float32)
+    _chk(lib().sage_oracle_norm_rope_bf16(_p(x), B, H, S, D, strides_bshd(S, H, D), _p(g), eps,
+                                          _p(cos) if cos is not None else None,
+                                          _p(sin) if sin is not None else None, table_batch_rows, _p(y)),
+         "norm_rope_bf16")
+    return y
 
 
 def quant_q(q_bf16, scale, blkq, npad_mult=None):

@@ -8,6 +8,8 @@ Sources (relative to the reference checkout):
   serenitymojo/ops/parity/sdpa_math_ref.txt        tags dh128 [1,8,32,128], dh512 [1,64,1,512]
       inputs are the closed forms of ops/parity/sdpa_math_parity.mojo:32-50
   serenitymojo/ops_smoke2.mojo:239-278              q/k/v/out literals, [1,4,2,8], scale 0.35355339
+  serenitymojo/ops_smoke.mojo:78-96                 rms_norm x[3,6], g[6], eps 1e-6 -> y[3,6]
+  serenitymojo/ops_smoke2.mojo:92-120               rope x[3,8], cos/sin[3,4] -> interleaved y[3,8]
 
 Run once where the reference is mounted:  python tests/golden/make_fixtures.py [/root/reference]
 """
@@ -45,6 +47,27 @@ def main():
     kat["scale"] = 0.35355339
     with open(os.path.join(HERE, "ops_smoke2_sdpa_kat.json"), "w") as f:
         json.dump(kat, f, indent=0)
+
+    def literals(text, name, count):
+        m = re.search(r"var %s = _lf\((.*?)\n\s*\)" % name, text, re.S)
+        vals = [float(x) for x in re.findall(r"-?\d+\.\d+", m.group(1))]
+        assert len(vals) == count, (name, len(vals))
+        return vals
+
+    pre = {}
+    with open(os.path.join(ref, "serenitymojo/ops_smoke.mojo")) as f:
+        text = "\n".join(f.read().split("\n")[77:96])
+    pre["rms_x"] = literals(text, "x_rms", 18)
+    pre["rms_g"] = literals(text, "g_rms", 6)
+    pre["rms_y"] = literals(text, "y_rms_ref", 18)
+    pre["rms_eps"] = 1e-6
+    text = "\n".join(lines[91:120])
+    pre["rope_x"] = literals(text, "x_rope", 24)
+    pre["rope_cos"] = literals(text, "cos_rope", 12)
+    pre["rope_sin"] = literals(text, "sin_rope", 12)
+    pre["rope_y_interleaved"] = literals(text, "y_int_ref", 24)
+    with open(os.path.join(HERE, "ops_smoke_rmsnorm_rope_kat.json"), "w") as f:
+        json.dump(pre, f, indent=0)
     print("wrote fixtures to", HERE)
 
 

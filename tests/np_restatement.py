@@ -120,3 +120,46 @@ def attn_float64(q8, qs, blkq, k8, ks, blkk, v_f32, Sq, Skv, p_codec):
             l = p.astype(np.float64).sum(axis=1, keepdims=True)
             out[b, :, h, :] = (p_codec(p).astype(np.float64) @ v_f32[b, h, :Skv].astype(np.float64)) / l
     return out
+
+
+# ---------------------------------------------------------------------------
+# RMSNorm + interleaved RoPE in front of the quantizers (bf16 activations)
+#   ss   = sum of squares: runs of 8 consecutive channels left to right, then the run sums
+#          combined pairwise, neighbours first (fp32 throughout)
+#   inv  = 1 / sqrt(ss / D + eps)                       (fp32, IEEE)
+#   y    = bf16((x * inv) * gain)
+#   out[2i], out[2i+1] = bf16(y0*c - y1*s), bf16(y0*s + y1*c)   (products rounded separately)
+# ---------------------------------------------------------------------------
+def f32_to_bf16_bits_rne(x):
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    r = u + 0x7FFF + ((u >> 16) & 1)
+    return (r >> 16).astype(np.uint16)
+
+
+def norm_rope_bf16(x_bits_bshd, gain_bits, eps, cos=None, sin=None, table_batch_rows=0):
+    B, S, H, D = x_bits_bshd.shape
+    x = bf16_to_f32(x_bits_bshd)                                   # [B,S,H,D]
+    sq = (x * x).astype(np.float32).reshape(B, S, H, D // 8, 8)
+    part = np.zeros((B, S, H, D // 8), np.float32)
+    for e in range(8):
+        part = (part + sq[..., e]).astype(np.float32)
+    while part.shape[-1] > 1:
+        part = (part[..., 0::2] + part[..., 1::2]).astype(np.float32)
+    ss = part[..., 0]
+    mean = (ss / np.float32(D)).astype(np.float32)
+    inv = (np.float32(1.0) / np.sqrt((mean + np.float32(eps)).astype(np.float32))).astype(np.float32)
+    g = bf16_to_f32(gain_bits)
+    y = ((x * inv[..., None]).astype(np.float32) * g).astype(np.float32)
+    y = bf16_to_f32(f32_to_bf16_bits_rne(y))
+    if cos is None:
+        return f32_to_bf16_bits_rne(y)
+    half = D // 2
+    rows = (np.arange(B)[:, None, None] * table_batch_rows + np.arange(S)[None, :, None] * H + np.arange(H)[None, None, :])
+    c = np.asarray(cos, np.float32)[rows]                          # [B,S,H,half]
+    s = np.asarray(sin, np.float32)[rows]
+    y0, y1 = y[..., 0::2], y[..., 1::2]
+    o0 = ((y0 * c).astype(np.float32) - (y1 * s).astype(np.float32)).astype(np.float32)
+    o1 = ((y0 * s).astype(np.float32) + (y1 * c).astype(np.float32)).astype(np.float32)
+    out = np.empty((B, S, H, D), np.float32)
+    out[..., 0::2], out[..., 1::2] = o0, o1
+    return f32_to_bf16_bits_rne(out)

@@ -1,0 +1,100 @@
+"""The two ops in front of the path (RMSNorm over the head dim, interleaved RoPE) as the CPU
+checker restates them, against the vectors the reference's own smoke tests hold, the closed
+form its large-D test uses, algebraic properties, and an independent numpy restatement."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import np_restatement as R
+from mojodiffusion_amd.workloads import f32_to_bf16_bits, bf16_bits_to_f32
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def kat():
+    with open(os.path.join(HERE, "golden", "ops_smoke_rmsnorm_rope_kat.json")) as f:
+        return json.load(f)
+
+
+def test_rms_norm_reference_vector(oracle, kat):
+    """serenitymojo/ops_smoke.mojo:78-96."""
+    x = np.array(kat["rms_x"], np.float32).reshape(3, 6)
+    g = np.array(kat["rms_g"], np.float32)
+    got = oracle.rms_norm_f32(x, g, kat["rms_eps"])
+    np.testing.assert_allclose(got, np.array(kat["rms_y"]).reshape(3, 6), rtol=0, atol=2e-7)
+
+
+def test_rope_reference_vector(oracle, kat):
+    """serenitymojo/ops_smoke2.mojo:92-120."""
+    x = np.array(kat["rope_x"], np.float32).reshape(3, 8)
+    c = np.array(kat["rope_cos"], np.float32).reshape(3, 4)
+    s = np.array(kat["rope_sin"], np.float32).reshape(3, 4)
+    got = oracle.rope_interleaved_f32(x, c, s)
+    np.testing.assert_allclose(got, np.array(kat["rope_y_interleaved"]).reshape(3, 8), rtol=0, atol=3e-7)
+
+
+@pytest.mark.parametrize("D", [64, 128, 2560, 3072, 4096])
+def test_rms_norm_closed_form_at_scale(oracle, D):
+    """The sequence and float64 closed form of serenitymojo/ops_smoke2.mojo:372-403 (there for
+    D = 2560, 3072, 4096; the head dims 64 and 128 of this path added)."""
+    i = np.arange(D)
+    x = (np.float32(0.5) + (i % 17).astype(np.float32) * np.float32(0.1)).astype(np.float32)
+    x[1::2] = -x[1::2]
+    g = (np.float32(0.25) + (i % 5).astype(np.float32) * np.float32(0.1)).astype(np.float32)
+    ss = (x.astype(np.float64) ** 2).sum()
+    ref = x.astype(np.float64) / np.sqrt(ss / D + 1e-6) * g.astype(np.float64)
+    got = oracle.rms_norm_f32(x[None], g, 1e-6)[0]
+    np.testing.assert_allclose(got, ref, rtol=3e-7, atol=0)
+
+
+def test_properties(oracle):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((7, 128)).astype(np.float32)
+    ones = np.ones(128, np.float32)
+    y = oracle.rms_norm_f32(x, ones, 0.0)
+    np.testing.assert_allclose((y.astype(np.float64) ** 2).mean(-1), 1.0, rtol=1e-6)     # unit RMS
+    np.testing.assert_array_equal(oracle.rms_norm_f32(2.0 * x, ones, 0.0), y)             # scale-free (power of two: exact)
+    # a rotation keeps the length of every pair; angle 0 is the identity; angle pi/2 swaps with a sign
+    th = rng.uniform(-3, 3, (7, 64)).astype(np.float32)
+    r = oracle.rope_interleaved_f32(x, np.cos(th), np.sin(th))
+    np.testing.assert_allclose(r[:, 0::2] ** 2 + r[:, 1::2] ** 2, x[:, 0::2] ** 2 + x[:, 1::2] ** 2, rtol=2e-6)
+    np.testing.assert_array_equal(oracle.rope_interleaved_f32(x, np.ones((7, 64)), np.zeros((7, 64))), x)
+    q = oracle.rope_interleaved_f32(x, np.zeros((7, 64)), np.ones((7, 64)))
+    np.testing.assert_array_equal(q[:, 0::2], -x[:, 1::2])
+    np.testing.assert_array_equal(q[:, 1::2], x[:, 0::2])
+    # relative-position property: <rope(q, m), rope(k, n)> depends on m - n only
+    qv, kv = x[0:1], x[1:2]
+    base = 1.0 / (10000.0 ** (np.arange(64) / 64.0))
+    def rot(v, pos):
+        a = (pos * base)[None].astype(np.float32)
+        return oracle.rope_interleaved_f32(v, np.cos(a), np.sin(a)).astype(np.float64)
+    d1 = (rot(qv, 5) * rot(kv, 2)).sum()
+    d2 = (rot(qv, 13) * rot(kv, 10)).sum()
+    assert abs(d1 - d2) < 1e-4 * max(1.0, abs(d1))
+
+
+@pytest.mark.parametrize("D,with_rope,batch_rows", [(128, True, 0), (64, True, 0), (128, False, 0), (128, True, 3 * 37)])
+def test_bf16_pipeline_matches_numpy_restatement(oracle, D, with_rope, batch_rows):
+    rng = np.random.default_rng(11 + D)
+    B, S, H = 2, 37, 3
+    x = f32_to_bf16_bits(rng.standard_normal((B, S, H, D)).astype(np.float32) * 3.0)
+    x[0, 3, 1] = 0                                               # an all-zero row: inv = 1/sqrt(eps), output 0
+    gain = f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(D)).astype(np.float32))
+    rows = S * H * (B if batch_rows else 1)
+    th = rng.uniform(-3.14, 3.14, (rows, D // 2))
+    cos, sin = (np.cos(th).astype(np.float32), np.sin(th).astype(np.float32)) if with_rope else (None, None)
+    got = oracle.norm_rope_bf16(x, gain, 1e-6, cos, sin, batch_rows)
+    want = R.norm_rope_bf16(x, gain, 1e-6, cos, sin, batch_rows)
+    np.testing.assert_array_equal(got, want)
+    assert not bf16_bits_to_f32(got[0, 3, 1]).any()                 # (signed zeros allowed)
+    # and it is the composition of the two fp32 ops with a bf16 store in between, to bf16 precision
+    xf = bf16_bits_to_f32(x).reshape(-1, D)
+    y = oracle.rms_norm_f32(xf, bf16_bits_to_f32(gain), 1e-6)
+    if with_rope:
+        idx = (np.arange(B)[:, None, None] * batch_rows + np.arange(S)[None, :, None] * H + np.arange(H)[None, None, :]).reshape(-1)
+        y = oracle.rope_interleaved_f32(y, cos[idx], sin[idx])
+    # (a rotated pair can cancel, so the bf16 steps of the inputs show as absolute error)
+    np.testing.assert_allclose(bf16_bits_to_f32(got).reshape(-1, D), y, rtol=2.0 ** -6, atol=3e-2)
