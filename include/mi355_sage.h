@@ -84,6 +84,27 @@ int mi355_sage_sdpa_bf16_ex(
     int variant, int blkq, int blkk, int smooth_k,
     void* workspace, size_t workspace_bytes);
 
+/* mi355_sage_sdpa_bf16_ex on the PRE-norm projections: Q and K rows are RMS-normalised with
+ * their gains and rotated (interleaved RoPE) on the way into the quantizers, i.e. the three
+ * calls rms_norm / rope_interleaved / sdpa of serenitymojo/models/klein/single_block.mojo:977-982
+ * in one, with the arithmetic of serenitymojo/ops/norm.mojo:81-114 and ops/rope.mojo:104-122
+ * (bf16 stores between the steps included).  Arguments of the fused ops as in
+ * mi355_sage_quant_qk_norm_rope_bf16.  V is used as it is. */
+int mi355_sage_sdpa_bf16_norm_rope(
+    const void* Q, const void* K, const void* V, void* O,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems,
+    int causal,
+    void* stream,
+    int variant, int blkq, int blkk, int smooth_k,
+    const void* q_gain, const void* k_gain, float eps,
+    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+    void* workspace, size_t workspace_bytes);
+
 /* Replaces flame_cudnn_sdpa_bf16_train_fwd (cudnn_sdpa.cpp:470-484), the symbol
  * every Mojo caller binds (serenitymojo/ops/attention_flash.mojo:182-192): same
  * parameter list plus the three trailing arguments.  Stats receives the fp32
@@ -141,6 +162,27 @@ int mi355_sage_quant_qk_bf16(
     int B, int H, int N_q, int N_kv, int D, float scale,
     const int64_t* q_strides, const int64_t* k_strides,
     int64_t q_offset_elems, int64_t k_offset_elems,
+    int blkq, int blkk, int smooth_k,
+    void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+    void* scratch, size_t scratch_bytes, void* stream);
+
+/* The same with the two ops the callers run in front of attention fused in: every Q and K row
+ * goes through RMSNorm over D with a bf16 gain (serenitymojo/ops/norm.mojo:81-114,
+ * out = bf16(x * 1/sqrt(mean(x^2)+eps) * g)) and, when tables are given, interleaved RoPE with
+ * fp32 tables (serenitymojo/ops/rope.mojo:104-122, pairs (2i, 2i+1), result bf16) before it is
+ * quantized — the call order of serenitymojo/models/klein/single_block.mojo:977-981, without
+ * the two bf16 round trips through memory.  q_gain, k_gain: bf16 [D].  rope_cos / rope_sin:
+ * fp32 [rows, D/2], row = n*H + h (serenitymojo/sampling/klein_sampler.mojo:305-307), batch b
+ * starting at row b*rope_batch_rows (0 = one table for all batches); both NULL = norm only.
+ * Q rows and K rows use the same table (self-attention positions).  Gains and tables must be
+ * 16-byte aligned. */
+int mi355_sage_quant_qk_norm_rope_bf16(
+    const void* Q, const void* K,
+    int B, int H, int N_q, int N_kv, int D, float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    const void* q_gain, const void* k_gain, float eps,
+    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
     int blkq, int blkk, int smooth_k,
     void* q8, void* qscale, void* k8, void* kscale, void* kmean,
     void* scratch, size_t scratch_bytes, void* stream);

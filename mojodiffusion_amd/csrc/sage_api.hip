@@ -111,15 +111,38 @@ int internal_workspace(size_t need, void** out) {
     return 0;
 }
 
+// The optional ops in front of the quantizers (RMSNorm + interleaved RoPE of Q and of K).
+struct Pre {
+    PreOp q{}, k{};
+};
+
+// q_gain / k_gain null together = nothing to do.  Tables are optional on top of the gains.
+int make_pre(const void* q_gain, const void* k_gain, float eps, const void* rope_cos, const void* rope_sin,
+             int64_t rope_batch_rows, Pre* out) {
+    *out = Pre{};
+    if (!q_gain && !k_gain && !rope_cos && !rope_sin) return 0;
+    if (!q_gain || !k_gain) { SAGE_LOG("RMSNorm gains must be given for both Q and K"); return MI355_SAGE_EINVAL; }
+    if ((rope_cos == nullptr) != (rope_sin == nullptr)) return MI355_SAGE_EINVAL;
+    if (!(eps >= 0.0f) || rope_batch_rows < 0) return MI355_SAGE_EINVAL;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(q_gain) | reinterpret_cast<uintptr_t>(k_gain) |
+                           reinterpret_cast<uintptr_t>(rope_cos) | reinterpret_cast<uintptr_t>(rope_sin);
+    if (bits & 15) { SAGE_LOG("gains and RoPE tables must be 16-byte aligned"); return MI355_SAGE_EUNSUPPORTED; }
+    out->q = PreOp{static_cast<const uint16_t*>(q_gain), eps, static_cast<const float*>(rope_cos),
+                   static_cast<const float*>(rope_sin), rope_batch_rows};
+    out->k = out->q;
+    out->k.gain = static_cast<const uint16_t*>(k_gain);
+    return 0;
+}
+
 int quant_qk(const View& q, const View& k, int B, int H, int Nq, int Nkv, int D, float scale,
              int blkq, int blkk, int smooth_k, int8_t* q8, float* qscale, int8_t* k8, float* kscale,
-             float* kmean, double* partial, float* qshift, hipStream_t st) {
+             float* kmean, double* partial, float* qshift, const Pre& pre, hipStream_t st) {
     const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
-    if (smooth_k) SAGE_HIP(launch_kmean(k, B, H, Nkv, D, partial, kmean, st));
+    if (smooth_k) SAGE_HIP(launch_kmean(k, B, H, Nkv, D, partial, kmean, pre.k, st));
     SAGE_HIP(launch_quant_i8(q, B, H, Nq, D, pad_to(Nq, kTileQ), blkq, false, cmul, kmean, q8, qscale,
-                             smooth_k ? qshift : nullptr, st));
+                             smooth_k ? qshift : nullptr, pre.q, st));
     SAGE_HIP(launch_quant_i8(k, B, H, Nkv, D, pad_to(Nkv, kPadKV), blkk, true, 0.0f,
-                             smooth_k ? kmean : nullptr, k8, kscale, nullptr, st));
+                             smooth_k ? kmean : nullptr, k8, kscale, nullptr, pre.k, st));
     return 0;
 }
 
@@ -128,7 +151,8 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
               const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
               int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t stats_off,
               int causal, int real_N_kv, void* stream,
-              int variant, int blkq, int blkk, int smooth_k, void* workspace, size_t workspace_bytes) {
+              int variant, int blkq, int blkk, int smooth_k, void* workspace, size_t workspace_bytes,
+              const Pre& pre = Pre{}) {
     // argument checks in the order of serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393
     if (!Q || !K || !V || !O) return MI355_SAGE_EINVAL;
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
@@ -176,13 +200,14 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         // two launches: {Q quantize, V repack, K-mean group sums} then {K mean + K quantize}
         const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
         SAGE_HIP(launch_prep_fused(q, k, v, B, H, N_q, kv, D, pad_to(N_q, kTileQ), nkp, cmul, blkq, smooth_k != 0,
-                                   q8, qscale, static_cast<uint16_t*>(vq), partial, st));
-        SAGE_HIP(launch_kquant_fused(k, B, H, kv, D, nkp, blkk, smooth_k ? partial : nullptr, kmean, k8, kscale, st));
+                                   q8, qscale, static_cast<uint16_t*>(vq), partial, pre.q, pre.k, st));
+        SAGE_HIP(launch_kquant_fused(k, B, H, kv, D, nkp, blkk, smooth_k ? partial : nullptr, kmean, k8, kscale,
+                                     pre.k, st));
     } else {
         // Stats needs <q, kmean> per row, i.e. the mean before the Q quantizer; the e4m3 V path
         // has its own three launches
         if ((rc = quant_qk(q, k, B, H, N_q, kv, D, scale, blkq, blkk, smooth_k, q8, qscale, k8, kscale,
-                           kmean, partial, qshift, st)))
+                           kmean, partial, qshift, pre, st)))
             return rc;
         if (variant == MI355_SAGE_PV_FP16)
             SAGE_HIP(launch_quant_v_f16(v, B, H, kv, D, nkp, static_cast<uint16_t*>(vq), st));
@@ -285,7 +310,51 @@ int mi355_sage_quant_qk_bf16(const void* Q, const void* K, int B, int H, int N_q
     return quant_qk(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), B, H, N_q, N_kv, D,
                     scale, blkq, blkk, smooth_k, static_cast<int8_t*>(q8), static_cast<float*>(qscale),
                     static_cast<int8_t*>(k8), static_cast<float*>(kscale), static_cast<float*>(kmean),
-                    static_cast<double*>(scratch), nullptr, static_cast<hipStream_t>(stream));
+                    static_cast<double*>(scratch), nullptr, Pre{}, static_cast<hipStream_t>(stream));
+}
+
+int mi355_sage_quant_qk_norm_rope_bf16(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
+                                       float scale, const int64_t* q_strides, const int64_t* k_strides,
+                                       int64_t q_off, int64_t k_off,
+                                       const void* q_gain, const void* k_gain, float eps,
+                                       const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+                                       int blkq, int blkk, int smooth_k,
+                                       void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+                                       void* scratch, size_t scratch_bytes, void* stream) {
+    if (!Q || !K || !q8 || !qscale || !k8 || !kscale) return MI355_SAGE_EINVAL;
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
+    if (!q_strides || !k_strides) return MI355_SAGE_EINVAL;
+    if (smooth_k && (!kmean || !scratch)) return MI355_SAGE_EINVAL;
+    if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk)) return MI355_SAGE_EUNSUPPORTED;
+    if (smooth_k && scratch_bytes < mi355_sage_quant_scratch_bytes(B, H, N_kv, D)) return MI355_SAGE_EWORKSPACE;
+    int rc;
+    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off))) return rc;
+    Pre pre;
+    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
+    if (!pre.q.gain) return MI355_SAGE_EINVAL;
+    return quant_qk(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), B, H, N_q, N_kv, D,
+                    scale, blkq, blkk, smooth_k, static_cast<int8_t*>(q8), static_cast<float*>(qscale),
+                    static_cast<int8_t*>(k8), static_cast<float*>(kscale), static_cast<float*>(kmean),
+                    static_cast<double*>(scratch), nullptr, pre, static_cast<hipStream_t>(stream));
+}
+
+int mi355_sage_sdpa_bf16_norm_rope(const void* Q, const void* K, const void* V, void* O,
+                                   int B, int H, int N_q, int N_kv, int D, float scale,
+                                   const int64_t* q_strides, const int64_t* k_strides,
+                                   const int64_t* v_strides, const int64_t* o_strides,
+                                   int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
+                                   int causal, void* stream,
+                                   int variant, int blkq, int blkk, int smooth_k,
+                                   const void* q_gain, const void* k_gain, float eps,
+                                   const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+                                   void* workspace, size_t workspace_bytes) {
+    Pre pre;
+    int rc;
+    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
+    if (!pre.q.gain) return MI355_SAGE_EINVAL;
+    return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                     o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, blkq, blkk,
+                     smooth_k ? 1 : 0, workspace, workspace_bytes, pre);
 }
 
 int mi355_sage_quant_v_f16(const void* V, int B, int H, int N_kv, int D, const int64_t* v_strides,

@@ -23,26 +23,39 @@ struct View {
     int64_t sb, sh, sn;      // element strides (D stride is 1)
 };
 
+// RMSNorm over D (+ interleaved RoPE) applied to the rows of Q or K as the quantizers load
+// them: what serenitymojo/ops/norm.mojo:81-114 and ops/rope.mojo:104-122 leave in memory as
+// bf16 tensors, computed on the fly.  gain == null: rows are used as they are.
+struct PreOp {
+    const uint16_t* gain;        // bf16 [D]
+    float eps;
+    const float* cos;            // fp32 [rows, D/2], row = n*H + h (+ b*batch_rows); null = no rotation
+    const float* sin;
+    int64_t batch_rows;          // 0: all batches share the table
+};
+
 // ---- quantize kernels (sage_quant.hip) -------------------------------------
 // Q (is_k = false): x = f32(q)*cmul.  K (is_k = true): x = f32(k) - mean (mean may be null).
 // rowdot (Q only, may be null): [B,H,n_pad] <pre-scaled q row, mean>, needed for the
 // log-sum-exp output when K is smoothed.
 hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad,
                            int blk, bool is_k, float cmul, const float* mean,
-                           int8_t* codes, float* scales, float* rowdot, hipStream_t st);
+                           int8_t* codes, float* scales, float* rowdot, const PreOp& pre, hipStream_t st);
 
 // K mean: group partials (double, [B,H,ngroups,D]) then the final mean.
 hipError_t launch_kmean(const View& k, int B, int H, int N, int D,
-                        double* group_partials, float* kmean, hipStream_t st);
+                        double* group_partials, float* kmean, const PreOp& pre, hipStream_t st);
 
 // One-shot path: Q quantizer + V fp16 repack + K-mean group sums in one launch, then the
 // K quantizer that finishes the mean from the group partials itself (partial == null: no
 // smoothing).  Same arithmetic, bit for bit, as the separate launches above.
 hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B, int H, int Nq, int Nkv, int D,
                              int64_t nq_pad, int64_t nkv_pad, float cmul, int blkq, bool smooth_k,
-                             int8_t* q8, float* qscale, uint16_t* v16, double* partial, hipStream_t st);
+                             int8_t* q8, float* qscale, uint16_t* v16, double* partial,
+                             const PreOp& pre_q, const PreOp& pre_k, hipStream_t st);
 hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
-                               const double* partial, float* kmean, int8_t* codes, float* scales, hipStream_t st);
+                               const double* partial, float* kmean, int8_t* codes, float* scales,
+                               const PreOp& pre, hipStream_t st);
 
 hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t n_pad,
                               uint16_t* v16, hipStream_t st);

@@ -31,6 +31,68 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+__device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x0040u;
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ float round_to_bf16(float f) { return __uint_as_float(f32_to_bf16_rne(f) << 16); }
+
+// RMSNorm (+ RoPE) of one row, spread over the D/8 consecutive lanes that hold its 16-byte
+// chunks: x[0..7] are channels col..col+7.  Every lane of the group must call this (it
+// exchanges partial sums); `valid` false = a padding row, which stays zero.
+// Arithmetic, step for step (all fp32, no fused multiply-add):
+//   squares added left to right inside the chunk, chunk sums combined pairwise, neighbours
+//   first; inv = 1/sqrt(sum/D + eps); y = bf16((x*inv)*gain); rotation of (y[2i], y[2i+1]) by
+//   the table angle with both products rounded before the subtract / add; result bf16.
+template <int D>
+__device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, int row, int col, bool valid, float* x) {
+    constexpr int CPR = D / 8;
+    float a = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float sq = x[e] * x[e];
+        a = a + sq;
+    }
+#pragma unroll
+    for (int off = 1; off < CPR; off <<= 1) a = a + __shfl_xor(a, off, 64);
+    const float mean = a / (float)D;
+    const float inv = 1.0f / sqrtf(mean + p.eps);
+    const u32x4 gw = *reinterpret_cast<const u32x4*>(p.gain + col);
+    float g[8];
+    unpack8(gw, g);
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float t = x[e] * inv;
+        y[e] = round_to_bf16(t * g[e]);
+    }
+    if (p.cos != nullptr) {
+        float4 c4 = {1.f, 1.f, 1.f, 1.f}, s4 = {0.f, 0.f, 0.f, 0.f};
+        if (valid) {
+            const int64_t trow = (int64_t)b * p.batch_rows + (int64_t)row * H + h;
+            c4 = *reinterpret_cast<const float4*>(p.cos + trow * (D / 2) + col / 2);
+            s4 = *reinterpret_cast<const float4*>(p.sin + trow * (D / 2) + col / 2);
+        }
+        const float cv[4] = {c4.x, c4.y, c4.z, c4.w}, sv[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float y0 = y[2 * i], y1 = y[2 * i + 1];
+            const float p00 = y0 * cv[i], p11 = y1 * sv[i], p01 = y0 * sv[i], p10 = y1 * cv[i];
+            x[2 * i] = round_to_bf16(p00 - p11);
+            x[2 * i + 1] = round_to_bf16(p01 + p10);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = y[e];
+    }
+    if (!valid) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = 0.0f;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Per-block INT8 quantization.  One workgroup (256 threads) per (block, h, b);
 // the block's BLK x D tile lives in registers between the absmax pass and the
@@ -60,7 +122,7 @@ __device__ __forceinline__ void quant_i8_block(
     int t, int h, int b, const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, float cmul, const float* mean,
     int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, float* red,
-    Hook hook = Hook()) {
+    const PreOp& pre, Hook hook = Hook()) {
     constexpr int CPR = D / 8;                 // 16-byte chunks per row
     constexpr int NCH = BLK * CPR / 256;       // chunks per thread
     static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
@@ -86,6 +148,7 @@ __device__ __forceinline__ void quant_i8_block(
         const int c = i * 256 + tid;
         const int row = r0 + c / CPR, col = (c % CPR) * 8;
         unpack8(raw[i], v[i]);
+        if (pre.gain != nullptr) pre_apply<D>(pre, b, h, H, row, col, row < N, v[i]);
         if (IS_K) {
             if (mean != nullptr) {
                 const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
@@ -147,21 +210,21 @@ template <int D, int BLK, bool IS_K>
 __global__ __launch_bounds__(256) void quant_i8_kernel(
     const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
-    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot) {
+    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, PreOp pre) {
     __shared__ float red[4];
     const int h = blockIdx.y, b = blockIdx.z;
     quant_i8_block<D, BLK, IS_K>(blockIdx.x, h, b, x, sb, sh, sn, N, H, n_pad, cmul,
-                                 mean ? mean + ((int64_t)b * H + h) * D : nullptr, codes, scales, rowdot, red);
+                                 mean ? mean + ((int64_t)b * H + h) * D : nullptr, codes, scales, rowdot, red, pre);
 }
 
 template <int D, bool IS_K>
 static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t n_pad, int blk,
                                     float cmul, const float* mean, int8_t* codes, float* scales,
-                                    float* rowdot, hipStream_t st) {
+                                    float* rowdot, const PreOp& pre, hipStream_t st) {
     dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
 #define SAGE_LAUNCH_Q(BLK)                                                                    \
     hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K>), grid, block, 0, st, x.p, x.sb, x.sh,   \
-                       x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot)
+                       x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot, pre)
     switch (blk) {
         case 32: SAGE_LAUNCH_Q(32); break;
         case 64: SAGE_LAUNCH_Q(64); break;
@@ -174,14 +237,14 @@ static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t 
 
 hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad, int blk,
                            bool is_k, float cmul, const float* mean, int8_t* codes,
-                           float* scales, float* rowdot, hipStream_t st) {
+                           float* scales, float* rowdot, const PreOp& pre, hipStream_t st) {
     if (n_pad % blk != 0) return hipErrorInvalidValue;
     if (D == 128)
-        return is_k ? launch_quant_i8_d<128, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st)
-                    : launch_quant_i8_d<128, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st);
+        return is_k ? launch_quant_i8_d<128, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st)
+                    : launch_quant_i8_d<128, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st);
     if (D == 64)
-        return is_k ? launch_quant_i8_d<64, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st)
-                    : launch_quant_i8_d<64, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, st);
+        return is_k ? launch_quant_i8_d<64, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st)
+                    : launch_quant_i8_d<64, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st);
     return hipErrorInvalidValue;
 }
 
@@ -197,7 +260,7 @@ hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_
 template <int D>
 __device__ __forceinline__ void kmean_group_body(
     int g, int h, int b, int tid, const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int ngroups, double* __restrict__ partial, double (*leafsum)[D + 2]) {
+    int N, int H, int ngroups, double* __restrict__ partial, double (*leafsum)[D + 2], const PreOp& pre) {
     constexpr int CPR = D / 8;
     const int leaf = tid / CPR, col = (tid % CPR) * 8;
     const uint16_t* src = k + b * sb + h * sh + col;
@@ -214,6 +277,7 @@ __device__ __forceinline__ void kmean_group_body(
     for (int i = 0; i < kLeaf; i++) {
         float x[8];
         unpack8(w[i], x);
+        if (pre.gain != nullptr) pre_apply<D>(pre, b, h, H, s0 + i, col, g >= 0 && s0 + i < N, x);
         // rows past N contribute +0.0, which leaves a double sum unchanged
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += (double)x[e];
@@ -233,9 +297,9 @@ __device__ __forceinline__ void kmean_group_body(
 template <int D>
 __global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int ngroups, double* __restrict__ partial) {
+    int N, int H, int ngroups, double* __restrict__ partial, PreOp pre) {
     __shared__ double leafsum[16][D + 2];
-    kmean_group_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x, k, sb, sh, sn, N, H, ngroups, partial, leafsum);
+    kmean_group_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x, k, sb, sh, sn, N, H, ngroups, partial, leafsum, pre);
 }
 
 __global__ __launch_bounds__(256) void kmean_final_kernel(
@@ -259,15 +323,15 @@ __global__ __launch_bounds__(256) void kmean_final_kernel(
 }
 
 hipError_t launch_kmean(const View& k, int B, int H, int N, int D, double* partial,
-                        float* kmean, hipStream_t st) {
+                        float* kmean, const PreOp& pre, hipStream_t st) {
     const int ngroups = (N + kGroup - 1) / kGroup;
     dim3 grid((unsigned)ngroups, (unsigned)H, (unsigned)B);
     if (D == 128)
         hipLaunchKernelGGL((kmean_group_kernel<128>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
-                           N, H, ngroups, partial);
+                           N, H, ngroups, partial, pre);
     else if (D == 64)
         hipLaunchKernelGGL((kmean_group_kernel<64>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
-                           N, H, ngroups, partial);
+                           N, H, ngroups, partial, pre);
     else
         return hipErrorInvalidValue;
     hipError_t e = hipGetLastError();
@@ -383,6 +447,7 @@ struct PrepArgs {
     float cmul;
     int8_t* q8; float* qscale; uint16_t* v16; double* partial;
     int nq_blk, nv_tile, nk_wg, ngroups;      // per (b,h): Q blocks, V tiles, K-mean workgroups; K groups
+    PreOp pre_q, pre_k;
 };
 
 template <int D, int BLKQ>
@@ -399,7 +464,7 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
     const int b = bh / a.H, h = bh % a.H;
     if (r < a.nq_blk) {
         quant_i8_block<D, BLKQ, false>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, a.cmul, nullptr,
-                                       a.q8, a.qscale, nullptr, sm.red);
+                                       a.q8, a.qscale, nullptr, sm.red, a.pre_q);
     } else if (r < a.nq_blk + a.nv_tile) {
         quant_v_f16_body<D>(r - a.nq_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.v16, sm.tile);
     } else {
@@ -408,7 +473,7 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
         // groups past the end still take part in the barrier inside; they read nothing and
         // their sum is not stored
         kmean_group_body<D>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh, a.k.sn,
-                            a.Nkv, a.H, a.ngroups, a.partial, sm.leafsum[sub]);
+                            a.Nkv, a.H, a.ngroups, a.partial, sm.leafsum[sub], a.pre_k);
     }
 }
 
@@ -447,7 +512,7 @@ template <int D, int BLK>
 __global__ __launch_bounds__(256) void kquant_fused_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, const double* __restrict__ partial, int ngroups,
-    float* __restrict__ kmean, int8_t* __restrict__ codes, float* __restrict__ scales) {
+    float* __restrict__ kmean, int8_t* __restrict__ codes, float* __restrict__ scales, PreOp pre) {
     __shared__ float mean_s[D];
     __shared__ float red[4];
     const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -456,7 +521,7 @@ __global__ __launch_bounds__(256) void kquant_fused_kernel(
     MeanFromPartials<D> hook{smooth ? partial + bh * ngroups * D : nullptr, ngroups, N, mean_s,
                              (smooth && t == 0) ? kmean + bh * D : nullptr};
     quant_i8_block<D, BLK, true>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
-                                 codes, scales, nullptr, red, hook);
+                                 codes, scales, nullptr, red, pre, hook);
 }
 
 template <int D>
@@ -473,8 +538,10 @@ static hipError_t launch_prep_d(const PrepArgs& a, int B, int blkq, hipStream_t 
 
 hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B, int H, int Nq, int Nkv, int D,
                              int64_t nq_pad, int64_t nkv_pad, float cmul, int blkq, bool smooth_k,
-                             int8_t* q8, float* qscale, uint16_t* v16, double* partial, hipStream_t st) {
+                             int8_t* q8, float* qscale, uint16_t* v16, double* partial,
+                             const PreOp& pre_q, const PreOp& pre_k, hipStream_t st) {
     PrepArgs a{};
+    a.pre_q = pre_q; a.pre_k = pre_k;
     a.q = q; a.k = k; a.v = v; a.H = H; a.Nq = Nq; a.Nkv = Nkv; a.nq_pad = nq_pad; a.nkv_pad = nkv_pad;
     a.cmul = cmul; a.q8 = q8; a.qscale = qscale; a.v16 = v16; a.partial = partial;
     a.nq_blk = (int)(nq_pad / blkq);
@@ -488,12 +555,13 @@ hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B,
 }
 
 hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
-                               const double* partial, float* kmean, int8_t* codes, float* scales, hipStream_t st) {
+                               const double* partial, float* kmean, int8_t* codes, float* scales,
+                               const PreOp& pre, hipStream_t st) {
     const int ngroups = (N + kGroup - 1) / kGroup;
     dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
 #define SAGE_LAUNCH_KQ(DD, BLK)                                                                          \
     hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK>), grid, block, 0, st, k.p, k.sb, k.sh, k.sn, N, H, \
-                       n_pad, partial, ngroups, kmean, codes, scales)
+                       n_pad, partial, ngroups, kmean, codes, scales, pre)
     if (D == 128) {
         switch (blk) {
             case 32: SAGE_LAUNCH_KQ(128, 32); break;

@@ -1,0 +1,133 @@
+"""GPU parity of the quantizers with RMSNorm + interleaved RoPE fused in front: the INT8 codes,
+scales and the K mean must be bit-identical with what the CPU checker gets by running its
+norm/rope restatement first and its quantizers on the result; the one-shot call must agree with
+the unfused pipeline."""
+import numpy as np
+import pytest
+
+from mojodiffusion_amd import _lib
+from mojodiffusion_amd.workloads import WORKLOADS, make_inputs, f32_to_bf16_bits, bf16_bits_to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def _tables(rng, rows, D):
+    """RoPE tables of the sampler's shape: one angle per (row, pair)."""
+    th = rng.uniform(-np.pi, np.pi, (rows, D // 2))
+    return np.cos(th).astype(np.float32), np.sin(th).astype(np.float32)
+
+
+def _gains(rng, D):
+    return (f32_to_bf16_bits((1.0 + 0.3 * rng.standard_normal(D)).astype(np.float32)),
+            f32_to_bf16_bits((0.7 + 0.3 * rng.standard_normal(D)).astype(np.float32)))
+
+
+def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows):
+    import torch
+    import gpu_harness as H
+    L = _lib.lib()
+    B, S, Hh, D = q.shape
+    qd, kd = H.dev_bf16(q), H.dev_bf16(k)
+    gqd, gkd = H.dev_bf16(gq), H.dev_bf16(gk)
+    cd = torch.from_numpy(cos).cuda() if cos is not None else None
+    sd = torch.from_numpy(sin).cuda() if sin is not None else None
+    nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
+    q8 = torch.full((B, Hh, nqp, D), 77, dtype=torch.int8, device="cuda")
+    k8 = torch.full((B, Hh, nkp, D), 77, dtype=torch.int8, device="cuda")
+    qs = torch.full((B, Hh, nqp // blkq), -1.0, dtype=torch.float32, device="cuda")
+    ks = torch.full((B, Hh, nkp // blkk), -1.0, dtype=torch.float32, device="cuda")
+    km = torch.full((B, Hh, D), -1.0, dtype=torch.float32, device="cuda")
+    scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, Hh, S, D), 8), dtype=torch.uint8, device="cuda")
+    st = _lib.strides_bhnd(S, Hh, D)
+    rc = L.mi355_sage_quant_qk_norm_rope_bf16(
+        qd.data_ptr(), kd.data_ptr(), B, Hh, S, S, D, scale, st, st, 0, 0,
+        gqd.data_ptr(), gkd.data_ptr(), eps, cd.data_ptr() if cd is not None else None,
+        sd.data_ptr() if sd is not None else None, batch_rows, blkq, blkk, int(smooth),
+        q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr() if smooth else None,
+        scr.data_ptr(), scr.numel(), H.stream())
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    return q8.cpu().numpy(), qs.cpu().numpy(), k8.cpu().numpy(), ks.cpu().numpy(), km.cpu().numpy()
+
+
+@pytest.mark.parametrize("D,S,blkq,blkk,smooth,rope,per_batch", [
+    (128, 300, 128, 64, True, True, False), (128, 1100, 128, 64, True, True, True),
+    (64, 200, 64, 64, True, True, False), (128, 77, 32, 32, False, True, False),
+    (128, 513, 128, 64, True, False, False), (64, 1, 32, 32, True, True, False)])
+def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_batch):
+    rng = np.random.default_rng(100 + S)
+    B, Hh = 2, 3
+    q = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32) * 2.0)
+    k = f32_to_bf16_bits((rng.standard_normal((B, S, Hh, D)) + 1.5 * rng.standard_normal((B, 1, Hh, D))).astype(np.float32))
+    if S > 5:
+        q[1, 3, 0] = 0                                         # an all-zero row
+    gq, gk = _gains(rng, D)
+    cos, sin = _tables(rng, S * Hh * (B if per_batch else 1), D) if rope else (None, None)
+    batch_rows = S * Hh if per_batch else 0
+    eps, scale = 1e-6, 1.0 / np.sqrt(D)
+    got = _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows)
+    qn = oracle.norm_rope_bf16(q, gq, eps, cos, sin, batch_rows)
+    kn = oracle.norm_rope_bf16(k, gk, eps, cos, sin, batch_rows)
+    q8, qs = oracle.quant_q(qn, scale, blkq, int(_lib.lib().mi355_sage_pad_q(1)))
+    mu = oracle.kmean(kn) if smooth else None
+    k8, ks = oracle.quant_k(kn, mu, blkk, 128)
+    if smooth:
+        np.testing.assert_array_equal(got[4].view(np.uint32), mu.view(np.uint32))
+    np.testing.assert_array_equal(got[1][:, :, :qs.shape[2]].view(np.uint32), qs.view(np.uint32))
+    np.testing.assert_array_equal(got[3][:, :, :ks.shape[2]].view(np.uint32), ks.view(np.uint32))
+    np.testing.assert_array_equal(got[0], q8)
+    np.testing.assert_array_equal(got[2], k8)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_one_shot_equals_unfused_pipeline(oracle, variant):
+    """mi355_sage_sdpa_bf16_norm_rope on the projections == the plain one-shot call on
+    norm/rope'd tensors (the CPU checker's, which the test above proves equal to the fused
+    kernels' view bit for bit): same quantized tensors, hence the same output bits."""
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    rng = np.random.default_rng(9)
+    w = WORKLOADS[2].scaled(B=1, H=3, S=700)
+    q, k, v = make_inputs(w)
+    gq, gk = _gains(rng, w.D)
+    cos, sin = _tables(rng, w.S * w.H, w.D)
+    qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
+    got = A.qk_norm_rope_sdpa_nomask(qd, kd, vd, H.dev_bf16(gq), H.dev_bf16(gk), 1e-6,
+                                     torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), w.scale, variant)
+    torch.cuda.synchronize()
+    qn = oracle.norm_rope_bf16(q, gq, 1e-6, cos, sin, 0)
+    kn = oracle.norm_rope_bf16(k, gk, 1e-6, cos, sin, 0)
+    want = A.sdpa_nomask(H.dev_bf16(qn), H.dev_bf16(kn), vd, w.scale, variant)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(H.to_bits(got), H.to_bits(want))
+    # and against an fp32 attention on the fp32 norm/rope
+    qf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(q).reshape(-1, w.D), bf16_bits_to_f32(gq), 1e-6), cos, sin)
+    kf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(k).reshape(-1, w.D), bf16_bits_to_f32(gk), 1e-6), cos, sin)
+    ref = oracle.sdpa_f32(qf.reshape(q.shape), kf.reshape(k.shape), bf16_bits_to_f32(v), w.scale)
+    cos_sim, mx = H.cos_maxabs(got.float().cpu().numpy(), ref)
+    assert cos_sim >= 0.999, (cos_sim, mx)
+
+
+def test_argument_errors():
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    x = torch.zeros((1, 64, 2, 128), dtype=torch.bfloat16, device="cuda")
+    g = torch.ones(128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(A.Error):
+        A.qk_norm_rope_sdpa_nomask(x, x, x, g[:64], g, 1e-6, None, None, 0.1)
+    with pytest.raises(A.Error):
+        A.qk_norm_rope_sdpa_nomask(x, x, x, g, g, 1e-6, torch.zeros((5, 64), device="cuda"), torch.zeros((5, 64), device="cuda"), 0.1)
+    L = _lib.lib()
+    st = _lib.strides_bhnd(64, 2, 128)
+    o = torch.empty_like(x)
+    # gains missing -> -1; misaligned gain -> -2
+    rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 64, 64, 128, 0.1,
+                                          st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 1,
+                                          None, None, 1e-6, None, None, 0, None, 0)
+    assert rc == -1
+    rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 64, 64, 128, 0.1,
+                                          st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 1,
+                                          g.data_ptr() + 2, g.data_ptr(), 1e-6, None, None, 0, None, 0)
+    assert rc == -2
