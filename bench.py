@@ -51,8 +51,8 @@ def main():
                          "the known-size kernel the HBM traffic counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this hot path is measured on ONE GPU (heads are independent; see DESIGN.md for how "
-              "it would shard); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this hot path is measured on ONE GPU (heads are independent and would shard "
+              "without any exchange); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
