@@ -335,3 +335,49 @@ def test_full_size_properties(wid):
     o2 = _one_shot_dev(q, k2, v, w)
     cos = torch.nn.functional.cosine_similarity(o.float().flatten(), o2.float().flatten(), dim=0).item()
     assert cos >= (0.998 if wid == 3 else 0.999), cos
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_one_shot_call_in_a_hip_graph(variant):
+    """With a caller-held workspace the one-shot call allocates nothing and clears its scratch
+    with kernels, so it can be captured.  The graph is replayed several times with eager work
+    and synchronisations in between and changed inputs; every replay must reproduce the eager
+    result of the same inputs bit for bit."""
+    import torch
+    import gpu_harness as H
+    L = _lib.lib()
+    w = WORKLOADS[2].scaled(B=1, H=2, S=600)
+    q0, k0, v0 = (H.dev_bf16(x) for x in make_inputs(w))
+    q, k, v = q0.clone(), k0.clone(), v0.clone()            # static graph inputs
+    o = torch.empty_like(q)
+    st = _lib.strides_bhnd(w.S, w.H, w.D)
+    nws = L.mi355_sage_workspace_bytes(w.B, w.H, w.S, w.S, w.D, variant)
+    ws = torch.empty(nws, dtype=torch.uint8, device="cuda")
+
+    def call(out):
+        rc = L.mi355_sage_sdpa_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), w.B, w.H, w.S, w.S, w.D,
+                                    w.scale, st, st, st, st, 0, 0, 0, 0, 0, torch.cuda.current_stream().cuda_stream,
+                                    variant, ws.data_ptr(), nws)
+        assert rc == 0, rc
+
+    call(o)                                                  # warm-up outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        call(o)
+    for rep in range(4):
+        # new inputs, some unrelated eager work, then the replay
+        q.copy_(torch.roll(q0, rep, dims=1))
+        k.copy_(k0 * (1.0 + 0.25 * rep))
+        v.copy_(torch.roll(v0, -rep, dims=2))
+        junk = (q.float() @ q.float().transpose(-1, -2)).sum()
+        ws.fill_(0xAB)                                       # the call must not depend on old workspace contents
+        torch.cuda.synchronize()
+        o.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(o)
+        call(eager)
+        torch.cuda.synchronize()
+        assert torch.isfinite(junk)
+        np.testing.assert_array_equal(H.to_bits(o), H.to_bits(eager))
