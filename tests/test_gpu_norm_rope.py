@@ -79,8 +79,8 @@ def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_
     np.testing.assert_array_equal(got[2], k8)
 
 
-@pytest.mark.parametrize("variant", [0, 1])
-def test_one_shot_equals_unfused_pipeline(oracle, variant):
+@pytest.mark.parametrize("variant,wid", [(0, 2), (1, 2), (0, 1)])
+def test_one_shot_equals_unfused_pipeline(oracle, variant, wid):
     """mi355_sage_sdpa_bf16_norm_rope on the projections == the plain one-shot call on
     norm/rope'd tensors (the CPU checker's, which the test above proves equal to the fused
     kernels' view bit for bit): same quantized tensors, hence the same output bits."""
@@ -88,22 +88,30 @@ def test_one_shot_equals_unfused_pipeline(oracle, variant):
     import gpu_harness as H
     from mojodiffusion_amd import attention_sage as A
     rng = np.random.default_rng(9)
-    w = WORKLOADS[2].scaled(B=1, H=3, S=700)
+    w = WORKLOADS[wid].scaled(B=2 if wid == 1 else 1, H=3, S=700)      # wid 1: head dim 64
     q, k, v = make_inputs(w)
     gq, gk = _gains(rng, w.D)
     cos, sin = _tables(rng, w.S * w.H, w.D)
     qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
     got = A.qk_norm_rope_sdpa_nomask(qd, kd, vd, H.dev_bf16(gq), H.dev_bf16(gk), 1e-6,
-                                     torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), w.scale, variant)
+                                     torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), w.scale, variant,
+                                     blkq=w.blkq, blkk=w.blkk)
     torch.cuda.synchronize()
     qn = oracle.norm_rope_bf16(q, gq, 1e-6, cos, sin, 0)
     kn = oracle.norm_rope_bf16(k, gk, 1e-6, cos, sin, 0)
-    want = A.sdpa_nomask(H.dev_bf16(qn), H.dev_bf16(kn), vd, w.scale, variant)
+    want = torch.empty_like(qd)
+    st = _lib.strides_bhnd(w.S, w.H, w.D)
+    qnd, knd = H.dev_bf16(qn), H.dev_bf16(kn)
+    rc = _lib.lib().mi355_sage_sdpa_bf16_ex(qnd.data_ptr(), knd.data_ptr(), vd.data_ptr(), want.data_ptr(),
+                                            w.B, w.H, w.S, w.S, w.D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, H.stream(),
+                                            variant, w.blkq, w.blkk, 1, None, 0)
+    assert rc == 0, rc
     torch.cuda.synchronize()
     np.testing.assert_array_equal(H.to_bits(got), H.to_bits(want))
     # and against an fp32 attention on the fp32 norm/rope
-    qf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(q).reshape(-1, w.D), bf16_bits_to_f32(gq), 1e-6), cos, sin)
-    kf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(k).reshape(-1, w.D), bf16_bits_to_f32(gk), 1e-6), cos, sin)
+    cb, sb = np.tile(cos, (w.B, 1)), np.tile(sin, (w.B, 1))      # the table is shared by the batches
+    qf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(q).reshape(-1, w.D), bf16_bits_to_f32(gq), 1e-6), cb, sb)
+    kf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(k).reshape(-1, w.D), bf16_bits_to_f32(gk), 1e-6), cb, sb)
     ref = oracle.sdpa_f32(qf.reshape(q.shape), kf.reshape(k.shape), bf16_bits_to_f32(v), w.scale)
     cos_sim, mx = H.cos_maxabs(got.float().cpu().numpy(), ref)
     assert cos_sim >= 0.999, (cos_sim, mx)
