@@ -188,6 +188,8 @@ def rope_interleaved_f32(x, cos, sin):
     x = np.ascontiguousarray(x, dtype=np.float32)
     cos = np.ascontiguousarray(cos, dtype=np.float32)
     sin = np.ascontiguousarray(sin, dtype=np.float32)
+    if cos.shape != (x.shape[0], x.shape[1] // 2) or sin.shape != cos.shape:
+        raise ValueError("rope_interleaved_f32: cos/sin must be [rows, D/2] with one row per row of x")
     out = np.empty_like(x)
     _chk(lib().sage_oracle_rope_interleaved_f32(_p(x), _p(cos), _p(sin), x.shape[0], x.shape[1], _p(out)),
          "rope_interleaved_f32")
@@ -204,6 +206,11 @@ def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=
     if cos is not None:
         cos = np.ascontiguousarray(cos, dtype=np.float32)
         sin = np.ascontiguousarray(sin, dtype=np.float32)
+        need = (B - 1) * table_batch_rows + S * H
+        if cos.shape[0] < need or cos.shape[1] != D // 2 or sin.shape != cos.shape:
+            raise ValueError("norm_rope_bf16: cos/sin must be [>= %d, %d]" % (need, D // 2))
+    if g.shape != (D,):
+        raise ValueError("norm_rope_bf16: gain must be [%d]" % D)
     _chk(lib().sage_oracle_norm_rope_bf16(_p(x), B, H, S, D, strides_bshd(S, H, D), _p(g), eps,
                                           _p(cos) if cos is not None else None,
                                           _p(sin) if sin is not None else None, table_batch_rows, _p(y)),
