@@ -117,7 +117,7 @@ struct NoHook {
 // `mean` points at the D means of this (b,h) (global or LDS), or is null.  `hook` runs after
 // the tile's loads are issued and before anything reads `mean` (it may compute the mean into
 // LDS; it must end with a barrier if it does).
-template <int D, int BLK, bool IS_K, typename Hook = NoHook>
+template <int D, int BLK, bool IS_K, bool PRE, typename Hook = NoHook>
 __device__ __forceinline__ void quant_i8_block(
     int t, int h, int b, const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, float cmul, const float* mean,
@@ -148,7 +148,7 @@ __device__ __forceinline__ void quant_i8_block(
         const int c = i * 256 + tid;
         const int row = r0 + c / CPR, col = (c % CPR) * 8;
         unpack8(raw[i], v[i]);
-        if (pre.gain != nullptr) pre_apply<D>(pre, b, h, H, row, col, row < N, v[i]);
+        if constexpr (PRE) pre_apply<D>(pre, b, h, H, row, col, row < N, v[i]);
         if (IS_K) {
             if (mean != nullptr) {
                 const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
@@ -206,14 +206,14 @@ __device__ __forceinline__ void quant_i8_block(
     }
 }
 
-template <int D, int BLK, bool IS_K>
+template <int D, int BLK, bool IS_K, bool PRE>
 __global__ __launch_bounds__(256) void quant_i8_kernel(
     const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
     int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, PreOp pre) {
     __shared__ float red[4];
     const int h = blockIdx.y, b = blockIdx.z;
-    quant_i8_block<D, BLK, IS_K>(blockIdx.x, h, b, x, sb, sh, sn, N, H, n_pad, cmul,
+    quant_i8_block<D, BLK, IS_K, PRE>(blockIdx.x, h, b, x, sb, sh, sn, N, H, n_pad, cmul,
                                  mean ? mean + ((int64_t)b * H + h) * D : nullptr, codes, scales, rowdot, red, pre);
 }
 
@@ -222,9 +222,15 @@ static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t 
                                     float cmul, const float* mean, int8_t* codes, float* scales,
                                     float* rowdot, const PreOp& pre, hipStream_t st) {
     dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
-#define SAGE_LAUNCH_Q(BLK)                                                                    \
-    hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K>), grid, block, 0, st, x.p, x.sb, x.sh,   \
-                       x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot, pre)
+#define SAGE_LAUNCH_Q(BLK)                                                                          \
+    do {                                                                                           \
+        if (pre.gain != nullptr)                                                                   \
+            hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K, true>), grid, block, 0, st, x.p, x.sb, \
+                               x.sh, x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot, pre);   \
+        else                                                                                       \
+            hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K, false>), grid, block, 0, st, x.p, x.sb, \
+                               x.sh, x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot, pre);   \
+    } while (0)
     switch (blk) {
         case 32: SAGE_LAUNCH_Q(32); break;
         case 64: SAGE_LAUNCH_Q(64); break;
@@ -257,7 +263,7 @@ hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_
 // Kernel 2: one thread per (b, h, channel).
 // ---------------------------------------------------------------------------
 // Executed by 16*(D/8) consecutive threads; `tid` is the index among them.
-template <int D>
+template <int D, bool PRE>
 __device__ __forceinline__ void kmean_group_body(
     int g, int h, int b, int tid, const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int ngroups, double* __restrict__ partial, double (*leafsum)[D + 2], const PreOp& pre) {
@@ -277,7 +283,7 @@ __device__ __forceinline__ void kmean_group_body(
     for (int i = 0; i < kLeaf; i++) {
         float x[8];
         unpack8(w[i], x);
-        if (pre.gain != nullptr) pre_apply<D>(pre, b, h, H, s0 + i, col, g >= 0 && s0 + i < N, x);
+        if constexpr (PRE) pre_apply<D>(pre, b, h, H, s0 + i, col, g >= 0 && s0 + i < N, x);
         // rows past N contribute +0.0, which leaves a double sum unchanged
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += (double)x[e];
@@ -294,12 +300,12 @@ __device__ __forceinline__ void kmean_group_body(
     }
 }
 
-template <int D>
+template <int D, bool PRE>
 __global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int ngroups, double* __restrict__ partial, PreOp pre) {
     __shared__ double leafsum[16][D + 2];
-    kmean_group_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x, k, sb, sh, sn, N, H, ngroups, partial, leafsum, pre);
+    kmean_group_body<D, PRE>(blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x, k, sb, sh, sn, N, H, ngroups, partial, leafsum, pre);
 }
 
 __global__ __launch_bounds__(256) void kmean_final_kernel(
@@ -326,11 +332,18 @@ hipError_t launch_kmean(const View& k, int B, int H, int N, int D, double* parti
                         float* kmean, const PreOp& pre, hipStream_t st) {
     const int ngroups = (N + kGroup - 1) / kGroup;
     dim3 grid((unsigned)ngroups, (unsigned)H, (unsigned)B);
-    if (D == 128)
-        hipLaunchKernelGGL((kmean_group_kernel<128>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
+    const bool has_pre = pre.gain != nullptr;
+    if (D == 128 && has_pre)
+        hipLaunchKernelGGL((kmean_group_kernel<128, true>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
+                           N, H, ngroups, partial, pre);
+    else if (D == 128)
+        hipLaunchKernelGGL((kmean_group_kernel<128, false>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
+                           N, H, ngroups, partial, pre);
+    else if (D == 64 && has_pre)
+        hipLaunchKernelGGL((kmean_group_kernel<64, true>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
                            N, H, ngroups, partial, pre);
     else if (D == 64)
-        hipLaunchKernelGGL((kmean_group_kernel<64>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
+        hipLaunchKernelGGL((kmean_group_kernel<64, false>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
                            N, H, ngroups, partial, pre);
     else
         return hipErrorInvalidValue;
@@ -450,7 +463,7 @@ struct PrepArgs {
     PreOp pre_q, pre_k;
 };
 
-template <int D, int BLKQ>
+template <int D, int BLKQ, bool PRE>
 __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
     constexpr int GPW = 256 / (16 * (D / 8));             // K-mean groups per workgroup
     union Smem {
@@ -463,7 +476,7 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
     const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
     const int b = bh / a.H, h = bh % a.H;
     if (r < a.nq_blk) {
-        quant_i8_block<D, BLKQ, false>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, a.cmul, nullptr,
+        quant_i8_block<D, BLKQ, false, PRE>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, a.cmul, nullptr,
                                        a.q8, a.qscale, nullptr, sm.red, a.pre_q);
     } else if (r < a.nq_blk + a.nv_tile) {
         quant_v_f16_body<D>(r - a.nq_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.v16, sm.tile);
@@ -472,7 +485,7 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
         const int g = (r - a.nq_blk - a.nv_tile) * GPW + sub;
         // groups past the end still take part in the barrier inside; they read nothing and
         // their sum is not stored
-        kmean_group_body<D>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh, a.k.sn,
+        kmean_group_body<D, PRE>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh, a.k.sn,
                             a.Nkv, a.H, a.ngroups, a.partial, sm.leafsum[sub], a.pre_k);
     }
 }
@@ -508,7 +521,7 @@ struct MeanFromPartials {
     }
 };
 
-template <int D, int BLK>
+template <int D, int BLK, bool PRE>
 __global__ __launch_bounds__(256) void kquant_fused_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, const double* __restrict__ partial, int ngroups,
@@ -520,19 +533,26 @@ __global__ __launch_bounds__(256) void kquant_fused_kernel(
     const bool smooth = partial != nullptr;
     MeanFromPartials<D> hook{smooth ? partial + bh * ngroups * D : nullptr, ngroups, N, mean_s,
                              (smooth && t == 0) ? kmean + bh * D : nullptr};
-    quant_i8_block<D, BLK, true>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
+    quant_i8_block<D, BLK, true, PRE>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
                                  codes, scales, nullptr, red, pre, hook);
 }
 
 template <int D>
 static hipError_t launch_prep_d(const PrepArgs& a, int B, int blkq, hipStream_t st) {
     dim3 grid((unsigned)((int64_t)B * a.H * (a.nq_blk + a.nv_tile + a.nk_wg))), block(256);
+    const bool has_pre = a.pre_q.gain != nullptr;
+#define SAGE_LAUNCH_PREP(BLKQ)                                                                \
+    do {                                                                                      \
+        if (has_pre) hipLaunchKernelGGL((prep_kernel<D, BLKQ, true>), grid, block, 0, st, a); \
+        else hipLaunchKernelGGL((prep_kernel<D, BLKQ, false>), grid, block, 0, st, a);        \
+    } while (0)
     switch (blkq) {
-        case 32: hipLaunchKernelGGL((prep_kernel<D, 32>), grid, block, 0, st, a); break;
-        case 64: hipLaunchKernelGGL((prep_kernel<D, 64>), grid, block, 0, st, a); break;
-        case 128: hipLaunchKernelGGL((prep_kernel<D, 128>), grid, block, 0, st, a); break;
+        case 32: SAGE_LAUNCH_PREP(32); break;
+        case 64: SAGE_LAUNCH_PREP(64); break;
+        case 128: SAGE_LAUNCH_PREP(128); break;
         default: return hipErrorInvalidValue;
     }
+#undef SAGE_LAUNCH_PREP
     return hipGetLastError();
 }
 
@@ -559,9 +579,15 @@ hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_
                                const PreOp& pre, hipStream_t st) {
     const int ngroups = (N + kGroup - 1) / kGroup;
     dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
-#define SAGE_LAUNCH_KQ(DD, BLK)                                                                          \
-    hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK>), grid, block, 0, st, k.p, k.sb, k.sh, k.sn, N, H, \
-                       n_pad, partial, ngroups, kmean, codes, scales, pre)
+#define SAGE_LAUNCH_KQ(DD, BLK)                                                                      \
+    do {                                                                                             \
+        if (pre.gain != nullptr)                                                                     \
+            hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK, true>), grid, block, 0, st, k.p, k.sb,  \
+                               k.sh, k.sn, N, H, n_pad, partial, ngroups, kmean, codes, scales, pre); \
+        else                                                                                         \
+            hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK, false>), grid, block, 0, st, k.p, k.sb, \
+                               k.sh, k.sn, N, H, n_pad, partial, ngroups, kmean, codes, scales, pre); \
+    } while (0)
     if (D == 128) {
         switch (blk) {
             case 32: SAGE_LAUNCH_KQ(128, 32); break;
