@@ -126,6 +126,26 @@ int mi355_sage_sdpa_bf16_train_fwd(
     void* stream,
     int variant, void* workspace, size_t workspace_bytes);
 
+/* mi355_sage_sdpa_bf16_train_fwd on the pre-norm projections (default recipe: Q blocks of 128
+ * tokens, 32 for the e4m3 variant; K blocks of 64; K smoothing on), for the blocks that run
+ * rms_norm / rope_interleaved in front of sdpa_flash_train_fwd
+ * (serenitymojo/models/klein/single_block.mojo:977-982 with the flash arm of :102).  Stats is the
+ * log-sum-exp of the scores of the normalised, rotated Q and K. */
+int mi355_sage_sdpa_bf16_norm_rope_train_fwd(
+    const void* Q, const void* K, const void* V, void* O, void* Stats,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems, int64_t stats_offset_elems,
+    int causal, int real_N_q, int real_N_kv,
+    void* stream,
+    int variant,
+    const void* q_gain, const void* k_gain, float eps,
+    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+    void* workspace, size_t workspace_bytes);
+
 /* Bytes of workspace the one-shot calls need for this problem (0 on bad
  * arguments).  No counterpart in the reference, whose shim sizes its own. */
 size_t mi355_sage_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int variant);

@@ -178,6 +178,31 @@ def sdpa_cross_nomask(q, k, v, scale, variant=PV_FP16):
     return o.to(q.dtype)
 
 
+def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin):
+    _check_shapes(name, q_pre, k_pre, v, True)
+    _require_bf16(name, q_pre, k_pre, v)
+    _require_cuda(name, q_pre, k_pre, v)
+    B, S, H, Dh = q_pre.shape
+    if q_norm.numel() != Dh or k_norm.numel() != Dh:
+        raise Error("%s: weight must be [%d]" % (name, Dh))
+    gq = q_norm.to(device=q_pre.device, dtype=torch.bfloat16).contiguous()
+    gk = k_norm.to(device=q_pre.device, dtype=torch.bfloat16).contiguous()
+    batch_rows = 0
+    if (cos is None) != (sin is None):
+        raise Error("%s: cos and sin come together" % name)
+    if cos is not None:
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32:
+            raise Error("%s: cos/sin tables must be F32" % name)
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2:
+            raise Error("%s: cos/sin must be [rows, D/2]" % name)
+        if cos.shape[0] == B * S * H and B > 1:
+            batch_rows = S * H
+        elif cos.shape[0] != S * H:
+            raise Error("%s: cos/sin rows must be S*H (or B*S*H)" % name)
+        cos, sin = cos.contiguous(), sin.contiguous()
+    return gq, gk, cos, sin, batch_rows
+
+
 def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16,
                              blkq=None, blkk=64, smooth_k=True):
     """The attention block of a DiT layer from the projections on, in one call:
@@ -191,29 +216,8 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
     ops/norm.mojo:170-172 does when the gain's dtype differs); cos/sin: F32 [S*H, Dh/2]
     (sampling/klein_sampler.mojo:305-307) or [B*S*H, Dh/2], or None for norm only."""
     name = "qk_norm_rope_sdpa_nomask"
-    _check_shapes(name, q_pre, k_pre, v, True)
-    _require_bf16(name, q_pre, k_pre, v)
-    _require_cuda(name, q_pre, k_pre, v)
+    gq, gk, cos, sin, batch_rows = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin)
     B, S, H, Dh = q_pre.shape
-    if q_norm.numel() != Dh or k_norm.numel() != Dh:
-        raise Error("%s: weight must be [%d]" % (name, Dh))
-    gq = q_norm.to(device=q_pre.device, dtype=torch.bfloat16).contiguous()
-    gk = k_norm.to(device=q_pre.device, dtype=torch.bfloat16).contiguous()
-    batch_rows = 0
-    cp = sp = None
-    if (cos is None) != (sin is None):
-        raise Error("%s: cos and sin come together" % name)
-    if cos is not None:
-        if cos.dtype != torch.float32 or sin.dtype != torch.float32:
-            raise Error("%s: cos/sin tables must be F32" % name)
-        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2:
-            raise Error("%s: cos/sin must be [rows, D/2]" % name)
-        if cos.shape[0] == B * S * H and B > 1:
-            batch_rows = S * H
-        elif cos.shape[0] != S * H:
-            raise Error("%s: cos/sin rows must be S*H (or B*S*H)" % name)
-        cos, sin = cos.contiguous(), sin.contiguous()
-        cp, sp = cos.data_ptr(), sin.data_ptr()
     L = _lib.lib()
     o = torch.empty_like(q_pre)
     nbytes = L.mi355_sage_workspace_bytes(B, H, S, S, Dh, variant)
@@ -224,8 +228,34 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
     rc = L.mi355_sage_sdpa_bf16_norm_rope(
         q_pre.data_ptr(), k_pre.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, S, S, Dh, float(scale),
         st, st, st, st, 0, 0, 0, 0, 0, torch.cuda.current_stream(q_pre.device).cuda_stream,
-        variant, blkq, blkk, int(bool(smooth_k)), gq.data_ptr(), gk.data_ptr(), float(eps), cp, sp, batch_rows,
+        variant, blkq, blkk, int(bool(smooth_k)), gq.data_ptr(), gk.data_ptr(), float(eps),
+        cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
         ws.data_ptr(), ws.numel())
     if rc != 0:
         raise Error("%s: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (name, rc, B, S, H, Dh))
     return o
+
+
+def qk_norm_rope_sdpa_flash_train_fwd(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16):
+    """The same block where the caller keeps the attention statistics for a backward pass:
+    rms_norm / rope_interleaved followed by sdpa_flash_train_fwd
+    (serenitymojo/ops/attention_flash.mojo:149-202).  Returns an SdpaFlashFwd whose stats are the
+    log-sum-exp of the normalised, rotated Q and K."""
+    name = "qk_norm_rope_sdpa_flash_train_fwd"
+    gq, gk, cos, sin, batch_rows = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin)
+    B, S, H, Dh = q_pre.shape
+    L = _lib.lib()
+    o = torch.empty_like(q_pre)
+    stats = torch.empty((B, H, S, 1), dtype=torch.float32, device=q_pre.device)
+    nbytes = L.mi355_sage_workspace_bytes(B, H, S, S, Dh, variant)
+    ws = _workspace(max(nbytes, 256), q_pre.device)
+    st = _lib.strides_bhnd(S, H, Dh)
+    rc = L.mi355_sage_sdpa_bf16_norm_rope_train_fwd(
+        q_pre.data_ptr(), k_pre.data_ptr(), v.data_ptr(), o.data_ptr(), stats.data_ptr(), B, H, S, S, Dh, float(scale),
+        st, st, st, st, 0, 0, 0, 0, 0, 0, S, S, torch.cuda.current_stream(q_pre.device).cuda_stream,
+        variant, gq.data_ptr(), gk.data_ptr(), float(eps),
+        cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
+        ws.data_ptr(), ws.numel())
+    if rc != 0:
+        raise Error("%s: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (name, rc, B, S, H, Dh))
+    return SdpaFlashFwd(o, o, q_pre, k_pre, v, stats)

@@ -357,6 +357,28 @@ int mi355_sage_sdpa_bf16_norm_rope(const void* Q, const void* K, const void* V, 
                      smooth_k ? 1 : 0, workspace, workspace_bytes, pre);
 }
 
+int mi355_sage_sdpa_bf16_norm_rope_train_fwd(const void* Q, const void* K, const void* V, void* O, void* Stats,
+                                             int B, int H, int N_q, int N_kv, int D, float scale,
+                                             const int64_t* q_strides, const int64_t* k_strides,
+                                             const int64_t* v_strides, const int64_t* o_strides,
+                                             int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
+                                             int64_t stats_off, int causal, int real_N_q, int real_N_kv,
+                                             void* stream, int variant,
+                                             const void* q_gain, const void* k_gain, float eps,
+                                             const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+                                             void* workspace, size_t workspace_bytes) {
+    if (!Stats) return MI355_SAGE_EINVAL;
+    (void)real_N_q;
+    Pre pre;
+    int rc;
+    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
+    if (!pre.q.gain) return MI355_SAGE_EINVAL;
+    const int blkq = variant == MI355_SAGE_PV_FP8 ? 32 : 128;
+    return sdpa_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                     o_strides, q_off, k_off, v_off, o_off, stats_off, causal, real_N_kv, stream, variant,
+                     blkq, 64, 1, workspace, workspace_bytes, pre);
+}
+
 int mi355_sage_quant_v_f16(const void* V, int B, int H, int N_kv, int D, const int64_t* v_strides,
                            int64_t v_off, void* v16, void* stream) {
     if (!V || !v16 || !v_strides) return MI355_SAGE_EINVAL;

@@ -139,3 +139,29 @@ def test_argument_errors():
                                           st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 1,
                                           g.data_ptr() + 2, g.data_ptr(), 1e-6, None, None, 0, None, 0)
     assert rc == -2
+
+
+def test_fused_train_fwd_stats(oracle):
+    """Stats of the fused call = natural-log LSE of the scaled scores of the normalised, rotated
+    Q and K (computed here in float64 from the checker's bf16 norm/rope output), and O equals the
+    fused inference call bit for bit."""
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    rng = np.random.default_rng(21)
+    w = WORKLOADS[2].scaled(B=1, H=2, S=384)
+    q, k, v = make_inputs(w)
+    gq, gk = _gains(rng, w.D)
+    cos, sin = _tables(rng, w.S * w.H, w.D)
+    qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
+    gqd, gkd = H.dev_bf16(gq), H.dev_bf16(gk)
+    cd, sd = torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
+    fwd = A.qk_norm_rope_sdpa_flash_train_fwd(qd, kd, vd, gqd, gkd, 1e-6, cd, sd, w.scale)
+    inf = A.qk_norm_rope_sdpa_nomask(qd, kd, vd, gqd, gkd, 1e-6, cd, sd, w.scale)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(H.to_bits(fwd.o), H.to_bits(inf))
+    qn = bf16_bits_to_f32(oracle.norm_rope_bf16(q, gq, 1e-6, cos, sin, 0)).astype(np.float64)
+    kn = bf16_bits_to_f32(oracle.norm_rope_bf16(k, gk, 1e-6, cos, sin, 0)).astype(np.float64)
+    s = np.einsum("bihd,bjhd->bhij", qn, kn) * w.scale
+    lse = np.log(np.exp(s - s.max(-1, keepdims=True)).sum(-1)) + s.max(-1)
+    np.testing.assert_allclose(fwd.stats.cpu().numpy()[..., 0], lse, atol=3e-2)
