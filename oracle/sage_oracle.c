@@ -148,10 +148,15 @@ static int bad_args(const void* q, const void* k, const void* v, const void* o,
     return 0;
 }
 
-int sage_oracle_sdpa_f32(const float* q, const float* k, const float* v, float* o,
-                         int B, int H, int Nq, int Nkv, int D, float scale,
-                         const int64_t* qs, const int64_t* ks,
-                         const int64_t* vs, const int64_t* os) {
+/* mask_lo/mask_hi: keys in [mask_lo, mask_hi) are left out (serenitymojo/ops/attention.mojo:1790-1857
+ * adds -1e4 to them, which leaves exp() == 0 in fp32).  addmask: additive bias in natural-log
+ * units, contiguous [B,H,Nq,Nkv] (attention.mojo:1596-1647), or NULL.  stats (optional,
+ * [B,H,Nq]): natural-log log-sum-exp of the scaled, biased scores. */
+int sage_oracle_sdpa_f32_ex(const float* q, const float* k, const float* v, float* o,
+                            int B, int H, int Nq, int Nkv, int D, float scale,
+                            const int64_t* qs, const int64_t* ks,
+                            const int64_t* vs, const int64_t* os,
+                            int mask_lo, int mask_hi, const float* addmask, float* stats) {
     if (bad_args(q, k, v, o, B, H, Nq, Nkv, D, qs, ks, vs, os)) return -1;
     int64_t rows = (int64_t)B * H * Nq;
     int err = 0;
@@ -176,6 +181,8 @@ int sage_oracle_sdpa_f32(const float* q, const float* k, const float* v, float* 
                 double dot = 0.0;
                 for (int d = 0; d < D; d++) dot += (double)qr[d * qs[3]] * (double)kr[d * ks[3]];
                 double s = dot * (double)scale;
+                if (addmask) s += (double)addmask[(((int64_t)b * H + h) * Nq + i) * (int64_t)Nkv + j];
+                if (j >= mask_lo && j < mask_hi) s = -INFINITY;
                 sc[j] = s;
                 if (s > mx) mx = s;
             }
@@ -189,11 +196,19 @@ int sage_oracle_sdpa_f32(const float* q, const float* k, const float* v, float* 
             }
             float* orow = o + b * os[0] + h * os[1] + i * os[2];
             for (int d = 0; d < D; d++) orow[d * os[3]] = (float)(acc[d] / l);
+            if (stats) stats[((int64_t)b * H + h) * Nq + i] = (float)(mx + log(l));
         }
         free(sc);
         free(acc);
     }
     return err ? -1 : 0;
+}
+
+int sage_oracle_sdpa_f32(const float* q, const float* k, const float* v, float* o,
+                         int B, int H, int Nq, int Nkv, int D, float scale,
+                         const int64_t* qs, const int64_t* ks,
+                         const int64_t* vs, const int64_t* os) {
+    return sage_oracle_sdpa_f32_ex(q, k, v, o, B, H, Nq, Nkv, D, scale, qs, ks, vs, os, 0, 0, NULL, NULL);
 }
 
 int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, float* o,
@@ -255,41 +270,28 @@ static int bad_quant_args(const void* x, int B, int H, int N, int D, const int64
 /* ---- the two ops in front of the path: RMSNorm over D, interleaved RoPE -------------- */
 
 /* serenitymojo/ops/norm.mojo:47-79 (_rms_norm_kernel_f32): out = x * (1/sqrt(mean(x^2)+eps)) * g.
- * The reference adds the squares in the order of its 256-thread shared-memory tree; an fp32
- * sum's last bit depends on that order and nothing the reference holds pins it (its vectors
- * have 6 columns and a 1e-6 bar), so the order here is the one the GPU kernel can afford:
- * runs of 8 consecutive columns added left to right, then the run sums combined pairwise
- * (neighbours first: strides 1, 2, 4, ... runs).  Column counts that are not a multiple of 8
- * are added left to right. */
-static float sumsq_blocked(const float* v, int cols) {
-    int runs = cols / 8;
-    if (cols % 8 == 0 && runs > 0 && runs <= 1024) {
-        float part[1024];
-        for (int r = 0; r < runs; r++) {
-            float a = 0.0f;
-            for (int e = 0; e < 8; e++) {
-                float sq = v[r * 8 + e] * v[r * 8 + e];
-                a = a + sq;
-            }
-            part[r] = a;
+ * The order in which the squares are added is the reference's own (:56-72): a block of 256
+ * threads, thread t adds x[t]^2, x[t+256]^2, ... left to right into `local` (starting from 0),
+ * writes it to shared[t], then the tree  shared[t] += shared[t + active]  runs for
+ * active = 128, 64, ..., 1 — the far pairs first.  For D = 128 that is x[t]^2 + x[t+64]^2 first
+ * (the active = 128 step adds the zeros of the idle threads), then strides 32, 16, 8, 4, 2, 1. */
+static float sumsq_tree(const float* v, int cols) {
+    float shared[256];
+    for (int t = 0; t < 256; t++) {
+        float local = 0.0f;
+        for (int c = t; c < cols; c += 256) {
+            float sq = v[c] * v[c];
+            local = local + sq;
         }
-        /* pairwise, neighbours first; an odd one out moves up unchanged */
-        for (int n = runs; n > 1; n = (n + 1) / 2) {
-            for (int r = 0; r + 1 < n; r += 2) part[r / 2] = part[r] + part[r + 1];
-            if (n & 1) part[n / 2] = part[n - 1];
-        }
-        return part[0];
+        shared[t] = local;
     }
-    float a = 0.0f;
-    for (int c = 0; c < cols; c++) {
-        float sq = v[c] * v[c];
-        a = a + sq;
-    }
-    return a;
+    for (int active = 128; active > 0; active /= 2)
+        for (int t = 0; t < active; t++) shared[t] = shared[t] + shared[t + active];
+    return shared[0];
 }
 
 static float rms_inv(const float* v, int cols, float eps) {
-    float ss = sumsq_blocked(v, cols);
+    float ss = sumsq_tree(v, cols);
     float mean = ss / (float)cols;
     return 1.0f / sqrtf(mean + eps);           /* IEEE sqrt and divide (norm.mojo:73) */
 }
@@ -368,29 +370,45 @@ int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, co
 }
 
 /* One block of `rows` tokens by D channels, already transformed to fp32 in
- * `tile` (row-major rows x D): scale and codes. */
-static void quant_block_i8(const float* tile, int rows, int D, int8_t* dst, float* scale_out) {
+ * `tile` (row-major rows x D); keep[i] == 0 marks a masked token: it does not count for
+ * the block maximum and its codes are 0.  keep == NULL: every row counts. */
+static void quant_block_i8(const float* tile, const uint8_t* keep, int rows, int D, int8_t* dst, float* scale_out) {
     float amax = 0.0f;
-    for (int i = 0; i < rows * D; i++) {
-        float a = fabsf(tile[i]);
-        if (a > amax) amax = a;
+    for (int r = 0; r < rows; r++) {
+        if (keep && !keep[r]) continue;
+        for (int d = 0; d < D; d++) {
+            float a = fabsf(tile[r * D + d]);
+            if (a > amax) amax = a;
+        }
     }
     /* scale = amax/127, 1.0 for an all-zero block (ops/fp8_quant.mojo:117) */
     float sc = (amax > 0.0f) ? (amax / 127.0f) : 1.0f;
     *scale_out = sc;
-    for (int i = 0; i < rows * D; i++) {
-        float r = rintf(tile[i] / sc);          /* true divide (:138), RNE (:42-50) */
-        if (r > 127.0f) r = 127.0f;
-        if (r < -127.0f) r = -127.0f;
-        dst[i] = (int8_t)r;
-    }
+    for (int r = 0; r < rows; r++)
+        for (int d = 0; d < D; d++) {
+            float q = 0.0f;
+            if (!keep || keep[r]) {
+                q = rintf(tile[r * D + d] / sc);      /* true divide (:138), RNE (:42-50) */
+                if (q > 127.0f) q = 127.0f;
+                if (q < -127.0f) q = -127.0f;
+            }
+            dst[r * D + d] = (int8_t)q;
+        }
 }
 
-int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
-                        const int64_t* st, float scale, int blkq, int npad_mult,
-                        int8_t* q8, float* qscale) {
+static inline int key_kept(int s, int N, int mask_lo, int mask_hi) {
+    return s < N && !(s >= mask_lo && s < mask_hi);
+}
+
+static float c_of_scale(float scale) {
+    return (float)((double)scale * 1.4426950408889634074);   /* scale*log2(e), rounded once */
+}
+
+int sage_oracle_quant_q_ch(const uint16_t* q, int B, int H, int N, int D,
+                           const int64_t* st, float scale, const float* qmul, int blkq, int npad_mult,
+                           int8_t* q8, float* qscale) {
     if (bad_quant_args(q, B, H, N, D, st, blkq, npad_mult) || !q8 || !qscale) return -1;
-    const float c = (float)((double)scale * 1.4426950408889634074);   /* scale*log2(e), rounded once */
+    const float c = c_of_scale(scale);
     int64_t npad = sage_oracle_pad(N, npad_mult);
     int nblk = (N + blkq - 1) / blkq;
     memset(q8, 0, (size_t)B * H * npad * D);
@@ -405,12 +423,13 @@ int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
             int b = (int)(w / ((int64_t)nblk * H));
             int r0 = t * blkq;
             int rows = (N - r0 < blkq) ? (N - r0) : blkq;
+            const float* mul = qmul ? qmul + ((int64_t)b * H + h) * D : NULL;
             for (int i = 0; i < rows; i++) {
                 const uint16_t* src = q + b * st[0] + h * st[1] + (int64_t)(r0 + i) * st[2];
                 for (int d = 0; d < D; d++)
-                    tile[i * D + d] = sage_oracle_bf16_to_f32(src[d * st[3]]) * c;
+                    tile[i * D + d] = sage_oracle_bf16_to_f32(src[d * st[3]]) * (mul ? mul[d] : c);
             }
-            quant_block_i8(tile, rows, D, q8 + (((int64_t)b * H + h) * npad + r0) * D,
+            quant_block_i8(tile, NULL, rows, D, q8 + (((int64_t)b * H + h) * npad + r0) * D,
                            qscale + ((int64_t)b * H + h) * nblk + t);
         }
         free(tile);
@@ -418,9 +437,20 @@ int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
     return 0;
 }
 
-int sage_oracle_kmean(const uint16_t* k, int B, int H, int N, int D,
-                      const int64_t* st, float* kmean) {
-    if (bad_quant_args(k, B, H, N, D, st, 1, 1) || !kmean) return -1;
+int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
+                        const int64_t* st, float scale, int blkq, int npad_mult,
+                        int8_t* q8, float* qscale) {
+    return sage_oracle_quant_q_ch(q, B, H, N, D, st, scale, NULL, blkq, npad_mult, q8, qscale);
+}
+
+int sage_oracle_kstats(const uint16_t* k, int B, int H, int N, int D, const int64_t* st,
+                       float scale, int flags, int mask_lo, int mask_hi,
+                       float* kmean, float* qmul, float* kmul) {
+    if (bad_quant_args(k, B, H, N, D, st, 1, 1) || !kmean || !qmul || !kmul) return -1;
+    int kept = 0;
+    for (int s = 0; s < N; s++) kept += key_kept(s, N, mask_lo, mask_hi);
+    if (kept == 0) return -1;
+    const float c = c_of_scale(scale);
     int64_t work = (int64_t)B * H;
 #pragma omp parallel for schedule(static)
     for (int64_t w = 0; w < work; w++) {
@@ -428,28 +458,56 @@ int sage_oracle_kmean(const uint16_t* k, int B, int H, int N, int D,
         int b = (int)(w / H);
         for (int d = 0; d < D; d++) {
             /* fixed summation tree: 16-token leaves (tokens ascending), 16-leaf
-             * groups (leaves ascending), groups ascending */
+             * groups (leaves ascending), groups ascending; masked tokens add +0.0 */
             double sum = 0.0;
+            float kmax = -INFINITY, kmin = INFINITY;
             for (int g0 = 0; g0 < N; g0 += 256) {
                 double group = 0.0;
                 for (int u0 = g0; u0 < g0 + 256 && u0 < N; u0 += 16) {
                     int u1 = (u0 + 16 < N) ? u0 + 16 : N;
                     double leaf = 0.0;
-                    for (int s = u0; s < u1; s++)
-                        leaf += (double)sage_oracle_bf16_to_f32(k[b * st[0] + h * st[1] + (int64_t)s * st[2] + d * st[3]]);
+                    for (int s = u0; s < u1; s++) {
+                        if (!key_kept(s, N, mask_lo, mask_hi)) continue;
+                        float x = sage_oracle_bf16_to_f32(k[b * st[0] + h * st[1] + (int64_t)s * st[2] + d * st[3]]);
+                        leaf += (double)x;
+                        if (x > kmax) kmax = x;
+                        if (x < kmin) kmin = x;
+                    }
                     group += leaf;
                 }
                 sum += group;
             }
-            kmean[w * D + d] = (float)(sum / (double)N);
+            float mean = (flags & 1) ? (float)(sum / (double)kept) : 0.0f;
+            float s_d = 1.0f;
+            if (flags & 2) {
+                /* rounding is monotone, so the largest |k - mean| over the keys is reached at the
+                 * largest or the smallest key of the channel */
+                float hi = fabsf(kmax - mean), lo = fabsf(kmin - mean);
+                float amax = hi > lo ? hi : lo;
+                if (amax > 0.0f) s_d = sqrtf(amax);
+            }
+            kmean[w * D + d] = mean;
+            kmul[w * D + d] = 1.0f / s_d;
+            qmul[w * D + d] = c * s_d;
         }
     }
     return 0;
 }
 
-int sage_oracle_quant_k(const uint16_t* k, int B, int H, int N, int D,
-                        const int64_t* st, const float* kmean, int blkk, int npad_mult,
-                        int8_t* k8, float* kscale) {
+int sage_oracle_kmean(const uint16_t* k, int B, int H, int N, int D,
+                      const int64_t* st, float* kmean) {
+    if (bad_quant_args(k, B, H, N, D, st, 1, 1) || !kmean) return -1;
+    float* tmp = (float*)malloc(sizeof(float) * 2 * (size_t)B * H * D);
+    if (!tmp) return -1;
+    int rc = sage_oracle_kstats(k, B, H, N, D, st, 1.0f, 1, 0, 0, kmean, tmp, tmp + (size_t)B * H * D);
+    free(tmp);
+    return rc;
+}
+
+int sage_oracle_quant_k_ch(const uint16_t* k, int B, int H, int N, int D,
+                           const int64_t* st, const float* kmean, const float* kmul,
+                           int mask_lo, int mask_hi, int blkk, int npad_mult,
+                           int8_t* k8, float* kscale) {
     if (bad_quant_args(k, B, H, N, D, st, blkk, npad_mult) || !k8 || !kscale) return -1;
     int64_t npad = sage_oracle_pad(N, npad_mult);
     int nblk = (N + blkk - 1) / blkk;
@@ -458,6 +516,7 @@ int sage_oracle_quant_k(const uint16_t* k, int B, int H, int N, int D,
 #pragma omp parallel
     {
         float* tile = (float*)malloc(sizeof(float) * (size_t)blkk * D);
+        uint8_t* keep = (uint8_t*)malloc((size_t)blkk);
 #pragma omp for schedule(static)
         for (int64_t w = 0; w < work; w++) {
             int t = (int)(w % nblk);
@@ -466,19 +525,30 @@ int sage_oracle_quant_k(const uint16_t* k, int B, int H, int N, int D,
             int r0 = t * blkk;
             int rows = (N - r0 < blkk) ? (N - r0) : blkk;
             const float* mu = kmean ? kmean + ((int64_t)b * H + h) * D : NULL;
+            const float* mul = kmul ? kmul + ((int64_t)b * H + h) * D : NULL;
             for (int i = 0; i < rows; i++) {
                 const uint16_t* src = k + b * st[0] + h * st[1] + (int64_t)(r0 + i) * st[2];
+                keep[i] = (uint8_t)key_kept(r0 + i, N, mask_lo, mask_hi);
                 for (int d = 0; d < D; d++) {
                     float x = sage_oracle_bf16_to_f32(src[d * st[3]]);
-                    tile[i * D + d] = mu ? (x - mu[d]) : x;
+                    if (mu) x = x - mu[d];
+                    if (mul) x = x * mul[d];
+                    tile[i * D + d] = x;
                 }
             }
-            quant_block_i8(tile, rows, D, k8 + (((int64_t)b * H + h) * npad + r0) * D,
+            quant_block_i8(tile, keep, rows, D, k8 + (((int64_t)b * H + h) * npad + r0) * D,
                            kscale + ((int64_t)b * H + h) * nblk + t);
         }
         free(tile);
+        free(keep);
     }
     return 0;
+}
+
+int sage_oracle_quant_k(const uint16_t* k, int B, int H, int N, int D,
+                        const int64_t* st, const float* kmean, int blkk, int npad_mult,
+                        int8_t* k8, float* kscale) {
+    return sage_oracle_quant_k_ch(k, B, H, N, D, st, kmean, NULL, 0, 0, blkk, npad_mult, k8, kscale);
 }
 
 int sage_oracle_quant_v_f16(const uint16_t* v, int B, int H, int N, int D,
@@ -499,8 +569,9 @@ int sage_oracle_quant_v_f16(const uint16_t* v, int B, int H, int N, int D,
     return 0;
 }
 
-int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
-                            const int64_t* st, int npad_mult, uint8_t* v8, float* vscale) {
+int sage_oracle_quant_v_fp8_masked(const uint16_t* v, int B, int H, int N, int D,
+                                   const int64_t* st, int mask_lo, int mask_hi, int npad_mult,
+                                   uint8_t* v8, float* vscale) {
     if (bad_quant_args(v, B, H, N, D, st, 1, npad_mult) || !v8 || !vscale) return -1;
     int64_t npad = sage_oracle_pad(N, npad_mult);
     memset(v8, 0, (size_t)B * H * npad * D);
@@ -512,6 +583,7 @@ int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
         for (int d = 0; d < D; d++) {
             float amax = 0.0f;
             for (int s = 0; s < N; s++) {
+                if (!key_kept(s, N, mask_lo, mask_hi)) continue;
                 float a = fabsf(sage_oracle_bf16_to_f32(v[b * st[0] + h * st[1] + (int64_t)s * st[2] + d * st[3]]));
                 if (a > amax) amax = a;
             }
@@ -521,11 +593,17 @@ int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
         for (int s = 0; s < N; s++) {
             const uint16_t* src = v + b * st[0] + h * st[1] + (int64_t)s * st[2];
             uint8_t* dst = v8 + ((int64_t)w * npad + s) * D;
+            /* masked rows are encoded too (saturating): their probabilities are zero */
             for (int d = 0; d < D; d++)
                 dst[d] = sage_oracle_f32_to_e4m3(sage_oracle_bf16_to_f32(src[d * st[3]]) / vscale[w * D + d]);
         }
     }
     return 0;
+}
+
+int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
+                            const int64_t* st, int npad_mult, uint8_t* v8, float* vscale) {
+    return sage_oracle_quant_v_fp8_masked(v, B, H, N, D, st, 0, 0, npad_mult, v8, vscale);
 }
 
 /* ------------------------------------------------------------------------ */
@@ -538,11 +616,12 @@ static inline int32_t dot_i8(const int8_t* a, const int8_t* b, int D) {
     return acc;
 }
 
-int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t NqPad,
-                     const int8_t* k8, const float* kscale, int blkk, int64_t NkvPad,
-                     const void* vq, const float* vscale, int variant,
-                     int B, int H, int Nq, int Nkv, int D,
-                     uint16_t* o_bf16, float* o_f32, const int64_t* os) {
+int sage_oracle_attn_ex(const int8_t* q8, const float* qscale, int blkq, int64_t NqPad,
+                        const int8_t* k8, const float* kscale, int blkk, int64_t NkvPad,
+                        const void* vq, const float* vscale, int variant,
+                        int B, int H, int Nq, int Nkv, int D,
+                        int mask_lo, int mask_hi, const float* addmask, const float* qshift,
+                        uint16_t* o_bf16, float* o_f32, const int64_t* os, float* stats) {
     if (!q8 || !qscale || !k8 || !kscale || !vq || !os) return -1;
     if (!o_bf16 && !o_f32) return -1;
     if (B <= 0 || H <= 0 || Nq <= 0 || Nkv <= 0 || D <= 0 || blkq <= 0 || blkk <= 0) return -1;
@@ -580,15 +659,23 @@ int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t Nq
             float sq = qscale[bh * nqb + i / blkq];
             float mx = -INFINITY;
             for (int j = 0; j < Nkv; j++) {
+                if (!key_kept(j, Nkv, mask_lo, mask_hi)) { sc[j] = -INFINITY; continue; }
                 int32_t a = dot_i8(qr, k8 + (bh * NkvPad + j) * D, D);
                 float s = (float)a * (sq * kscale[bh * nkb + j / blkk]);
+                /* an additive mask is given in natural-log units per (b,h,i,j) */
+                if (addmask) s = s + addmask[(bh * Nq + i) * (int64_t)Nkv + j] * 1.44269504088896340736f;
                 sc[j] = s;
                 if (s > mx) mx = s;
             }
+            /* e4m3 probabilities are taken against an INTEGER reference (the row maximum rounded
+             * up): moving the reference by a whole number only shifts the exponent of every
+             * probability, so any kernel that keeps an integer reference within the format's
+             * range rounds each probability to the same significand. */
+            float mref = variant == 1 ? ceilf(mx) : mx;
             double l = 0.0;
             for (int d = 0; d < D; d++) acc[d] = 0.0f;
             for (int j = 0; j < Nkv; j++) {
-                float p = exp2f(sc[j] - mx);
+                float p = exp2f(sc[j] - mref);
                 l += (double)p;
                 float pq = variant == 0
                     ? sage_oracle_f16_to_f32(sage_oracle_f32_to_f16(p))
@@ -605,6 +692,12 @@ int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t Nq
                 if (o_f32) o_f32[off] = (float)o;
                 if (o_bf16) o_bf16[off] = sage_oracle_f32_to_bf16((float)o);
             }
+            if (stats) {
+                /* natural-log log-sum-exp of the scaled scores; K smoothing lowered every score of
+                 * the row by qshift (log2 units) */
+                double lse2 = (double)mref + log2(l) + (qshift ? (double)qshift[bh * NqPad + i] : 0.0);
+                stats[bh * Nq + i] = (float)(lse2 * 0.69314718055994530942);
+            }
         }
         free(sc);
         free(acc);
@@ -613,12 +706,40 @@ int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t Nq
     return err ? -1 : 0;
 }
 
-int sage_oracle_sdpa_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                          uint16_t* o, float* o_f32,
-                          int B, int H, int Nq, int Nkv, int D, float scale,
-                          const int64_t* qs, const int64_t* ks,
-                          const int64_t* vs, const int64_t* os,
-                          int variant, int blkq, int blkk, int smooth_k) {
+int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t NqPad,
+                     const int8_t* k8, const float* kscale, int blkk, int64_t NkvPad,
+                     const void* vq, const float* vscale, int variant,
+                     int B, int H, int Nq, int Nkv, int D,
+                     uint16_t* o_bf16, float* o_f32, const int64_t* os) {
+    return sage_oracle_attn_ex(q8, qscale, blkq, NqPad, k8, kscale, blkk, NkvPad, vq, vscale, variant,
+                               B, H, Nq, Nkv, D, 0, 0, NULL, NULL, o_bf16, o_f32, os, NULL);
+}
+
+/* <q*c, kmean> per query row (log2 units): what K smoothing subtracts from every score of the row. */
+static void rowdot_q(const uint16_t* q, int B, int H, int N, int D, const int64_t* st, float scale,
+                     const float* kmean, int64_t npad, float* out) {
+    const float c = c_of_scale(scale);
+    int64_t work = (int64_t)B * H * N;
+#pragma omp parallel for schedule(static)
+    for (int64_t w = 0; w < work; w++) {
+        int i = (int)(w % N);
+        int64_t bh = w / N;
+        int h = (int)(bh % H), b = (int)(bh / H);
+        const uint16_t* src = q + b * st[0] + h * st[1] + (int64_t)i * st[2];
+        double dot = 0.0;
+        for (int d = 0; d < D; d++)
+            dot += (double)(sage_oracle_bf16_to_f32(src[d * st[3]]) * c) * (double)kmean[bh * D + d];
+        out[bh * npad + i] = (float)dot;
+    }
+}
+
+int sage_oracle_sdpa_bf16_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                             uint16_t* o, float* o_f32, float* stats,
+                             int B, int H, int Nq, int Nkv, int D, float scale,
+                             const int64_t* qs, const int64_t* ks,
+                             const int64_t* vs, const int64_t* os,
+                             int variant, int blkq, int blkk, int k_flags,
+                             int mask_lo, int mask_hi, const float* addmask) {
     if (bad_args(q, k, v, o ? (void*)o : (void*)o_f32, B, H, Nq, Nkv, D, qs, ks, vs, os)) return -1;
     if (blkq <= 0 || blkk <= 0) return -1;
     int64_t nqp = sage_oracle_pad(Nq, blkq), nkp = sage_oracle_pad(Nkv, blkk);
@@ -628,20 +749,34 @@ int sage_oracle_sdpa_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* 
     int8_t* k8 = (int8_t*)malloc(bh * nkp * D);
     float* qsc = (float*)malloc(sizeof(float) * bh * nqb);
     float* ksc = (float*)malloc(sizeof(float) * bh * nkb);
-    float* mu = (float*)malloc(sizeof(float) * bh * D);
+    float* mu = (float*)malloc(sizeof(float) * bh * D * 3);
     float* vsc = (float*)malloc(sizeof(float) * bh * D);
+    float* shift = stats ? (float*)malloc(sizeof(float) * bh * nqp) : NULL;
     void* vq = malloc(bh * nkp * D * (variant == 0 ? 2 : 1));
     int rc = -1;
-    if (q8 && k8 && qsc && ksc && mu && vsc && vq) {
-        rc = sage_oracle_quant_q(q, B, H, Nq, D, qs, scale, blkq, blkq, q8, qsc);
-        if (!rc && smooth_k) rc = sage_oracle_kmean(k, B, H, Nkv, D, ks, mu);
-        if (!rc) rc = sage_oracle_quant_k(k, B, H, Nkv, D, ks, smooth_k ? mu : NULL, blkk, blkk, k8, ksc);
+    if (q8 && k8 && qsc && ksc && mu && vsc && vq && (!stats || shift)) {
+        float* qmul = mu + bh * D;
+        float* kmul = mu + 2 * bh * D;
+        rc = sage_oracle_kstats(k, B, H, Nkv, D, ks, scale, k_flags, mask_lo, mask_hi, mu, qmul, kmul);
+        if (!rc) rc = sage_oracle_quant_q_ch(q, B, H, Nq, D, qs, scale, qmul, blkq, blkq, q8, qsc);
+        if (!rc) rc = sage_oracle_quant_k_ch(k, B, H, Nkv, D, ks, mu, kmul, mask_lo, mask_hi, blkk, blkk, k8, ksc);
         if (!rc) rc = variant == 0
             ? sage_oracle_quant_v_f16(v, B, H, Nkv, D, vs, blkk, (uint16_t*)vq)
-            : sage_oracle_quant_v_fp8(v, B, H, Nkv, D, vs, blkk, (uint8_t*)vq, vsc);
-        if (!rc) rc = sage_oracle_attn(q8, qsc, blkq, nqp, k8, ksc, blkk, nkp, vq, vsc, variant,
-                                       B, H, Nq, Nkv, D, o, o_f32, os);
+            : sage_oracle_quant_v_fp8_masked(v, B, H, Nkv, D, vs, mask_lo, mask_hi, blkk, (uint8_t*)vq, vsc);
+        if (!rc && stats) rowdot_q(q, B, H, Nq, D, qs, scale, mu, nqp, shift);
+        if (!rc) rc = sage_oracle_attn_ex(q8, qsc, blkq, nqp, k8, ksc, blkk, nkp, vq, vsc, variant,
+                                          B, H, Nq, Nkv, D, mask_lo, mask_hi, addmask, shift, o, o_f32, os, stats);
     }
-    free(q8); free(k8); free(qsc); free(ksc); free(mu); free(vsc); free(vq);
+    free(q8); free(k8); free(qsc); free(ksc); free(mu); free(vsc); free(vq); free(shift);
     return rc;
+}
+
+int sage_oracle_sdpa_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                          uint16_t* o, float* o_f32,
+                          int B, int H, int Nq, int Nkv, int D, float scale,
+                          const int64_t* qs, const int64_t* ks,
+                          const int64_t* vs, const int64_t* os,
+                          int variant, int blkq, int blkk, int k_flags) {
+    return sage_oracle_sdpa_bf16_ex(q, k, v, o, o_f32, NULL, B, H, Nq, Nkv, D, scale, qs, ks, vs, os,
+                                    variant, blkq, blkk, k_flags, 0, 0, NULL);
 }

@@ -18,9 +18,14 @@
  *       (ops/tests/fp8_quant_smoke.mojo:108-143) + torch / numpy library codecs.
  *   sage_oracle_rms_norm_f32 / _rope_interleaved_f32 ... reference vectors
  *       (ops_smoke.mojo:78-96, ops_smoke2.mojo:95-120) + the closed form of
- *       ops_smoke2.mojo:372-403.  sage_oracle_norm_rope_bf16 composes them with RNE bf16
- *       stores; its last-bit behaviour (summation order, no FMA) is PARITY UNPINNED.
- *   sage_oracle_quant_q / _kmean / _quant_k / _quant_v_* , sage_oracle_attn:
+ *       ops_smoke2.mojo:372-403.  The squares are added in the order the reference's kernel
+ *       spells out (ops/norm.mojo:56-72).  sage_oracle_norm_rope_bf16 composes the two with RNE
+ *       bf16 stores; whether the reference's compiler contracts the products of the rotation
+ *       into fused multiply-adds is the one thing its text cannot pin (PARITY UNPINNED there;
+ *       this file uses separately rounded products).
+ *   sage_oracle_sdpa_f32_ex (key range mask, additive mask) ... reduces to sage_oracle_sdpa_f32
+ *       on the kept keys / with a zero mask; float64 brute force (tests/).
+ *   sage_oracle_quant_q* / _kstats / _kmean / _quant_k* / _quant_v_* , sage_oracle_attn*:
  *       PARITY UNPINNED by the reference — it holds no INT8 / SageAttention
  *       code, test or vector.  They are pinned only by closed forms, invariants
  *       and an independent numpy restatement (tests/), never by reference data.
@@ -58,6 +63,16 @@ int sage_oracle_sdpa_f32(const float* q, const float* k, const float* v, float* 
                          const int64_t* qs, const int64_t* ks,
                          const int64_t* vs, const int64_t* os);
 
+/* The same with keys [mask_lo, mask_hi) left out (what serenitymojo/ops/attention.mojo:1790-1857
+ * does with a -1e4 bias), an optional additive bias in natural-log units, contiguous
+ * [B,H,Nq,Nkv] (attention.mojo:1596-1647, :1897-1936), and an optional log-sum-exp output
+ * stats [B,H,Nq] (natural log, of the scaled and biased scores). */
+int sage_oracle_sdpa_f32_ex(const float* q, const float* k, const float* v, float* o,
+                            int B, int H, int Nq, int Nkv, int D, float scale,
+                            const int64_t* qs, const int64_t* ks,
+                            const int64_t* vs, const int64_t* os,
+                            int mask_lo, int mask_hi, const float* addmask, float* stats);
+
 /* One-key-at-a-time online-softmax recurrence in fp32, restating
  * serenitymojo/ops/attention.mojo:744-801 (m starts at -3e38, natural exp). */
 int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, float* o,
@@ -67,8 +82,8 @@ int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, 
 
 /* ---- the two ops in front of the path (fused into the quantizers by the product) ---- */
 /* RMSNorm rows x cols in fp32: serenitymojo/ops/norm.mojo:47-79.  Pinned by the reference's
- * vector serenitymojo/ops_smoke.mojo:78-96 and the closed form of ops_smoke2.mojo:372-403
- * (to their fp32 tolerance; the summation order of the squares is this file's own). */
+ * vector serenitymojo/ops_smoke.mojo:78-96 and the closed form of ops_smoke2.mojo:372-403;
+ * the squares are added in the order of the reference's kernel (norm.mojo:56-72). */
 int sage_oracle_rms_norm_f32(const float* x, const float* g, int64_t rows, int cols, float eps, float* out);
 /* Interleaved RoPE in fp32: serenitymojo/ops/rope.mojo:7-9.  Pinned by ops_smoke2.mojo:95-120. */
 int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const float* sn,
@@ -92,6 +107,34 @@ int64_t sage_oracle_pad(int64_t n, int64_t mult);
 int sage_oracle_quant_q(const uint16_t* q, int B, int H, int N, int D,
                         const int64_t* strides, float scale, int blkq, int npad_mult,
                         int8_t* q8, float* qscale);
+
+/* Per-channel K statistics over the kept keys (token s is kept unless mask_lo <= s < mask_hi),
+ * per (b,h,d):
+ *   mean  (flags & 1): the summation tree of sage_oracle_kmean below with masked tokens adding
+ *         +0.0, divided by the number of kept keys; 0 when the flag is clear.
+ *   s_d   (flags & 2): sqrtf(max over kept keys of |f32(k) - mean|) (1 when that maximum is 0);
+ *         1 when the flag is clear.  This balances the channels between K and Q: K is divided
+ *         and Q multiplied by s_d, which leaves every score unchanged in real arithmetic and
+ *         takes the square root of a channel's excess range out of each side.
+ *   kmul = 1.0f / s_d,  qmul = c * s_d  with c = fp32(scale*log2(e)).
+ * kmean, qmul, kmul: [B,H,D].  Returns -1 when no key is kept. */
+int sage_oracle_kstats(const uint16_t* k, int B, int H, int N, int D, const int64_t* strides,
+                       float scale, int flags, int mask_lo, int mask_hi,
+                       float* kmean, float* qmul, float* kmul);
+
+/* Q with a per-channel multiplier: x = f32(bf16) * qmul[b,h,d] (qmul NULL: the scalar c),
+ * then the per-block INT8 rule of sage_oracle_quant_q. */
+int sage_oracle_quant_q_ch(const uint16_t* q, int B, int H, int N, int D,
+                           const int64_t* strides, float scale, const float* qmul, int blkq, int npad_mult,
+                           int8_t* q8, float* qscale);
+
+/* K with mean and per-channel multiplier: x = (f32(bf16) - kmean[b,h,d]) * kmul[b,h,d] (two
+ * fp32 operations; either pointer may be NULL), then the per-block INT8 rule.  Masked tokens
+ * do not count for their block's maximum and get code 0. */
+int sage_oracle_quant_k_ch(const uint16_t* k, int B, int H, int N, int D,
+                           const int64_t* strides, const float* kmean, const float* kmul,
+                           int mask_lo, int mask_hi, int blkk, int npad_mult,
+                           int8_t* k8, float* kscale);
 
 /* K mean over tokens per (b,h,d) with a fixed summation tree in double:
  * 16-token leaves (tokens ascending), groups of 16 leaves (ascending), groups
@@ -118,10 +161,18 @@ int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
                             const int64_t* strides, int npad_mult,
                             uint8_t* v8, float* vscale);
 
+/* The same with the channel maximum taken over the kept keys only. */
+int sage_oracle_quant_v_fp8_masked(const uint16_t* v, int B, int H, int N, int D,
+                                   const int64_t* strides, int mask_lo, int mask_hi, int npad_mult,
+                                   uint8_t* v8, float* vscale);
+
 /* ---- quantized attention ------------------------------------------------ */
 /* s[i,j] = float(sum_d q8*k8) * (qscale*kscale)   (log2 domain)
- * p = exp2(s - max_j s);  variant 0: P16 = f16(p), O = sum P16*V16 / sum p
- *                         variant 1: P8 = e4m3(p*448), O = sum P8*V8 * vscale / (448 * sum p)
+ * variant 0: p = exp2(s - max_j s), P16 = f16(p), O = sum P16*V16 / sum p
+ * variant 1: p = exp2(s - ceil(max_j s)), P8 = e4m3(p*448), O = sum P8*V8 * vscale / (448 * sum p)
+ *            (an integer reference: shifting it by a whole number only moves the exponent of
+ *            every probability, so their e4m3 significands do not depend on which integer an
+ *            implementation that walks the keys in tiles happens to hold)
  * O -> bf16 RNE in the caller's strides; o_f32 (optional, same strides) gets
  * the unrounded value.  Padded tensors as produced by the quantizers above
  * with token pads NqPad / NkvPad. */
@@ -131,14 +182,33 @@ int sage_oracle_attn(const int8_t* q8, const float* qscale, int blkq, int64_t Nq
                      int B, int H, int Nq, int Nkv, int D,
                      uint16_t* o_bf16, float* o_f32, const int64_t* os);
 
+/* The same with keys [mask_lo, mask_hi) masked, an optional additive bias (natural-log units,
+ * contiguous [B,H,Nq,Nkv], converted to the log2 domain with one fp32 multiply and added to the
+ * dequantised score), qshift [B,H,NqPad] (log2 units, may be NULL) and an optional stats output
+ * [B,H,Nq]: (reference + log2(sum p) + qshift) * ln 2. */
+int sage_oracle_attn_ex(const int8_t* q8, const float* qscale, int blkq, int64_t NqPad,
+                        const int8_t* k8, const float* kscale, int blkk, int64_t NkvPad,
+                        const void* vq, const float* vscale, int variant,
+                        int B, int H, int Nq, int Nkv, int D,
+                        int mask_lo, int mask_hi, const float* addmask, const float* qshift,
+                        uint16_t* o_bf16, float* o_f32, const int64_t* os, float* stats);
+
 /* Whole path on bf16 inputs (quantize + attention), the CPU baseline's unit
- * of work.  Allocates its own temporaries.  smooth_k: 0/1. */
+ * of work.  Allocates its own temporaries.  k_flags: bit 0 = K mean smoothing, bit 1 =
+ * per-channel Q/K balancing. */
 int sage_oracle_sdpa_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                           uint16_t* o, float* o_f32,
                           int B, int H, int Nq, int Nkv, int D, float scale,
                           const int64_t* qs, const int64_t* ks,
                           const int64_t* vs, const int64_t* os,
-                          int variant, int blkq, int blkk, int smooth_k);
+                          int variant, int blkq, int blkk, int k_flags);
+int sage_oracle_sdpa_bf16_ex(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                             uint16_t* o, float* o_f32, float* stats,
+                             int B, int H, int Nq, int Nkv, int D, float scale,
+                             const int64_t* qs, const int64_t* ks,
+                             const int64_t* vs, const int64_t* os,
+                             int variant, int blkq, int blkk, int k_flags,
+                             int mask_lo, int mask_hi, const float* addmask);
 
 int sage_oracle_num_threads(void);
 

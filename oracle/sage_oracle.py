@@ -58,6 +58,30 @@ def lib():
         L.sage_oracle_quant_q.restype = ctypes.c_int
         L.sage_oracle_quant_q.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_float,
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_sdpa_f32_ex.restype = ctypes.c_int
+        L.sage_oracle_sdpa_f32_ex.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [
+                                              ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_kstats.restype = ctypes.c_int
+        L.sage_oracle_kstats.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_float] + [ctypes.c_int] * 3 + [
+                                         ctypes.c_void_p] * 3
+        L.sage_oracle_quant_q_ch.restype = ctypes.c_int
+        L.sage_oracle_quant_q_ch.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_float, ctypes.c_void_p,
+                                             ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_quant_k_ch.restype = ctypes.c_int
+        L.sage_oracle_quant_k_ch.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p, ctypes.c_void_p] + [
+                                             ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_quant_v_fp8_masked.restype = ctypes.c_int
+        L.sage_oracle_quant_v_fp8_masked.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p] + [ctypes.c_int] * 3 + [
+                                                     ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_attn_ex.restype = ctypes.c_int
+        L.sage_oracle_attn_ex.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
+                                          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
+                                          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int] + [ctypes.c_int] * 5 + [
+                                          ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                          ctypes.c_void_p, ctypes.c_void_p, _i64p, ctypes.c_void_p]
+        L.sage_oracle_sdpa_bf16_ex.restype = ctypes.c_int
+        L.sage_oracle_sdpa_bf16_ex.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [
+                                               ctypes.c_int] * 6 + [ctypes.c_void_p]
         L.sage_oracle_kmean.restype = ctypes.c_int
         L.sage_oracle_kmean.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p]
         L.sage_oracle_quant_k.restype = ctypes.c_int
@@ -162,16 +186,25 @@ def _dims_bshd(q, k):
     return B, H, Sq, Skv, D
 
 
-def sdpa_f32(q, k, v, scale, online=False):
-    """fp32 inputs [B,S,H,D] -> fp32 output [B,Sq,H,D]."""
+def sdpa_f32(q, k, v, scale, online=False, mask_lo=0, mask_hi=0, addmask=None, want_stats=False):
+    """fp32 inputs [B,S,H,D] -> fp32 output [B,Sq,H,D].  Keys [mask_lo, mask_hi) are left out;
+    addmask: additive bias [B,H,Sq,Skv] fp32 (natural-log units); want_stats: also return the
+    log-sum-exp [B,H,Sq]."""
     q, k, v = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v))
     B, H, Sq, Skv, D = _dims_bshd(q, k)
     o = np.empty_like(q)
-    fn = lib().sage_oracle_sdpa_online_f32 if online else lib().sage_oracle_sdpa_f32
-    _chk(fn(_p(q), _p(k), _p(v), _p(o), B, H, Sq, Skv, D, scale,
-            strides_bshd(Sq, H, D), strides_bshd(Skv, H, D), strides_bshd(Skv, H, D),
-            strides_bshd(Sq, H, D)), "sdpa_f32")
-    return o
+    args = (_p(q), _p(k), _p(v), _p(o), B, H, Sq, Skv, D, scale,
+            strides_bshd(Sq, H, D), strides_bshd(Skv, H, D), strides_bshd(Skv, H, D), strides_bshd(Sq, H, D))
+    if online:
+        assert mask_hi <= mask_lo and addmask is None and not want_stats
+        _chk(lib().sage_oracle_sdpa_online_f32(*args), "sdpa_online_f32")
+        return o
+    if addmask is not None:
+        addmask = np.ascontiguousarray(addmask, dtype=np.float32)
+        assert addmask.shape == (B, H, Sq, Skv)
+    stats = np.empty((B, H, Sq), np.float32) if want_stats else None
+    _chk(lib().sage_oracle_sdpa_f32_ex(*args, mask_lo, mask_hi, _p(addmask), _p(stats)), "sdpa_f32")
+    return (o, stats) if want_stats else o
 
 
 def rms_norm_f32(x, g, eps):
@@ -230,6 +263,43 @@ def quant_q(q_bf16, scale, blkq, npad_mult=None):
     return q8, sc
 
 
+def kstats(k_bf16, scale, flags, mask_lo=0, mask_hi=0):
+    """Per-channel K statistics.  Returns (kmean, qmul, kmul), each [B,H,D] fp32."""
+    k = np.ascontiguousarray(k_bf16, dtype=np.uint16)
+    B, S, H, D = k.shape
+    mu, qm, km = (np.empty((B, H, D), np.float32) for _ in range(3))
+    _chk(lib().sage_oracle_kstats(_p(k), B, H, S, D, strides_bshd(S, H, D), scale, flags, mask_lo, mask_hi,
+                                  _p(mu), _p(qm), _p(km)), "kstats")
+    return mu, qm, km
+
+
+def quant_q_ch(q_bf16, scale, qmul, blkq, npad_mult=None):
+    """Q with a per-channel multiplier qmul [B,H,D] (None: the scalar c)."""
+    q = np.ascontiguousarray(q_bf16, dtype=np.uint16)
+    B, S, H, D = q.shape
+    mult = npad_mult or blkq
+    q8 = np.empty((B, H, pad(S, mult), D), np.int8)
+    sc = np.empty((B, H, (S + blkq - 1) // blkq), np.float32)
+    if qmul is not None:
+        qmul = np.ascontiguousarray(qmul, dtype=np.float32)
+    _chk(lib().sage_oracle_quant_q_ch(_p(q), B, H, S, D, strides_bshd(S, H, D), scale, _p(qmul), blkq, mult,
+                                      _p(q8), _p(sc)), "quant_q_ch")
+    return q8, sc
+
+
+def quant_k_ch(k_bf16, mu, kmul, blkk, npad_mult=None, mask_lo=0, mask_hi=0):
+    k = np.ascontiguousarray(k_bf16, dtype=np.uint16)
+    B, S, H, D = k.shape
+    mult = npad_mult or blkk
+    k8 = np.empty((B, H, pad(S, mult), D), np.int8)
+    sc = np.empty((B, H, (S + blkk - 1) // blkk), np.float32)
+    mu = None if mu is None else np.ascontiguousarray(mu, dtype=np.float32)
+    kmul = None if kmul is None else np.ascontiguousarray(kmul, dtype=np.float32)
+    _chk(lib().sage_oracle_quant_k_ch(_p(k), B, H, S, D, strides_bshd(S, H, D), _p(mu), _p(kmul),
+                                      mask_lo, mask_hi, blkk, mult, _p(k8), _p(sc)), "quant_k_ch")
+    return k8, sc
+
+
 def kmean(k_bf16):
     k = np.ascontiguousarray(k_bf16, dtype=np.uint16)
     B, S, H, D = k.shape
@@ -260,41 +330,59 @@ def quant_v_f16(v_bf16, npad_mult):
     return v16
 
 
-def quant_v_fp8(v_bf16, npad_mult):
+def quant_v_fp8(v_bf16, npad_mult, mask_lo=0, mask_hi=0):
     v = np.ascontiguousarray(v_bf16, dtype=np.uint16)
     B, S, H, D = v.shape
     v8 = np.empty((B, H, pad(S, npad_mult), D), np.uint8)
     vs = np.empty((B, H, D), np.float32)
-    _chk(lib().sage_oracle_quant_v_fp8(_p(v), B, H, S, D, strides_bshd(S, H, D), npad_mult,
-                                       _p(v8), _p(vs)), "quant_v_fp8")
+    _chk(lib().sage_oracle_quant_v_fp8_masked(_p(v), B, H, S, D, strides_bshd(S, H, D), mask_lo, mask_hi,
+                                              npad_mult, _p(v8), _p(vs)), "quant_v_fp8")
     return v8, vs
 
 
-def attn(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv):
+def attn(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv, mask_lo=0, mask_hi=0,
+         addmask=None, qshift=None, want_stats=False):
     """Quantized tensors in the oracle's plain [B,H,Npad,D] layout.
-    Returns (o_bf16 uint16 [B,Sq,H,D], o_f32 [B,Sq,H,D])."""
+    Returns (o_bf16 uint16 [B,Sq,H,D], o_f32 [B,Sq,H,D]) and, with want_stats, stats [B,H,Sq]."""
     B, H, NqPad, D = q8.shape
     NkvPad = k8.shape[2]
     o16 = np.empty((B, Sq, H, D), np.uint16)
     o32 = np.empty((B, Sq, H, D), np.float32)
-    _chk(lib().sage_oracle_attn(_p(q8), _p(qscale), blkq, NqPad, _p(k8), _p(kscale), blkk, NkvPad,
-                                _p(vq), _p(vscale), variant, B, H, Sq, Skv, D,
-                                _p(o16), _p(o32), strides_bshd(Sq, H, D)), "attn")
-    return o16, o32
+    if addmask is not None:
+        addmask = np.ascontiguousarray(addmask, dtype=np.float32)
+        assert addmask.shape == (B, H, Sq, Skv)
+    if qshift is not None:
+        qshift = np.ascontiguousarray(qshift, dtype=np.float32)
+        assert qshift.shape == (B, H, NqPad)
+    stats = np.empty((B, H, Sq), np.float32) if want_stats else None
+    _chk(lib().sage_oracle_attn_ex(_p(q8), _p(qscale), blkq, NqPad, _p(k8), _p(kscale), blkk, NkvPad,
+                                   _p(vq), _p(vscale), variant, B, H, Sq, Skv, D, mask_lo, mask_hi,
+                                   _p(addmask), _p(qshift), _p(o16), _p(o32), strides_bshd(Sq, H, D), _p(stats)), "attn")
+    return (o16, o32, stats) if want_stats else (o16, o32)
 
 
-def sdpa_bf16(q, k, v, scale, variant=0, blkq=128, blkk=64, smooth_k=True):
+K_SMOOTH = 1
+K_BALANCE = 2
+
+
+def sdpa_bf16(q, k, v, scale, variant=0, blkq=128, blkk=64, smooth_k=True, balance=True,
+              mask_lo=0, mask_hi=0, addmask=None, want_stats=False):
     """Whole quantized path on bf16 (uint16) [B,S,H,D] inputs.
-    Returns (o_bf16 uint16, o_f32)."""
+    Returns (o_bf16 uint16, o_f32) and, with want_stats, stats [B,H,Sq]."""
     q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
     B, H, Sq, Skv, D = _dims_bshd(q, k)
     o16 = np.empty((B, Sq, H, D), np.uint16)
     o32 = np.empty((B, Sq, H, D), np.float32)
-    _chk(lib().sage_oracle_sdpa_bf16(_p(q), _p(k), _p(v), _p(o16), _p(o32), B, H, Sq, Skv, D, scale,
-                                     strides_bshd(Sq, H, D), strides_bshd(Skv, H, D),
-                                     strides_bshd(Skv, H, D), strides_bshd(Sq, H, D),
-                                     variant, blkq, blkk, 1 if smooth_k else 0), "sdpa_bf16")
-    return o16, o32
+    if addmask is not None:
+        addmask = np.ascontiguousarray(addmask, dtype=np.float32)
+        assert addmask.shape == (B, H, Sq, Skv)
+    stats = np.empty((B, H, Sq), np.float32) if want_stats else None
+    flags = (K_SMOOTH if smooth_k else 0) | (K_BALANCE if balance else 0)
+    _chk(lib().sage_oracle_sdpa_bf16_ex(_p(q), _p(k), _p(v), _p(o16), _p(o32), _p(stats), B, H, Sq, Skv, D, scale,
+                                        strides_bshd(Sq, H, D), strides_bshd(Skv, H, D),
+                                        strides_bshd(Skv, H, D), strides_bshd(Sq, H, D),
+                                        variant, blkq, blkk, flags, mask_lo, mask_hi, _p(addmask)), "sdpa_bf16")
+    return (o16, o32, stats) if want_stats else (o16, o32)
 
 
 def num_threads():

@@ -50,6 +50,28 @@ def test_rms_norm_closed_form_at_scale(oracle, D):
     np.testing.assert_allclose(got, ref, rtol=3e-7, atol=0)
 
 
+def test_sum_of_squares_follows_the_reference_tree(oracle):
+    """serenitymojo/ops/norm.mojo:56-72 folds a 256-slot array in halves, far pairs first.  With
+    x[0]^2 = 2^24 and 127 ones that order keeps 126 of the 127 ones (only the first partner,
+    x[64]^2, is lost to a tie), a left-to-right sum keeps none, and runs of 8 combined
+    neighbours-first keep 120 — so the result tells the orders apart."""
+    x = np.ones((1, 128), np.float32)
+    x[0, 0] = 4096.0
+    ss = np.float32(2.0 ** 24 + 126.0)
+    inv = np.float32(1.0) / np.sqrt(np.float32(ss / np.float32(128.0)) + np.float32(0.0))
+    got = oracle.rms_norm_f32(x, np.ones(128, np.float32), 0.0)
+    assert got[0, 1] == np.float32(inv) and got[0, 0] == np.float32(np.float32(4096.0) * inv)
+    for wrong in (2.0 ** 24, 2.0 ** 24 + 120.0):
+        bad = np.float32(1.0) / np.sqrt(np.float32(np.float32(wrong) / np.float32(128.0)))
+        assert got[0, 1] != bad
+    # D = 64: slots 64..255 are zero, the first real fold is x[t]^2 + x[t+32]^2
+    x64 = np.ones((1, 64), np.float32)
+    x64[0, 0] = 4096.0
+    ss64 = np.float32(2.0 ** 24 + 62.0)
+    inv64 = np.float32(1.0) / np.sqrt(np.float32(ss64 / np.float32(64.0)))
+    assert oracle.rms_norm_f32(x64, np.ones(64, np.float32), 0.0)[0, 1] == inv64
+
+
 def test_properties(oracle):
     rng = np.random.default_rng(5)
     x = rng.standard_normal((7, 128)).astype(np.float32)

@@ -96,6 +96,72 @@ def test_quant_k_smoothed_matches_numpy_on_workload_stats(oracle, wid):
         assert ks.mean() < 0.6 * ks_raw.mean()
 
 
+@pytest.mark.parametrize("smooth,balance", [(True, True), (False, True), (True, False), (False, False)])
+@pytest.mark.parametrize("S,mask", [(320, (0, 0)), (300, (40, 200)), (130, (64, 128)), (200, (150, 200))])
+def test_kstats_and_balanced_quantizers_match_numpy(oracle, smooth, balance, S, mask):
+    """Per-channel statistics (mean, balancing factor) and the Q / K codes they lead to, against
+    the numpy restatement (exact mean by math.fsum, numpy's correctly rounded sqrt and divide)."""
+    w = WORKLOADS[3].scaled(B=1, H=2, S=S)               # two K channels of each head carry 8x the range
+    q, k, _ = make_inputs(w)
+    flags = (1 if smooth else 0) | (2 if balance else 0)
+    mu, qmul, kmul = oracle.kstats(k, w.scale, flags, *mask)
+    mu_n, qmul_n, kmul_n = R.kstats(k, w.scale, smooth, balance, *mask)
+    np.testing.assert_array_equal(mu, mu_n)
+    np.testing.assert_array_equal(qmul, qmul_n)
+    np.testing.assert_array_equal(kmul, kmul_n)
+    k8, ks = oracle.quant_k_ch(k, mu, kmul, w.blkk, 128, *mask)
+    k8n, ksn = R.quant_k(k, mu_n, w.blkk, 128, kmul_n, *mask)
+    np.testing.assert_array_equal(ks, ksn)
+    np.testing.assert_array_equal(k8, k8n)
+    q8, qs = oracle.quant_q_ch(q, w.scale, qmul, w.blkq, 256)
+    q8n, qsn = R.quant_q_ch(q, qmul_n, w.blkq, 256)
+    np.testing.assert_array_equal(qs, qsn)
+    np.testing.assert_array_equal(q8, q8n)
+    if mask[1] > mask[0]:
+        assert not k8[:, :, mask[0]:mask[1]].any()       # masked keys carry code 0
+
+
+def test_kstats_closed_forms(oracle):
+    """What the balancing factor is, independent of any restatement: s_d^2 is the channel's
+    largest |k - mean|; qmul * kmul is c up to the two roundings; with both flags clear the
+    multipliers are exactly (c, 1) and the mean 0; the balanced channels all have the same
+    largest magnitude sqrt(amax) on the K side; and the scores q.k are unchanged."""
+    w = WORKLOADS[3].scaled(B=1, H=2, S=256)
+    q, k, _ = make_inputs(w)
+    c = np.float32(np.float64(np.float32(w.scale)) * R.LOG2E)
+    mu0, qm0, km0 = oracle.kstats(k, w.scale, 0)
+    assert not mu0.any() and np.all(qm0 == c) and np.all(km0 == 1.0)
+    mu, qm, km = oracle.kstats(k, w.scale, 3)
+    x = R.bf16_to_f32(k).transpose(0, 2, 1, 3)
+    amax = np.abs((x - mu[:, :, None, :]).astype(np.float32)).max(axis=2)
+    sd = qm / c
+    np.testing.assert_allclose(sd.astype(np.float64) ** 2, amax, rtol=3e-7)
+    np.testing.assert_allclose(qm.astype(np.float64) * km, c, rtol=2e-7)
+    # the two outlier channels of each head get a factor ~sqrt(8) above the rest
+    ratio = np.sort(sd, axis=-1)
+    assert np.all(ratio[..., -2] > 2.0 * ratio[..., -3]) and np.all(ratio[..., -3] < 1.5 * ratio[..., 0])
+    kb = ((x - mu[:, :, None, :]).astype(np.float32) * km[:, :, None, :]).astype(np.float32)
+    np.testing.assert_allclose(np.abs(kb).max(axis=2), np.sqrt(amax), rtol=3e-7)
+    qb = R.bf16_to_f32(q).transpose(0, 2, 1, 3) * qm[:, :, None, :]
+    s_bal = np.einsum("bhid,bhjd->bhij", qb.astype(np.float64), kb.astype(np.float64))
+    s_raw = np.einsum("bhid,bhjd->bhij", (R.bf16_to_f32(q).transpose(0, 2, 1, 3) * c).astype(np.float64),
+                      (x - mu[:, :, None, :]).astype(np.float64))
+    np.testing.assert_allclose(s_bal, s_raw, atol=2e-5)
+    # a constant channel has nothing to balance: factor 1
+    k2 = k.copy()
+    k2[:, :, 0, 7] = k2[0, 0, 0, 7]
+    _, qm2, km2 = oracle.kstats(k2, w.scale, 3)
+    assert np.all(km2[:, 0, 7] == 1.0) and np.all(qm2[:, 0, 7] == c)
+    # masked keys do not influence the statistics
+    k3 = k.copy()
+    k3[:, 100:180] = f32_to_bf16_bits(np.full((1, 80, 2, w.D), 1000.0, np.float32))
+    a = oracle.kstats(k, w.scale, 3, 100, 180)
+    b = oracle.kstats(k3, w.scale, 3, 100, 180)
+    for u, v in zip(a, b):
+        np.testing.assert_array_equal(u, v)
+    assert oracle.lib().sage_oracle_kstats(None, 1, 1, 1, 1, None, 1.0, 0, 0, 0, None, None, None) == -1
+
+
 def test_quant_v(oracle):
     rng = np.random.default_rng(13)
     v = _rand_bits(rng, (2, 150, 3, 32), std=3.0)
@@ -110,6 +176,14 @@ def test_quant_v(oracle):
     # the channel absmax maps to +-448 exactly
     dec = oracle.e4m3_to_f32(v8)
     assert np.all(np.abs(dec[:, :, :150]).max(axis=2)[vs != 1.0] == 448.0)
+    # channel maximum over the kept keys only; a masked row beyond it saturates
+    v[:, 20:40] = f32_to_bf16_bits(np.full((2, 20, 3, 32), 50.0, np.float32))
+    v8m, vsm = oracle.quant_v_fp8(v, 64, 20, 40)
+    v8mn, vsmn = R.quant_v_fp8(v, 64, 20, 40)
+    np.testing.assert_array_equal(vsm, vsmn)
+    np.testing.assert_array_equal(v8m, v8mn)
+    np.testing.assert_array_equal(vsm, oracle.quant_v_fp8(np.delete(v, np.s_[20:40], axis=1), 64)[1])
+    assert np.all(oracle.e4m3_to_f32(v8m[:, :, 20:40])[(vsm != 1.0)[:, :, None, :].repeat(20, 2)] == 448.0)
 
 
 def test_bad_args(oracle):
