@@ -31,6 +31,7 @@ METRIC = "effective attention TOPS at H=24,S=4608,D=128; % of INT8/FP8 MFMA peak
 PEAK_INT8_TOPS = 5000.0      # MI355X dense INT8 MFMA, published
 PEAK_FP8_TOPS = 5000.0       # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0
+K_FLAGS = 3                  # K mean smoothing + per-channel Q/K balancing (the default recipe)
 
 # HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
 # (KiB per dispatch, one run each) scaled by the readings of the same counters for a 256 MiB
@@ -89,7 +90,7 @@ def main():
     def step():
         rc = L.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
                                        B, H, S, S, D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, stream,
-                                       w.variant, w.blkq, w.blkk, 1, ws.data_ptr(), nws)
+                                       w.variant, w.blkq, w.blkk, K_FLAGS, ws.data_ptr(), nws)
         if rc != 0:
             raise RuntimeError("mi355_sage_sdpa_bf16_ex rc=%d" % rc)
 
@@ -110,25 +111,27 @@ def main():
     k8 = torch.empty((B, H, nkp, D), dtype=torch.int8, device=dev)
     qs = torch.empty((B, H, nqp // w.blkq), dtype=torch.float32, device=dev)
     ks = torch.empty((B, H, nkp // w.blkk), dtype=torch.float32, device=dev)
-    km = torch.empty((B, H, D), dtype=torch.float32, device=dev)
+    km, qm, kmu = (torch.empty((B, H, D), dtype=torch.float32, device=dev) for _ in range(3))
     vsc = torch.empty((B, H, D), dtype=torch.float32, device=dev)
     vq = torch.empty((B, H, nkp // 64, D, 64), dtype=torch.int16 if w.variant == 0 else torch.uint8, device=dev)
     scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, H, S, D), 8), dtype=torch.uint8, device=dev)
 
     def stage_quant_qk():
         return L.mi355_sage_quant_qk_bf16(qd.data_ptr(), kd.data_ptr(), B, H, S, S, D, w.scale, st, st, 0, 0,
-                                          w.blkq, w.blkk, 1, q8.data_ptr(), qs.data_ptr(), k8.data_ptr(),
-                                          ks.data_ptr(), km.data_ptr(), scr.data_ptr(), scr.numel(), stream)
+                                          w.blkq, w.blkk, K_FLAGS, 0, 0, q8.data_ptr(), qs.data_ptr(), k8.data_ptr(),
+                                          ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
+                                          scr.data_ptr(), scr.numel(), stream)
 
     def stage_quant_v():
         if w.variant == 0:
-            return L.mi355_sage_quant_v_f16(vd.data_ptr(), B, H, S, D, st, 0, vq.data_ptr(), stream)
-        return L.mi355_sage_quant_v_fp8(vd.data_ptr(), B, H, S, D, st, 0, vq.data_ptr(), vsc.data_ptr(), stream)
+            return L.mi355_sage_quant_v_f16(vd.data_ptr(), B, H, S, D, st, 0, 0, 0, vq.data_ptr(), stream)
+        return L.mi355_sage_quant_v_fp8(vd.data_ptr(), B, H, S, D, st, 0, 0, 0, vq.data_ptr(), vsc.data_ptr(),
+                                        scr.data_ptr(), scr.numel(), stream)
 
     def stage_attn():
         return L.mi355_sage_attn_fwd(q8.data_ptr(), qs.data_ptr(), w.blkq, k8.data_ptr(), ks.data_ptr(), w.blkk,
-                                     vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, D,
-                                     o.data_ptr(), st, 0, None, stream)
+                                     vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, 0, 0, D,
+                                     o.data_ptr(), st, 0, None, None, stream)
 
     def time_stage(fn, n):
         assert fn() == 0
@@ -169,7 +172,7 @@ def main():
         "config": {
             "workload": w.name,
             "B": B, "H": H, "S": S, "D": D,
-            "recipe": "K mean-smoothed; Q int8 per %d tokens; K int8 per %d tokens; PV %s" % (
+            "recipe": "K mean-smoothed, Q/K channel-balanced; Q int8 per %d tokens; K int8 per %d tokens; PV %s" % (
                 w.blkq, w.blkk, "fp16" if w.variant == 0 else "fp8-e4m3 with per-channel V scales"),
             "ops_per_step": w.ops,
             "pct_of_peak": round(100.0 * tops / peak, 2),

@@ -5,7 +5,7 @@
  * The library sits behind the same seam as the reference's native attention
  * shim: raw device pointers, dims, four ELEMENT strides per tensor describing
  * the memory as logical [B, H, N, D], element offsets, a stream, an int return
- * code.  Work is enqueued on the caller's stream; no call synchronizes.
+ * code.  Work is enqueued on the caller's stream; no call waits for the device.
  *
  * Conventions shared by every entry point
  *   - tensors are caller-allocated device memory; stride arrays are host
@@ -14,8 +14,8 @@
  *   - q/k/v/o are bf16; the innermost (D) stride must be 1 and every row start
  *     must be 16-byte aligned (callers hand out 16-byte-aligned scratch views,
  *     serenitymojo/scratch_ring.mojo:49);
- *   - D is 64 or 128; attention is full, non-causal, unmasked; N_q may differ
- *     from N_kv;
+ *   - D is 64 or 128; attention is full and non-causal; trailing keys (real_N_kv) or one
+ *     range of keys (_keymask) can be masked; N_q may differ from N_kv;
  *   - return 0 on success; -1 for a null pointer, a non-positive dimension or
  *     null strides (serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393); -2 for an
  *     unsupported configuration; -3 for a workspace that is too small; a
@@ -41,21 +41,30 @@ extern "C" {
 #define MI355_SAGE_PV_FP16 0   /* INT8 QK^T, FP16 P*V              */
 #define MI355_SAGE_PV_FP8  1   /* INT8 QK^T, FP8-e4m3 P*V, per-channel V scales */
 
+/* Quantization recipe flags (k_flags). */
+#define MI355_SAGE_K_SMOOTH  1   /* subtract the per-channel mean of K over the keys          */
+#define MI355_SAGE_K_BALANCE 2   /* per channel d: K / s_d, Q * s_d with s_d = sqrt(max|K - mean|)
+                                    over the keys: scores are unchanged, and a channel whose
+                                    range is r times the others' costs each side sqrt(r), not
+                                    one side r, of its INT8 resolution                         */
+
 /* ------------------------------------------------------------------------
  * One-shot drop-in.
  * Replaces flame_cudnn_sdpa_bf16 (serenitymojo/ops/cshim/cudnn_sdpa.cpp:375-387):
  * the parameter list up to `stream` is identical; `variant`, `workspace` and
- * `workspace_bytes` are appended.  Quantizes Q/K (K mean-smoothed, Q in
- * 128-token blocks for variant 0 and 32-token blocks for variant 1, K in
- * 64-token blocks), repacks or quantizes V, runs the attention kernel and
- * writes bf16 O in the caller's strides.
+ * `workspace_bytes` are appended.  Quantizes Q/K (K mean-smoothed, Q and K
+ * channel-balanced, Q in 128-token blocks for variant 0 and 32-token blocks for
+ * variant 1, K in 64-token blocks), repacks or quantizes V, runs the attention
+ * kernel and writes bf16 O in the caller's strides.
  *
- * workspace == NULL: the library keeps one internal device buffer per device,
- * grown on demand (the counterpart of the reference shim's lazily allocated,
- * never-freed workspace, cudnn_sdpa.cpp:218-231); a call that does not grow it
- * allocates nothing.  Otherwise workspace_bytes must be at least
- * mi355_sage_workspace_bytes(...) and the pointer 256-byte aligned.
- * `causal` must be 0.
+ * workspace == NULL: the library keeps one internal device buffer per (device,
+ * stream), grown on demand and never freed (the counterpart of the reference
+ * shim's lazily allocated, never-freed workspace, cudnn_sdpa.cpp:218-231); a call
+ * that does not grow it allocates nothing, and a call that would have to grow it
+ * while its stream is being captured into a graph returns -3.  Otherwise
+ * workspace_bytes must be at least mi355_sage_workspace_bytes(...) and the
+ * pointer 256-byte aligned; calls that share one workspace must be ordered on one
+ * stream.  `causal` must be 0.
  * ---------------------------------------------------------------------- */
 int mi355_sage_sdpa_bf16(
     const void* Q, const void* K, const void* V, void* O,
@@ -70,7 +79,8 @@ int mi355_sage_sdpa_bf16(
     int variant, void* workspace, size_t workspace_bytes);
 
 /* Same with the quantization recipe spelled out: blkq / blkk = tokens per Q / K
- * scale block (32, 64 or 128 each), smooth_k 0/1. */
+ * scale block (32, 64 or 128 each), k_flags = MI355_SAGE_K_SMOOTH | MI355_SAGE_K_BALANCE
+ * or a subset. */
 int mi355_sage_sdpa_bf16_ex(
     const void* Q, const void* K, const void* V, void* O,
     int B, int H, int N_q, int N_kv, int D,
@@ -81,7 +91,7 @@ int mi355_sage_sdpa_bf16_ex(
     int64_t v_offset_elems, int64_t o_offset_elems,
     int causal,
     void* stream,
-    int variant, int blkq, int blkk, int smooth_k,
+    int variant, int blkq, int blkk, int k_flags,
     void* workspace, size_t workspace_bytes);
 
 /* mi355_sage_sdpa_bf16_ex on the PRE-norm projections: Q and K rows are RMS-normalised with
@@ -89,7 +99,8 @@ int mi355_sage_sdpa_bf16_ex(
  * calls rms_norm / rope_interleaved / sdpa of serenitymojo/models/klein/single_block.mojo:977-982
  * in one, with the arithmetic of serenitymojo/ops/norm.mojo:81-114 and ops/rope.mojo:104-122
  * (bf16 stores between the steps included).  Arguments of the fused ops as in
- * mi355_sage_quant_qk_norm_rope_bf16.  V is used as it is. */
+ * mi355_sage_quant_qk_norm_rope_bf16.  V is used as it is.  With tables N_q must equal N_kv
+ * (one table row per position, shared by Q and K); otherwise -2. */
 int mi355_sage_sdpa_bf16_norm_rope(
     const void* Q, const void* K, const void* V, void* O,
     int B, int H, int N_q, int N_kv, int D,
@@ -100,7 +111,7 @@ int mi355_sage_sdpa_bf16_norm_rope(
     int64_t v_offset_elems, int64_t o_offset_elems,
     int causal,
     void* stream,
-    int variant, int blkq, int blkk, int smooth_k,
+    int variant, int blkq, int blkk, int k_flags,
     const void* q_gain, const void* k_gain, float eps,
     const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
     void* workspace, size_t workspace_bytes);
@@ -126,8 +137,27 @@ int mi355_sage_sdpa_bf16_train_fwd(
     void* stream,
     int variant, void* workspace, size_t workspace_bytes);
 
+/* Joint text + image attention with padded text keys masked: replaces sdpa_qwen_keymask
+ * (serenitymojo/ops/attention.mojo:1790-1857, kernel :804-870), which keeps the text keys
+ * [0, real_txt_len), masks [real_txt_len, N_TXT) and keeps the image keys [N_TXT, S): pass
+ * mask_lo = real_txt_len, mask_hi = N_TXT (0 <= mask_lo <= mask_hi <= N_kv; equal = no mask).
+ * Masked keys are left out of the scores, of the K statistics and scale blocks, and of the V
+ * scales.  Stats may be NULL.  Default recipe of mi355_sage_sdpa_bf16. */
+int mi355_sage_sdpa_bf16_keymask(
+    const void* Q, const void* K, const void* V, void* O, void* Stats,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems,
+    int64_t stats_offset_elems,
+    int mask_lo, int mask_hi,
+    void* stream,
+    int variant, void* workspace, size_t workspace_bytes);
+
 /* mi355_sage_sdpa_bf16_train_fwd on the pre-norm projections (default recipe: Q blocks of 128
- * tokens, 32 for the e4m3 variant; K blocks of 64; K smoothing on), for the blocks that run
+ * tokens, 32 for the e4m3 variant; K blocks of 64; K smoothing and balancing on), for the blocks that run
  * rms_norm / rope_interleaved in front of sdpa_flash_train_fwd
  * (serenitymojo/models/klein/single_block.mojo:977-982 with the flash arm of :102).  Stats is the
  * log-sum-exp of the scores of the normalised, rotated Q and K. */
@@ -158,44 +188,50 @@ size_t mi355_sage_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int va
  * Quantized tensor layouts (device memory, caller-allocated):
  *   q8      int8  [B, H, pad_q(N_q),  D]   pad rows are 0
  *   qscale  fp32  [B, H, pad_q(N_q)/blkq]  pad blocks are 1.0
- *   k8      int8  [B, H, pad_kv(N_kv), D]
+ *   k8      int8  [B, H, pad_kv(N_kv), D]   pad rows and masked keys are 0
  *   kscale  fp32  [B, H, pad_kv(N_kv)/blkk]
- *   kmean   fp32  [B, H, D]
+ *   kmean, qmul, kmul  fp32 [B, H, D]       per-channel mean of K (0 without smoothing) and
+ *                                           the multipliers of Q and K (scale*log2(e) and 1
+ *                                           without balancing)
  *   v16     fp16  [B, H, pad_kv/64, D, 64]  64-key tiles, channel-major inside a
  *                                           tile, key k of a tile stored at slot
- *                                           mi355_sage_v_slot(k, PV_FP16)
+ *                                           mi355_sage_v_slot(k, PV_FP16); masked keys 0
  *   v8      e4m3  [B, H, pad_kv/64, D, 64]  same with mi355_sage_v_slot(k, PV_FP8)
  *   vscale  fp32  [B, H, D]
+ * mask_lo / mask_hi: keys mask_lo <= s < mask_hi take no part (0, 0 = none).
  * ---------------------------------------------------------------------- */
 int64_t mi355_sage_pad_q(int64_t n);    /* query tokens round up to the query tile  */
 int64_t mi355_sage_pad_kv(int64_t n);   /* key tokens round up to 128               */
 int     mi355_sage_v_slot(int key_in_tile, int variant);
 
-/* Bytes of scratch mi355_sage_quant_qk_bf16 / _quant_v_fp8 need (partial sums). */
+/* Bytes of scratch mi355_sage_quant_qk_bf16 / _quant_v_fp8 need (per-group partial results). */
 size_t mi355_sage_quant_scratch_bytes(int B, int H, int N_kv, int D);
 
-/* Q: x = f32(q) * fp32(scale*log2(e));  K: x = f32(k) - kmean (if smooth_k).
+/* Per channel over the kept keys: mean (K_SMOOTH), s_d = sqrt(max|f32(k) - mean|) (K_BALANCE;
+ * 1 when that maximum is 0), kmul = 1/s_d, qmul = fp32(scale*log2(e)) * s_d.
+ * Q: x = f32(q) * qmul;  K: x = (f32(k) - kmean) * kmul.
  * Per block: amax -> s = amax/127 (1.0 when 0) -> code = clamp(rne(x/s), +-127).
- * kmean is written when smooth_k != 0 (pass NULL otherwise). */
+ * kmean, qmul and kmul are always written. */
 int mi355_sage_quant_qk_bf16(
     const void* Q, const void* K,
     int B, int H, int N_q, int N_kv, int D, float scale,
     const int64_t* q_strides, const int64_t* k_strides,
     int64_t q_offset_elems, int64_t k_offset_elems,
-    int blkq, int blkk, int smooth_k,
-    void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+    int blkq, int blkk, int k_flags, int mask_lo, int mask_hi,
+    void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
     void* scratch, size_t scratch_bytes, void* stream);
 
 /* The same with the two ops the callers run in front of attention fused in: every Q and K row
  * goes through RMSNorm over D with a bf16 gain (serenitymojo/ops/norm.mojo:81-114,
- * out = bf16(x * 1/sqrt(mean(x^2)+eps) * g)) and, when tables are given, interleaved RoPE with
- * fp32 tables (serenitymojo/ops/rope.mojo:104-122, pairs (2i, 2i+1), result bf16) before it is
- * quantized — the call order of serenitymojo/models/klein/single_block.mojo:977-981, without
- * the two bf16 round trips through memory.  q_gain, k_gain: bf16 [D].  rope_cos / rope_sin:
- * fp32 [rows, D/2], row = n*H + h (serenitymojo/sampling/klein_sampler.mojo:305-307), batch b
- * starting at row b*rope_batch_rows (0 = one table for all batches); both NULL = norm only.
- * Q rows and K rows use the same table (self-attention positions).  Gains and tables must be
- * 16-byte aligned. */
+ * out = bf16(x * 1/sqrt(mean(x^2)+eps) * g), squares added in the order of norm.mojo:56-72) and,
+ * when tables are given, interleaved RoPE with fp32 tables (serenitymojo/ops/rope.mojo:104-122,
+ * pairs (2i, 2i+1), result bf16) before it is quantized — the call order of
+ * serenitymojo/models/klein/single_block.mojo:977-981, without the two bf16 round trips through
+ * memory.  q_gain, k_gain: bf16 [D].  rope_cos / rope_sin: fp32 [rows, D/2], row = n*H + h
+ * (serenitymojo/sampling/klein_sampler.mojo:305-307), batch b starting at row
+ * b*rope_batch_rows (0 = one table for all batches); both NULL = norm only.  Q rows and K rows
+ * use the same table (self-attention positions), so with tables N_q must equal N_kv (-2
+ * otherwise).  Gains and tables must be 16-byte aligned. */
 int mi355_sage_quant_qk_norm_rope_bf16(
     const void* Q, const void* K,
     int B, int H, int N_q, int N_kv, int D, float scale,
@@ -203,31 +239,33 @@ int mi355_sage_quant_qk_norm_rope_bf16(
     int64_t q_offset_elems, int64_t k_offset_elems,
     const void* q_gain, const void* k_gain, float eps,
     const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
-    int blkq, int blkk, int smooth_k,
-    void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+    int blkq, int blkk, int k_flags,
+    void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
     void* scratch, size_t scratch_bytes, void* stream);
 
 /* V -> fp16 (round-to-nearest-even, finite overflow saturates), tiled layout. */
 int mi355_sage_quant_v_f16(
     const void* V, int B, int H, int N_kv, int D,
-    const int64_t* v_strides, int64_t v_offset_elems,
+    const int64_t* v_strides, int64_t v_offset_elems, int mask_lo, int mask_hi,
     void* v16, void* stream);
 
-/* V -> e4m3 with per-(b,h,channel) scale amax/448 (1.0 when 0), tiled layout. */
+/* V -> e4m3 with per-(b,h,channel) scale amax/448 over the kept keys (1.0 when 0), tiled layout. */
 int mi355_sage_quant_v_fp8(
     const void* V, int B, int H, int N_kv, int D,
-    const int64_t* v_strides, int64_t v_offset_elems,
-    void* v8, void* vscale, void* stream);
+    const int64_t* v_strides, int64_t v_offset_elems, int mask_lo, int mask_hi,
+    void* v8, void* vscale, void* scratch, size_t scratch_bytes, void* stream);
 
-/* Attention on the quantized tensors.  stats may be NULL.  kv_valid = number of
- * real keys (<= N_kv); keys beyond it are masked. */
+/* Attention on the quantized tensors.  kv_valid = number of real keys (<= N_kv); keys beyond
+ * it and keys in [mask_lo, mask_hi) are masked.  stats may be NULL; with stats, qshift
+ * ([B,H,pad_q(N_q)] fp32, log2 units, may be NULL) is added to every row's log-sum-exp: the
+ * amount K smoothing lowered that row's scores by. */
 int mi355_sage_attn_fwd(
     const void* q8, const void* qscale, int blkq,
     const void* k8, const void* kscale, int blkk,
     const void* vq, const void* vscale, int variant,
-    int B, int H, int N_q, int N_kv, int kv_valid, int D,
+    int B, int H, int N_q, int N_kv, int kv_valid, int mask_lo, int mask_hi, int D,
     void* O, const int64_t* o_strides, int64_t o_offset_elems,
-    void* stats, void* stream);
+    const void* qshift, void* stats, void* stream);
 
 /* Library identification: "mi355_sage <version> gfx950". */
 const char* mi355_sage_version(void);

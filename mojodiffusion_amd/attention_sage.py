@@ -5,7 +5,7 @@ Function names, argument meaning and error behaviour follow
 serenitymojo/ops/attention_flash.mojo (sdpa_flash_train_fwd :149-202, _rect
 :205-264, sdpa_flash_fwd_padmask :267-342, sdpa_flash_train_fwd_f32 :457-475) and
 serenitymojo/ops/attention.mojo (sdpa_nomask :1690-1718, sdpa_nomask_tiled
-:1762-1787, sdpa_cross_nomask :1860-1894).  Tensors are [B, S, H, Dh]; torch is
+:1762-1787, sdpa_qwen_keymask :1790-1857, sdpa_cross_nomask :1860-1894).  Tensors are [B, S, H, Dh]; torch is
 used only to own device memory and the stream.  What differs from the cuDNN path:
 no 128-padding copies are needed (ragged S is handled in the kernels), so the
 `*_pad` members of the result alias the caller's tensors.
@@ -39,9 +39,12 @@ _workspaces = {}
 
 
 def _workspace(nbytes, device):
-    """Caller-side workspace reuse: one growing buffer per device, so steady-state
-    calls allocate nothing."""
-    key = (device.type, device.index)
+    """Caller-side workspace reuse: one growing buffer per (device, stream), so steady-state
+    calls allocate nothing and calls on different streams never share scratch memory.  A
+    buffer that is replaced stays alive for the work already queued on its stream: torch's
+    allocator hands its memory out again only to that same stream."""
+    stream = torch.cuda.current_stream(device)
+    key = (device.type, device.index, stream.cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -63,7 +66,7 @@ def _require_cuda(name, *ts):
             raise Error("%s: tensors must be contiguous [B,S,H,Dh]" % name)
 
 
-def _call_train_fwd(name, q, k, v, scale, real_q, real_kv, variant, want_stats):
+def _call_train_fwd(name, q, k, v, scale, real_q, real_kv, variant, want_stats, mask=None):
     B, Sq, H, Dh = q.shape
     Skv = k.shape[1]
     L = _lib.lib()
@@ -74,7 +77,12 @@ def _call_train_fwd(name, q, k, v, scale, real_q, real_kv, variant, want_stats):
     qs = _lib.strides_bhnd(Sq, H, Dh)
     ks = _lib.strides_bhnd(Skv, H, Dh)
     stream = torch.cuda.current_stream(q.device).cuda_stream
-    if want_stats:
+    if mask is not None:
+        rc = L.mi355_sage_sdpa_bf16_keymask(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), stats.data_ptr() if want_stats else None,
+            B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, 0, 0, 0, 0, 0,
+            mask[0], mask[1], stream, variant, ws.data_ptr(), ws.numel())
+    elif want_stats:
         rc = L.mi355_sage_sdpa_bf16_train_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), stats.data_ptr(),
             B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, 0, 0, 0, 0, 0,
@@ -159,10 +167,39 @@ def sdpa_nomask(q, k, v, scale, variant=PV_FP16):
     return o.to(q.dtype)
 
 
+def _nomask(name, q, k, v, scale, variant, square, mask=None):
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise Error("%s: q/k/v dtype mismatch" % name)
+    _check_shapes(name, q, k, v, square)
+    _require_cuda(name, q, k, v)
+    if q.dtype == torch.bfloat16:
+        return _call_train_fwd(name, q, k, v, scale, q.shape[1], k.shape[1], variant, False, mask)[0]
+    o = _call_train_fwd(name, q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16),
+                        scale, q.shape[1], k.shape[1], variant, False, mask)[0]
+    return o.to(q.dtype)
+
+
 def sdpa_nomask_tiled(q, k, v, scale, variant=PV_FP16):
     """attention.mojo:1762-1787: the long-sequence entry (video DiTs).  The
-    quantized kernel never materialises scores, so it is the same call."""
-    return sdpa_nomask(q, k, v, scale, variant)
+    quantized kernel never materialises scores, so it is the same kernel."""
+    return _nomask("sdpa_nomask_tiled", q, k, v, scale, variant, True)
+
+
+def sdpa_qwen_keymask(q, k, v, n_txt, real_txt_len, scale, variant=PV_FP16):
+    """attention.mojo:1790-1857: joint attention, tokens ordered TXT then IMG; text keys
+    [0, real_txt_len) and image keys [n_txt, S) are kept, the padded text keys
+    [real_txt_len, n_txt) are masked.  n_txt is the reference's compile-time N_TXT."""
+    if n_txt > q.shape[1] if q.dim() == 4 else False:
+        raise Error("sdpa_qwen_keymask: N_TXT must be <= S")
+    if real_txt_len < 0 or real_txt_len > n_txt:
+        raise Error("sdpa_qwen_keymask: real_txt_len out of range")
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise Error("sdpa_qwen_keymask: q/k/v dtype mismatch")
+    if q.dim() != 4:
+        raise Error("sdpa_qwen_keymask: q must be rank-4 [B,S,H,Dh]")
+    if k.shape != q.shape or v.shape != q.shape:
+        raise Error("sdpa_qwen_keymask: k/v shape mismatch")
+    return _nomask("sdpa_qwen_keymask", q, k, v, scale, variant, True, (real_txt_len, n_txt))
 
 
 def sdpa_cross_nomask(q, k, v, scale, variant=PV_FP16):
@@ -204,7 +241,7 @@ def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin):
 
 
 def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16,
-                             blkq=None, blkk=64, smooth_k=True):
+                             blkq=None, blkk=64, k_flags=_lib.K_SMOOTH | _lib.K_BALANCE):
     """The attention block of a DiT layer from the projections on, in one call:
 
         q = rope_interleaved(rms_norm(q_pre, q_norm, eps), cos, sin)
@@ -228,7 +265,7 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
     rc = L.mi355_sage_sdpa_bf16_norm_rope(
         q_pre.data_ptr(), k_pre.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, S, S, Dh, float(scale),
         st, st, st, st, 0, 0, 0, 0, 0, torch.cuda.current_stream(q_pre.device).cuda_stream,
-        variant, blkq, blkk, int(bool(smooth_k)), gq.data_ptr(), gk.data_ptr(), float(eps),
+        variant, blkq, blkk, int(k_flags), gq.data_ptr(), gk.data_ptr(), float(eps),
         cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
         ws.data_ptr(), ws.numel())
     if rc != 0:

@@ -5,6 +5,7 @@
 
 #include <cstdio>
 #include <mutex>
+#include <vector>
 
 using namespace sage;
 
@@ -62,12 +63,13 @@ int check_kv_len(int N_kv, int blkk) {
 
 // Workspace layout of the one-shot calls.
 struct Carve {
-    size_t q8, k8, vq, qscale, kscale, kmean, vscale, partial, qshift, total;
+    size_t q8, k8, vq, qscale, kscale, kmean, qmul, kmul, vscale, kpart_sum, kpart_mm, vpart, qshift, total;
 };
 
 Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     const size_t bh = (size_t)B * H;
     const size_t nqp = (size_t)pad_to(Nq, kTileQ), nkp = (size_t)pad_to(Nkv, kPadKV);
+    const size_t ng = (size_t)((Nkv + kGroup - 1) / kGroup);
     Carve c{};
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
@@ -77,37 +79,68 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.qscale = take(bh * (nqp / 32) * sizeof(float));      // smallest block is 32 tokens
     c.kscale = take(bh * (nkp / 32) * sizeof(float));
     c.kmean = take(bh * D * sizeof(float));
+    c.qmul = take(bh * D * sizeof(float));
+    c.kmul = take(bh * D * sizeof(float));
     c.vscale = take(bh * D * sizeof(float));
-    c.partial = take(bh * ((Nkv + kGroup - 1) / kGroup) * D * sizeof(double));
+    c.kpart_sum = take(bh * ng * D * sizeof(double));
+    c.kpart_mm = take(bh * ng * D * 2 * sizeof(float));
+    c.vpart = take(variant == MI355_SAGE_PV_FP16 ? 0 : bh * ng * D * sizeof(float));
     c.qshift = take(bh * nqp * sizeof(float));
     c.total = off;
     return c;
 }
 
-// Internal workspace: one buffer per device, grown on demand, never freed
-// while the process lives (same lifetime as the cuDNN shim's per-graph workspace).
-std::mutex g_ws_mutex;
-struct DevWs { void* p = nullptr; size_t bytes = 0; };
-DevWs g_ws[64];
+// Scratch of the stage quantizers: K group sums and minima / maxima, V group maxima.
+struct ScratchCarve {
+    size_t kpart_sum, kpart_mm, vpart, total;
+};
+ScratchCarve scratch_carve(int B, int H, int Nkv, int D) {
+    const size_t n = (size_t)B * H * ((Nkv + kGroup - 1) / kGroup) * D;
+    ScratchCarve c{};
+    c.kpart_sum = 0;
+    c.kpart_mm = align_up(n * sizeof(double));
+    c.vpart = c.kpart_mm + align_up(n * 2 * sizeof(float));
+    c.total = c.vpart + align_up(n * sizeof(float));
+    return c;
+}
 
-int internal_workspace(size_t need, void** out) {
+// Internal workspaces (workspace == NULL): one buffer per (device, stream), so calls on
+// different streams never share one.  A buffer that has become too small is replaced by a
+// larger one and kept allocated until the process ends: work queued earlier may still be
+// using it, and waiting for that work would make the call synchronise.  Sizes at least double,
+// so the retired buffers of a stream add up to less than its current one.  Allocation is not
+// possible while the stream is being captured into a graph: such a call fails with
+// MI355_SAGE_EWORKSPACE unless the buffer is already large enough.
+std::mutex g_ws_mutex;
+struct StreamWs { int dev; hipStream_t stream; void* p; size_t bytes; };
+std::vector<StreamWs> g_ws;
+
+int internal_workspace(size_t need, hipStream_t stream, void** out) {
     int dev = 0;
     SAGE_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64) return MI355_SAGE_EUNSUPPORTED;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    DevWs& w = g_ws[dev];
-    if (w.bytes < need) {
-        // The old buffer may still be in use by work queued earlier; wait before freeing.
-        if (w.p) {
-            SAGE_HIP(hipDeviceSynchronize());
-            SAGE_HIP(hipFree(w.p));
-            w.p = nullptr;
-            w.bytes = 0;
+    StreamWs* w = nullptr;
+    for (auto& e : g_ws)
+        if (e.dev == dev && e.stream == stream) { w = &e; break; }
+    if (w == nullptr || w->bytes < need) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+            SAGE_LOG("the internal workspace would have to grow to %zu bytes while the stream is being captured; "
+                     "pass a workspace or run the call once before capturing", need);
+            return MI355_SAGE_EWORKSPACE;
         }
-        SAGE_HIP(hipMalloc(&w.p, need));
-        w.bytes = need;
+        const size_t bytes = w ? (need > 2 * w->bytes ? need : 2 * w->bytes) : need;
+        void* p = nullptr;
+        SAGE_HIP(hipMalloc(&p, bytes));
+        if (w == nullptr) {
+            g_ws.push_back(StreamWs{dev, stream, p, bytes});
+            w = &g_ws.back();
+        } else {
+            w->p = p;              // the old buffer stays allocated (see above)
+            w->bytes = bytes;
+        }
     }
-    *out = w.p;
+    *out = w->p;
     return 0;
 }
 
@@ -134,25 +167,73 @@ int make_pre(const void* q_gain, const void* k_gain, float eps, const void* rope
     return 0;
 }
 
-int quant_qk(const View& q, const View& k, int B, int H, int Nq, int Nkv, int D, float scale,
-             int blkq, int blkk, int smooth_k, int8_t* q8, float* qscale, int8_t* k8, float* kscale,
-             float* kmean, double* partial, float* qshift, const Pre& pre, hipStream_t st) {
-    const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
-    if (smooth_k) SAGE_HIP(launch_kmean(k, B, H, Nkv, D, partial, kmean, pre.k, st));
-    SAGE_HIP(launch_quant_i8(q, B, H, Nq, D, pad_to(Nq, kTileQ), blkq, false, cmul, kmean, q8, qscale,
-                             smooth_k ? qshift : nullptr, pre.q, st));
-    SAGE_HIP(launch_quant_i8(k, B, H, Nkv, D, pad_to(Nkv, kPadKV), blkk, true, 0.0f,
-                             smooth_k ? kmean : nullptr, k8, kscale, nullptr, pre.k, st));
+float cmul_of(float scale) { return (float)((double)scale * 1.4426950408889634074); }   // scale*log2(e), rounded once
+
+// Clips the masked key range to [0, n) and counts the keys that remain.
+int clip_mask(int n, int mask_lo, int mask_hi, KeyMask* km) {
+    int lo = mask_lo < 0 ? 0 : mask_lo, hi = mask_hi > n ? n : mask_hi;
+    if (hi <= lo) lo = hi = 0;
+    *km = KeyMask{lo, hi};
+    return n - (hi - lo);
+}
+
+struct QuantOut {
+    int8_t* q8; float* qscale; int8_t* k8; float* kscale;
+    float *kmean, *qmul, *kmul;
+    double* kpart_sum; float* kpart_mm;
+    float* rowdot;
+};
+
+// K statistics + Q / K encoders (+ the V passes when vq is given): launches 1-3.
+int quantize(const View& q, const View& k, const View* v, int B, int H, int Nq, int Nkv, int D, float scale,
+             int blkq, int blkk, int k_flags, const KeyMask& km, int kept, const QuantOut& o,
+             int variant, void* vq, float* vscale, float* vpart, const Pre& pre, hipStream_t st) {
+    const float cmul = cmul_of(scale);
+    const int64_t nqp = pad_to(Nq, kTileQ), nkp = pad_to(Nkv, kPadKV);
+    const bool kstats = (k_flags & 3) != 0;
+    PrepArgs p{};
+    p.k = k; p.H = H; p.Nkv = Nkv; p.nkv_pad = nkp; p.km = km; p.pre_k = pre.k;
+    p.vmode = 2;
+    if (v != nullptr) {
+        p.v = *v;
+        p.vmode = variant == MI355_SAGE_PV_FP16 ? 0 : 1;
+        p.v16 = static_cast<uint16_t*>(vq);
+        p.vpart = vpart;
+    }
+    p.kpart_sum = kstats ? o.kpart_sum : nullptr;
+    p.kpart_mm = o.kpart_mm;
+    SAGE_HIP(launch_prep(p, B, D, st));
+
+    FinalArgs f{};
+    f.total = (int64_t)B * H * D; f.D = D; f.ngroups = (Nkv + kGroup - 1) / kGroup; f.kept = kept;
+    f.flags = k_flags; f.cmul = cmul;
+    f.kpart_sum = p.kpart_sum; f.kpart_mm = o.kpart_mm;
+    f.kmean = o.kmean; f.qmul = o.qmul; f.kmul = o.kmul;
+    f.vpart = vpart; f.vscale = p.vmode == 1 ? vscale : nullptr;
+    SAGE_HIP(launch_stats_final(f, st));
+
+    QuantArgs a{};
+    a.q = q; a.k = k; a.H = H; a.Nq = Nq; a.Nkv = Nkv; a.nq_pad = nqp; a.nkv_pad = nkp; a.km = km;
+    a.blkq = blkq; a.blkk = blkk; a.cmul = cmul;
+    a.kmean = o.kmean; a.qmul = o.qmul; a.kmul = o.kmul; a.vscale = vscale;
+    a.q8 = o.q8; a.qscale = o.qscale; a.rowdot = o.rowdot; a.k8 = o.k8; a.kscale = o.kscale;
+    if (p.vmode == 1) { a.v = *v; a.v8 = static_cast<uint8_t*>(vq); }
+    a.pre_q = pre.q; a.pre_k = pre.k;
+    SAGE_HIP(launch_quant(a, B, D, st));
     return 0;
 }
+
+struct MaskArgs {
+    int lo = 0, hi = 0;        // keys lo <= s < hi are masked
+};
 
 int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
               int B, int H, int N_q, int N_kv, int D, float scale,
               const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
               int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t stats_off,
               int causal, int real_N_kv, void* stream,
-              int variant, int blkq, int blkk, int smooth_k, void* workspace, size_t workspace_bytes,
-              const Pre& pre = Pre{}) {
+              int variant, int blkq, int blkk, int k_flags, void* workspace, size_t workspace_bytes,
+              const Pre& pre = Pre{}, const MaskArgs& mask = MaskArgs{}) {
     // argument checks in the order of serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393
     if (!Q || !K || !V || !O) return MI355_SAGE_EINVAL;
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
@@ -161,15 +242,24 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if (!dims_ok(D)) { SAGE_LOG("head dim %d not supported (64 or 128)", D); return MI355_SAGE_EUNSUPPORTED; }
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
     if (!blk_ok(blkq) || !blk_ok(blkk)) { SAGE_LOG("block sizes must be 32, 64 or 128"); return MI355_SAGE_EUNSUPPORTED; }
+    if (k_flags & ~3) return MI355_SAGE_EUNSUPPORTED;
     int rc;
     if ((rc = check_kv_len(N_kv, blkk))) return rc;
     if ((rc = check_view("Q", Q, qs, q_off)) || (rc = check_view("K", K, ks, k_off)) ||
         (rc = check_view("V", V, vs, v_off)) || (rc = check_view("O", O, os, o_off)))
         return rc;
+    if (pre.q.gain != nullptr && pre.q.cos != nullptr && N_q != N_kv) {
+        SAGE_LOG("fused RoPE uses one table row per position of Q and K alike: N_q must equal N_kv");
+        return MI355_SAGE_EUNSUPPORTED;
+    }
     // Keys past the real length are excluded from the statistics and the scores alike:
     // the quantizers see only the first kv tokens.
     const int kv = (real_N_kv > 0 && real_N_kv < N_kv) ? real_N_kv : N_kv;
+    KeyMask km;
+    const int kept = clip_mask(kv, mask.lo, mask.hi, &km);
+    if (kept <= 0) { SAGE_LOG("every key is masked"); return MI355_SAGE_EINVAL; }
 
+    hipStream_t st = static_cast<hipStream_t>(stream);
     const Carve c = carve(B, H, N_q, kv, D, variant);
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     if (ws) {
@@ -180,59 +270,53 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         if (reinterpret_cast<uintptr_t>(ws) & (kAlign - 1)) return MI355_SAGE_EUNSUPPORTED;
     } else {
         void* p = nullptr;
-        if ((rc = internal_workspace(c.total, &p))) return rc;
+        if ((rc = internal_workspace(c.total, st, &p))) return rc;
         ws = static_cast<uint8_t*>(p);
     }
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    int8_t* q8 = reinterpret_cast<int8_t*>(ws + c.q8);
-    int8_t* k8 = reinterpret_cast<int8_t*>(ws + c.k8);
+    QuantOut o{};
+    o.q8 = reinterpret_cast<int8_t*>(ws + c.q8);
+    o.k8 = reinterpret_cast<int8_t*>(ws + c.k8);
+    o.qscale = reinterpret_cast<float*>(ws + c.qscale);
+    o.kscale = reinterpret_cast<float*>(ws + c.kscale);
+    o.kmean = reinterpret_cast<float*>(ws + c.kmean);
+    o.qmul = reinterpret_cast<float*>(ws + c.qmul);
+    o.kmul = reinterpret_cast<float*>(ws + c.kmul);
+    o.kpart_sum = reinterpret_cast<double*>(ws + c.kpart_sum);
+    o.kpart_mm = reinterpret_cast<float*>(ws + c.kpart_mm);
+    // Stats needs <q, kmean> per row: K smoothing lowers every score of a row by it
+    float* qshift = (Stats && (k_flags & MI355_SAGE_K_SMOOTH)) ? reinterpret_cast<float*>(ws + c.qshift) : nullptr;
+    o.rowdot = qshift;
     void* vq = ws + c.vq;
-    float* qscale = reinterpret_cast<float*>(ws + c.qscale);
-    float* kscale = reinterpret_cast<float*>(ws + c.kscale);
-    float* kmean = reinterpret_cast<float*>(ws + c.kmean);
     float* vscale = reinterpret_cast<float*>(ws + c.vscale);
-    double* partial = reinterpret_cast<double*>(ws + c.partial);
-    float* qshift = Stats ? reinterpret_cast<float*>(ws + c.qshift) : nullptr;
+    float* vpart = reinterpret_cast<float*>(ws + c.vpart);
 
     const View q = make_view(Q, qs, q_off), k = make_view(K, ks, k_off), v = make_view(V, vs, v_off);
-    const int64_t nkp = pad_to(kv, kPadKV);
-    if (variant == MI355_SAGE_PV_FP16 && !Stats) {
-        // two launches: {Q quantize, V repack, K-mean group sums} then {K mean + K quantize}
-        const float cmul = (float)((double)scale * 1.4426950408889634074);   // scale*log2(e), rounded once
-        SAGE_HIP(launch_prep_fused(q, k, v, B, H, N_q, kv, D, pad_to(N_q, kTileQ), nkp, cmul, blkq, smooth_k != 0,
-                                   q8, qscale, static_cast<uint16_t*>(vq), partial, pre.q, pre.k, st));
-        SAGE_HIP(launch_kquant_fused(k, B, H, kv, D, nkp, blkk, smooth_k ? partial : nullptr, kmean, k8, kscale,
-                                     pre.k, st));
-    } else {
-        // Stats needs <q, kmean> per row, i.e. the mean before the Q quantizer; the e4m3 V path
-        // has its own three launches
-        if ((rc = quant_qk(q, k, B, H, N_q, kv, D, scale, blkq, blkk, smooth_k, q8, qscale, k8, kscale,
-                           kmean, partial, qshift, pre, st)))
-            return rc;
-        if (variant == MI355_SAGE_PV_FP16)
-            SAGE_HIP(launch_quant_v_f16(v, B, H, kv, D, nkp, static_cast<uint16_t*>(vq), st));
-        else
-            SAGE_HIP(launch_quant_v_fp8(v, B, H, kv, D, nkp, static_cast<uint8_t*>(vq), vscale, st));
-    }
+    if ((rc = quantize(q, k, &v, B, H, N_q, kv, D, scale, blkq, blkk, k_flags, km, kept, o, variant, vq, vscale,
+                       vpart, pre, st)))
+        return rc;
 
     AttnArgs a{};
-    a.q8 = q8; a.qscale = qscale; a.blkq = blkq;
-    a.k8 = k8; a.kscale = kscale; a.blkk = blkk;
-    a.vq = vq; a.vscale = vscale; a.qshift = smooth_k ? qshift : nullptr;
+    a.q8 = o.q8; a.qscale = o.qscale; a.blkq = blkq;
+    a.k8 = o.k8; a.kscale = o.kscale; a.blkk = blkk;
+    a.vq = vq; a.vscale = vscale; a.qshift = qshift;
     a.variant = variant;
+    a.km = km;
     a.B = B; a.H = H; a.Nq = N_q; a.Nkv = kv; a.kv_valid = kv; a.D = D;
-    a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = nkp;
+    a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(kv, kPadKV);
     a.o = static_cast<uint16_t*>(O) + o_off; a.osb = os[0]; a.osh = os[1]; a.osn = os[2];
     a.stats = Stats ? static_cast<float*>(Stats) + stats_off : nullptr;
     SAGE_HIP(launch_attn(a, st));
     return MI355_SAGE_OK;
 }
 
+int default_blkq(int variant) { return variant == MI355_SAGE_PV_FP8 ? 32 : 128; }
+constexpr int kDefaultFlags = MI355_SAGE_K_SMOOTH | MI355_SAGE_K_BALANCE;
+
 }  // namespace
 
 extern "C" {
 
-const char* mi355_sage_version(void) { return "mi355_sage 0.1 gfx950"; }
+const char* mi355_sage_version(void) { return "mi355_sage 0.2 gfx950"; }
 
 int64_t mi355_sage_pad_q(int64_t n) { return pad_to(n, kTileQ); }
 int64_t mi355_sage_pad_kv(int64_t n) { return pad_to(n, kPadKV); }
@@ -250,7 +334,7 @@ size_t mi355_sage_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int va
 
 size_t mi355_sage_quant_scratch_bytes(int B, int H, int N_kv, int D) {
     if (B <= 0 || H <= 0 || N_kv <= 0 || D <= 0) return 0;
-    return align_up((size_t)B * H * ((N_kv + kGroup - 1) / kGroup) * D * sizeof(double));
+    return scratch_carve(B, H, N_kv, D).total;
 }
 
 int mi355_sage_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
@@ -260,10 +344,9 @@ int mi355_sage_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
                          int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
                          int causal, void* stream,
                          int variant, void* workspace, size_t workspace_bytes) {
-    const int blkq = variant == MI355_SAGE_PV_FP8 ? 32 : 128;
     return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
-                     o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, blkq, 64, 1,
-                     workspace, workspace_bytes);
+                     o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, default_blkq(variant), 64,
+                     kDefaultFlags, workspace, workspace_bytes);
 }
 
 int mi355_sage_sdpa_bf16_ex(const void* Q, const void* K, const void* V, void* O,
@@ -272,11 +355,11 @@ int mi355_sage_sdpa_bf16_ex(const void* Q, const void* K, const void* V, void* O
                             const int64_t* v_strides, const int64_t* o_strides,
                             int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
                             int causal, void* stream,
-                            int variant, int blkq, int blkk, int smooth_k,
+                            int variant, int blkq, int blkk, int k_flags,
                             void* workspace, size_t workspace_bytes) {
     return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, blkq, blkk,
-                     smooth_k ? 1 : 0, workspace, workspace_bytes);
+                     k_flags, workspace, workspace_bytes);
 }
 
 int mi355_sage_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V, void* O, void* Stats,
@@ -288,29 +371,65 @@ int mi355_sage_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V, 
                                    void* stream, int variant, void* workspace, size_t workspace_bytes) {
     if (!Stats) return MI355_SAGE_EINVAL;              // cudnn_sdpa.cpp:485
     (void)real_N_q;                                    // padded query rows are computed and ignored
-    const int blkq = variant == MI355_SAGE_PV_FP8 ? 32 : 128;
     return sdpa_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, stats_off, causal, real_N_kv, stream, variant,
-                     blkq, 64, 1, workspace, workspace_bytes);
+                     default_blkq(variant), 64, kDefaultFlags, workspace, workspace_bytes);
+}
+
+int mi355_sage_sdpa_bf16_keymask(const void* Q, const void* K, const void* V, void* O, void* Stats,
+                                 int B, int H, int N_q, int N_kv, int D, float scale,
+                                 const int64_t* q_strides, const int64_t* k_strides,
+                                 const int64_t* v_strides, const int64_t* o_strides,
+                                 int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
+                                 int64_t stats_off, int mask_lo, int mask_hi,
+                                 void* stream, int variant, void* workspace, size_t workspace_bytes) {
+    if (mask_lo < 0 || mask_hi < mask_lo || mask_hi > N_kv) return MI355_SAGE_EINVAL;
+    MaskArgs m;
+    m.lo = mask_lo; m.hi = mask_hi;
+    return sdpa_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                     o_strides, q_off, k_off, v_off, o_off, stats_off, 0, 0, stream, variant,
+                     default_blkq(variant), 64, kDefaultFlags, workspace, workspace_bytes, Pre{}, m);
+}
+
+static int quant_qk_entry(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
+                          float scale, const int64_t* q_strides, const int64_t* k_strides,
+                          int64_t q_off, int64_t k_off, const Pre& pre, int blkq, int blkk, int k_flags,
+                          int mask_lo, int mask_hi,
+                          void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
+                          void* scratch, size_t scratch_bytes, void* stream) {
+    if (!Q || !K || !q8 || !qscale || !k8 || !kscale || !kmean || !qmul || !kmul) return MI355_SAGE_EINVAL;
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
+    if (!q_strides || !k_strides) return MI355_SAGE_EINVAL;
+    if ((k_flags & 3) && !scratch) return MI355_SAGE_EINVAL;
+    if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk) || (k_flags & ~3)) return MI355_SAGE_EUNSUPPORTED;
+    const ScratchCarve sc = scratch_carve(B, H, N_kv, D);
+    if ((k_flags & 3) && scratch_bytes < sc.total) return MI355_SAGE_EWORKSPACE;
+    if (pre.q.gain != nullptr && pre.q.cos != nullptr && N_q != N_kv) return MI355_SAGE_EUNSUPPORTED;
+    int rc;
+    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off))) return rc;
+    KeyMask km;
+    const int kept = clip_mask(N_kv, mask_lo, mask_hi, &km);
+    if (kept <= 0) return MI355_SAGE_EINVAL;
+    QuantOut o{};
+    o.q8 = static_cast<int8_t*>(q8); o.qscale = static_cast<float*>(qscale);
+    o.k8 = static_cast<int8_t*>(k8); o.kscale = static_cast<float*>(kscale);
+    o.kmean = static_cast<float*>(kmean); o.qmul = static_cast<float*>(qmul); o.kmul = static_cast<float*>(kmul);
+    o.kpart_sum = reinterpret_cast<double*>(static_cast<uint8_t*>(scratch) + sc.kpart_sum);
+    o.kpart_mm = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + sc.kpart_mm);
+    return quantize(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), nullptr, B, H, N_q, N_kv, D,
+                    scale, blkq, blkk, k_flags, km, kept, o, 0, nullptr, nullptr, nullptr, pre,
+                    static_cast<hipStream_t>(stream));
 }
 
 int mi355_sage_quant_qk_bf16(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
                              float scale, const int64_t* q_strides, const int64_t* k_strides,
-                             int64_t q_off, int64_t k_off, int blkq, int blkk, int smooth_k,
-                             void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+                             int64_t q_off, int64_t k_off, int blkq, int blkk, int k_flags,
+                             int mask_lo, int mask_hi,
+                             void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
                              void* scratch, size_t scratch_bytes, void* stream) {
-    if (!Q || !K || !q8 || !qscale || !k8 || !kscale) return MI355_SAGE_EINVAL;
-    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
-    if (!q_strides || !k_strides) return MI355_SAGE_EINVAL;
-    if (smooth_k && (!kmean || !scratch)) return MI355_SAGE_EINVAL;
-    if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk)) return MI355_SAGE_EUNSUPPORTED;
-    if (smooth_k && scratch_bytes < mi355_sage_quant_scratch_bytes(B, H, N_kv, D)) return MI355_SAGE_EWORKSPACE;
-    int rc;
-    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off))) return rc;
-    return quant_qk(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), B, H, N_q, N_kv, D,
-                    scale, blkq, blkk, smooth_k, static_cast<int8_t*>(q8), static_cast<float*>(qscale),
-                    static_cast<int8_t*>(k8), static_cast<float*>(kscale), static_cast<float*>(kmean),
-                    static_cast<double*>(scratch), nullptr, Pre{}, static_cast<hipStream_t>(stream));
+    return quant_qk_entry(Q, K, B, H, N_q, N_kv, D, scale, q_strides, k_strides, q_off, k_off, Pre{}, blkq, blkk,
+                          k_flags, mask_lo, mask_hi, q8, qscale, k8, kscale, kmean, qmul, kmul, scratch,
+                          scratch_bytes, stream);
 }
 
 int mi355_sage_quant_qk_norm_rope_bf16(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
@@ -318,24 +437,16 @@ int mi355_sage_quant_qk_norm_rope_bf16(const void* Q, const void* K, int B, int 
                                        int64_t q_off, int64_t k_off,
                                        const void* q_gain, const void* k_gain, float eps,
                                        const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
-                                       int blkq, int blkk, int smooth_k,
-                                       void* q8, void* qscale, void* k8, void* kscale, void* kmean,
+                                       int blkq, int blkk, int k_flags,
+                                       void* q8, void* qscale, void* k8, void* kscale,
+                                       void* kmean, void* qmul, void* kmul,
                                        void* scratch, size_t scratch_bytes, void* stream) {
-    if (!Q || !K || !q8 || !qscale || !k8 || !kscale) return MI355_SAGE_EINVAL;
-    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
-    if (!q_strides || !k_strides) return MI355_SAGE_EINVAL;
-    if (smooth_k && (!kmean || !scratch)) return MI355_SAGE_EINVAL;
-    if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk)) return MI355_SAGE_EUNSUPPORTED;
-    if (smooth_k && scratch_bytes < mi355_sage_quant_scratch_bytes(B, H, N_kv, D)) return MI355_SAGE_EWORKSPACE;
-    int rc;
-    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off))) return rc;
     Pre pre;
+    int rc;
     if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
     if (!pre.q.gain) return MI355_SAGE_EINVAL;
-    return quant_qk(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), B, H, N_q, N_kv, D,
-                    scale, blkq, blkk, smooth_k, static_cast<int8_t*>(q8), static_cast<float*>(qscale),
-                    static_cast<int8_t*>(k8), static_cast<float*>(kscale), static_cast<float*>(kmean),
-                    static_cast<double*>(scratch), nullptr, pre, static_cast<hipStream_t>(stream));
+    return quant_qk_entry(Q, K, B, H, N_q, N_kv, D, scale, q_strides, k_strides, q_off, k_off, pre, blkq, blkk,
+                          k_flags, 0, 0, q8, qscale, k8, kscale, kmean, qmul, kmul, scratch, scratch_bytes, stream);
 }
 
 int mi355_sage_sdpa_bf16_norm_rope(const void* Q, const void* K, const void* V, void* O,
@@ -344,7 +455,7 @@ int mi355_sage_sdpa_bf16_norm_rope(const void* Q, const void* K, const void* V, 
                                    const int64_t* v_strides, const int64_t* o_strides,
                                    int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
                                    int causal, void* stream,
-                                   int variant, int blkq, int blkk, int smooth_k,
+                                   int variant, int blkq, int blkk, int k_flags,
                                    const void* q_gain, const void* k_gain, float eps,
                                    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
                                    void* workspace, size_t workspace_bytes) {
@@ -354,7 +465,7 @@ int mi355_sage_sdpa_bf16_norm_rope(const void* Q, const void* K, const void* V, 
     if (!pre.q.gain) return MI355_SAGE_EINVAL;
     return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, blkq, blkk,
-                     smooth_k ? 1 : 0, workspace, workspace_bytes, pre);
+                     k_flags, workspace, workspace_bytes, pre);
 }
 
 int mi355_sage_sdpa_bf16_norm_rope_train_fwd(const void* Q, const void* K, const void* V, void* O, void* Stats,
@@ -373,41 +484,58 @@ int mi355_sage_sdpa_bf16_norm_rope_train_fwd(const void* Q, const void* K, const
     int rc;
     if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
     if (!pre.q.gain) return MI355_SAGE_EINVAL;
-    const int blkq = variant == MI355_SAGE_PV_FP8 ? 32 : 128;
     return sdpa_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, stats_off, causal, real_N_kv, stream, variant,
-                     blkq, 64, 1, workspace, workspace_bytes, pre);
+                     default_blkq(variant), 64, kDefaultFlags, workspace, workspace_bytes, pre);
 }
 
 int mi355_sage_quant_v_f16(const void* V, int B, int H, int N_kv, int D, const int64_t* v_strides,
-                           int64_t v_off, void* v16, void* stream) {
+                           int64_t v_off, int mask_lo, int mask_hi, void* v16, void* stream) {
     if (!V || !v16 || !v_strides) return MI355_SAGE_EINVAL;
     if (B <= 0 || H <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
     if (!dims_ok(D)) return MI355_SAGE_EUNSUPPORTED;
     int rc;
     if ((rc = check_view("V", V, v_strides, v_off))) return rc;
-    SAGE_HIP(launch_quant_v_f16(make_view(V, v_strides, v_off), B, H, N_kv, D, pad_to(N_kv, kPadKV),
-                                static_cast<uint16_t*>(v16), static_cast<hipStream_t>(stream)));
+    PrepArgs p{};
+    p.v = make_view(V, v_strides, v_off); p.H = H; p.Nkv = N_kv; p.nkv_pad = pad_to(N_kv, kPadKV);
+    clip_mask(N_kv, mask_lo, mask_hi, &p.km);
+    p.vmode = 0; p.v16 = static_cast<uint16_t*>(v16);
+    SAGE_HIP(launch_prep(p, B, D, static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
 }
 
 int mi355_sage_quant_v_fp8(const void* V, int B, int H, int N_kv, int D, const int64_t* v_strides,
-                           int64_t v_off, void* v8, void* vscale, void* stream) {
-    if (!V || !v8 || !vscale || !v_strides) return MI355_SAGE_EINVAL;
+                           int64_t v_off, int mask_lo, int mask_hi, void* v8, void* vscale,
+                           void* scratch, size_t scratch_bytes, void* stream) {
+    if (!V || !v8 || !vscale || !v_strides || !scratch) return MI355_SAGE_EINVAL;
     if (B <= 0 || H <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
     if (!dims_ok(D)) return MI355_SAGE_EUNSUPPORTED;
+    const ScratchCarve sc = scratch_carve(B, H, N_kv, D);
+    if (scratch_bytes < sc.total) return MI355_SAGE_EWORKSPACE;
     int rc;
     if ((rc = check_view("V", V, v_strides, v_off))) return rc;
-    SAGE_HIP(launch_quant_v_fp8(make_view(V, v_strides, v_off), B, H, N_kv, D, pad_to(N_kv, kPadKV),
-                                static_cast<uint8_t*>(v8), static_cast<float*>(vscale),
-                                static_cast<hipStream_t>(stream)));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    PrepArgs p{};
+    p.v = make_view(V, v_strides, v_off); p.H = H; p.Nkv = N_kv; p.nkv_pad = pad_to(N_kv, kPadKV);
+    if (clip_mask(N_kv, mask_lo, mask_hi, &p.km) <= 0) return MI355_SAGE_EINVAL;
+    p.vmode = 1; p.vpart = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + sc.vpart);
+    SAGE_HIP(launch_prep(p, B, D, st));
+    FinalArgs f{};
+    f.total = (int64_t)B * H * D; f.D = D; f.ngroups = (N_kv + kGroup - 1) / kGroup;
+    f.vpart = p.vpart; f.vscale = static_cast<float*>(vscale);
+    SAGE_HIP(launch_stats_final(f, st));
+    QuantArgs a{};
+    a.v = p.v; a.H = H; a.Nkv = N_kv; a.nkv_pad = p.nkv_pad; a.km = p.km; a.blkq = 32; a.blkk = 32;
+    a.vscale = f.vscale; a.v8 = static_cast<uint8_t*>(v8);
+    SAGE_HIP(launch_quant(a, B, D, st));
     return MI355_SAGE_OK;
 }
 
 int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void* k8, const void* kscale,
                         int blkk, const void* vq, const void* vscale, int variant, int B, int H, int N_q,
-                        int N_kv, int kv_valid, int D, void* O, const int64_t* o_strides, int64_t o_off,
-                        void* stats, void* stream) {
+                        int N_kv, int kv_valid, int mask_lo, int mask_hi, int D,
+                        void* O, const int64_t* o_strides, int64_t o_off,
+                        const void* qshift, void* stats, void* stream) {
     if (!q8 || !qscale || !k8 || !kscale || !vq || !O || !o_strides) return MI355_SAGE_EINVAL;
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
     if (kv_valid <= 0 || kv_valid > N_kv) return MI355_SAGE_EINVAL;
@@ -420,8 +548,9 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     AttnArgs a{};
     a.q8 = static_cast<const int8_t*>(q8); a.qscale = static_cast<const float*>(qscale); a.blkq = blkq;
     a.k8 = static_cast<const int8_t*>(k8); a.kscale = static_cast<const float*>(kscale); a.blkk = blkk;
-    a.vq = vq; a.vscale = static_cast<const float*>(vscale); a.qshift = nullptr;
+    a.vq = vq; a.vscale = static_cast<const float*>(vscale); a.qshift = static_cast<const float*>(qshift);
     a.variant = variant;
+    if (clip_mask(kv_valid, mask_lo, mask_hi, &a.km) <= 0) return MI355_SAGE_EINVAL;
     a.B = B; a.H = H; a.Nq = N_q; a.Nkv = N_kv; a.kv_valid = kv_valid; a.D = D;
     a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(N_kv, kPadKV);
     a.o = static_cast<uint16_t*>(O) + o_off; a.osb = o_strides[0]; a.osh = o_strides[1]; a.osn = o_strides[2];

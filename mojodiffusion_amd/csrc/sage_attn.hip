@@ -64,7 +64,7 @@ __device__ __forceinline__ void dma16(const void* gbase_uniform, uint32_t goff, 
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(lds_base_uniform), "v"(goff), "s"(gbase_uniform)
-                 : "memory");
+                 : "memory");      // (m0 is a reserved register to the compiler: it never keeps a value in it across statements)
 }
 // Wait until at most N of this wave's copies are still in flight (they complete in order).
 template <int N> __device__ __forceinline__ void dma_wait() {
@@ -104,11 +104,15 @@ __device__ __forceinline__ v16i mfma_i8_from_magic(const v4i& a, const v4i& b) {
 // exceeds it by more than tau powers of two; until then p = exp2(s - m_used) may reach
 // 2^tau.  fp16 P holds 2^8 without loss.  The e4m3 variant maps p = 2^tau to the format
 // maximum 448, i.e. it stores e4m3(p * 448 / 2^tau); the factor cancels against the
-// normaliser, which sums the same scaled values.  tau = 1 keeps all but one binade of the
-// e4m3 range below p = 1.
+// normaliser, which sums the same scaled values.  Its reference is always a whole number
+// (the maximum rounded up): a probability's e4m3 significand then depends on the fractional
+// part of its score only, not on which whole number the reference happens to be, so the
+// stored probabilities are those of a softmax taken against ceil(row maximum) up to a power
+// of two, and the rescale factors are exact.
 template <int VARIANT> struct Lazy {
     static constexpr float tau = VARIANT == 0 ? 8.0f : 1.0f;
     static constexpr float log2_pscale = VARIANT == 0 ? 0.0f : 7.807354922057604f;     // log2(448 / 2)
+    static constexpr bool integer_ref = VARIANT == 1;
 };
 
 template <int D, int VARIANT, bool STATS>
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
     const float* __restrict__ qshift,
-    int H, int Nq, int kv_valid, int64_t nq_pad, int64_t nkv_pad,
+    int H, int Nq, int kv_valid, int mask_lo, int mask_hi, int64_t nq_pad, int64_t nkv_pad,
     uint16_t* __restrict__ o, int64_t osb, int64_t osh, int64_t osn,
     float* __restrict__ stats, int n_qtiles, int total_wg) {
     constexpr int VB = (VARIANT == 0) ? 2 : 1;          // bytes per V element
@@ -235,8 +239,18 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     for (int d = 0; d < DB; d++)
 #pragma unroll
         for (int i = 0; i < 16; i++) oacc[d][i] = 0.0f;
-    float m_used = -INFINITY;      // reference maximum the exponentials are taken against (log2 domain)
-    float l_run = 0.0f;            // this lane's share of the row sum (times pscale)
+    // reference maximum the exponentials are taken against (log2 domain); finite from the start
+    // so that a tile whose keys are all masked (every score -inf) still yields p = 0, not NaN
+    float m_used = -3.0e38f;
+    float l_run = 0.0f;            // fp16 variant: this lane's share of the row sum
+    // e4m3 variant: the row sum is taken over the ROUNDED probabilities, on the matrix pipe — one
+    // more product per tile against a tile of ones (e4m3 1.0 = 0x38) gives every lane the sum over
+    // all 64 keys of its query, in every accumulator element; element 0 is the one that is kept
+    // to scale.  It is rescaled together with the output accumulators.
+    v16f lacc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) lacc[i] = 0.0f;
+    const v8i ones8 = {0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838};
 
     // Loop-carried fragments: K of the tile whose scores come next, the first PD units of
     // V^T of the tile whose P.V comes next, and the packed probabilities of two tiles (parity).
@@ -266,6 +280,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             const v8i pw = {(int)p[pb][0], (int)p[pb][1], (int)p[pb][2], (int)p[pb][3],
                             (int)p[pb][4], (int)p[pb][5], (int)p[pb][6], (int)p[pb][7]};
             oacc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pw, oacc[d], 0, 0, 0, 0, 0, 0);
+            if (u == NUNIT - 1) lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones8, pw, lacc, 0, 0, 0, 0, 0, 0);
         }
     };
 
@@ -291,11 +306,10 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     // max / compare / cross-lane chain from the common path.  A reference that has become too
     // low shows up as a large tile sum (every p is non-negative, so sum <= 2^12 bounds each
     // p, far inside fp16 range); then the tile is redone the careful way.
-    auto iteration = [&](int t, auto x_tag, auto first_tag, auto mask_tag, auto opt_tag) {
+    auto iteration = [&](int t, auto x_tag, auto first_tag) {
         constexpr int X = decltype(x_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
-        constexpr bool MASK = decltype(mask_tag)::value;
-        constexpr bool OPT = decltype(opt_tag)::value;
+        constexpr bool OPT = VARIANT == 0 && !FIRST;
         const int slot_vprev = (t + NSV - 1) % NSV, slot_knext = (t + 1) % NSK;
 
         // ---- S^T = K(t) . Q^T : two 32-key blocks
@@ -310,13 +324,18 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         float f[2], c0[2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) f[kb] = sq * kscale_of(t * 2 + kb);
-        if (MASK) {
+        // Tiles that hold masked keys (the ragged end, the masked range) are rare: a real branch.
+        // A masked score becomes -inf (as an integer: below every real accumulator), which the
+        // exponent path below turns into p = 0 without any further test.
+        const int key0 = t * kTileKV;
+        if (key0 + kTileKV > kv_valid || (key0 < mask_hi && key0 + kTileKV > mask_lo)) {
+            asm volatile("" ::: "memory");
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int key = t * kTileKV + kb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                    if (key >= kv_valid) s[kb][i] = (int)0xFF800000;     // -inf as fp32, below every real accumulator
+                    const int key = key0 + kb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                    if (key >= kv_valid || (key >= mask_lo && key < mask_hi)) s[kb][i] = (int)0xFF800000;
                 }
         }
         float corr = 1.0f;
@@ -334,13 +353,14 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
                     mb = max(max(mb, s[kb][i + 2]), s[kb][i + 3]);
                 }
                 const int mi = max(max(ma, mb), max(s[kb][14], s[kb][15]));
-                const float mk = MASK && mi < 0 ? -INFINITY : (float)(mi - kMagicI) * (f[kb] * (1.0f / kMagicUnit));
+                const float mk = mi < 0 ? -INFINITY : (float)(mi - kMagicI) * (f[kb] * (1.0f / kMagicUnit));
                 mt = fmaxf(mt, mk);
             }
             const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);
             mt = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
             refresh = __any(mt > m_used + tau);
-            const float m_new = refresh ? fmaxf(m_used, mt) : m_used;
+            float m_new = m_used;
+            if (refresh) m_new = Lazy<VARIANT>::integer_ref ? ceilf(fmaxf(m_used, mt)) : fmaxf(m_used, mt);
             corr = __builtin_amdgcn_exp2f(m_used - m_new);           // 1 when nothing changed
             m_used = m_new;
             l_run *= corr;             // already includes tile t-1's probabilities
@@ -355,10 +375,6 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             const int kb = n >> 4, i = n & 15;
             float p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
             float p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
-            if (MASK) {
-                if (s[kb][i] < 0) p0 = 0.0f;
-                if (s[kb][i + 1] < 0) p1 = 0.0f;
-            }
             if constexpr (VARIANT == 0) {
                 const v2h pr = {(_Float16)p0, (_Float16)p1};
                 const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
@@ -366,7 +382,6 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
                 l_run = __builtin_amdgcn_fdot2(pr, ones, l_run, false);
                 p[X][n >> 1] = __builtin_bit_cast(uint32_t, pr);
             } else {
-                l_run += p0 + p1;
                 const int w = n >> 2;
                 if (n & 2) p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, (int)p[X][w], true);
                 else p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
@@ -378,7 +393,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             // Pin the group here: an empty volatile statement that consumes the results keeps the
             // compiler from sinking the exponentials below the matrix instructions they are meant
             // to overlap with.
-            asm volatile("" : "+v"(l_run), "+v"(p[X][VARIANT == 0 ? (g * EPU) >> 1 : (g * EPU) >> 2]));
+            if constexpr (VARIANT == 0) asm volatile("" : "+v"(l_run), "+v"(p[X][(g * EPU) >> 1]));
+            else asm volatile("" : "+v"(p[X][(g * EPU) >> 2]));
         };
 
         // At the midpoint every wave has finished iteration t-1 completely, so the ring slots
@@ -422,6 +438,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             for (int d = 0; d < DB; d++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) oacc[d][i] *= corr;
+            lacc[0] *= corr;
         }
         // first V^T fragments of tile t for the next iteration (published by this iteration's midpoint)
 #pragma unroll
@@ -429,34 +446,18 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         read_kf(slot_knext, 1);
     };
 
-    const bool ragged = (kv_valid & (kTileKV - 1)) != 0;
     using T = std::true_type;
     using F = std::false_type;
     using X0 = std::integral_constant<int, 0>;
     using X1 = std::integral_constant<int, 1>;
-    using OPT = std::integral_constant<bool, VARIANT == 0>;
-    if (last == 0) {
-        if (ragged) iteration(0, X0{}, T{}, T{}, F{});
-        else iteration(0, X0{}, T{}, F{}, F{});
-    } else {
-        iteration(0, X0{}, T{}, F{}, F{});
+    iteration(0, X0{}, T{});
+    {
         int t = 1;
-        for (; t + 1 < last; t += 2) {
-            iteration(t, X1{}, F{}, F{}, OPT{});
-            iteration(t + 1, X0{}, F{}, F{}, OPT{});
+        for (; t < last; t += 2) {
+            iteration(t, X1{}, F{});
+            iteration(t + 1, X0{}, F{});
         }
-        if (t < last) {
-            iteration(t, X1{}, F{}, F{}, OPT{});
-            t++;
-        }
-        // t == last
-        if (t & 1) {
-            if (ragged) iteration(t, X1{}, F{}, T{}, F{});
-            else iteration(t, X1{}, F{}, F{}, F{});
-        } else {
-            if (ragged) iteration(t, X0{}, F{}, T{}, F{});
-            else iteration(t, X0{}, F{}, F{}, F{});
-        }
+        if (t == last) iteration(t, X1{}, F{});
     }
     // ---- drain: P.V of the last tile ------------------------------------------------------
     auto drain = [&](auto x_tag) {
@@ -472,9 +473,11 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
 
     // ---- epilogue: normalise, bf16 round-to-nearest-even, caller's strides ---------
     float l_tot;
-    {
+    if constexpr (VARIANT == 0) {
         const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
         l_tot = __uint_as_float(r.x) + __uint_as_float(r.y);
+    } else {
+        l_tot = lacc[0];
     }
     const float inv = 1.0f / l_tot;      // l carries pscale, which cancels the pscale in P
     if (qrow < Nq) {
@@ -514,11 +517,11 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     if (a.stats != nullptr)
         hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, true>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
                            a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
-                           a.kv_valid, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
+                           a.kv_valid, a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
     else
         hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, false>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
                            a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
-                           a.kv_valid, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
+                           a.kv_valid, a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
     return hipGetLastError();
 }
 

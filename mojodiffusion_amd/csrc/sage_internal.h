@@ -34,34 +34,60 @@ struct PreOp {
     int64_t batch_rows;          // 0: all batches share the table
 };
 
-// ---- quantize kernels (sage_quant.hip) -------------------------------------
-// Q (is_k = false): x = f32(q)*cmul.  K (is_k = true): x = f32(k) - mean (mean may be null).
-// rowdot (Q only, may be null): [B,H,n_pad] <pre-scaled q row, mean>, needed for the
-// log-sum-exp output when K is smoothed.
-hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad,
-                           int blk, bool is_k, float cmul, const float* mean,
-                           int8_t* codes, float* scales, float* rowdot, const PreOp& pre, hipStream_t st);
+// Keys lo <= s < hi take no part (statistics, scale blocks, scores); lo >= hi: no such range.
+struct KeyMask {
+    int lo, hi;
+};
 
-// K mean: group partials (double, [B,H,ngroups,D]) then the final mean.
-hipError_t launch_kmean(const View& k, int B, int H, int N, int D,
-                        double* group_partials, float* kmean, const PreOp& pre, hipStream_t st);
+// ---- quantize kernels (sage_quant.hip): three launches --------------------------------
+// Launch 1: passes over V and K whose results the later launches need.
+struct PrepArgs {
+    View k, v;
+    int H, Nkv;
+    int64_t nkv_pad;
+    KeyMask km;
+    int vmode;                       // 0: fp16 repack into v16; 1: channel maxima per group into vpart; 2: no V pass
+    uint16_t* v16;
+    float* vpart;                    // [B,H,ngroups,D]
+    double* kpart_sum;               // [B,H,ngroups,D] group sums; null: no K pass
+    float* kpart_mm;                 // [B,H,ngroups,D,2] group minima / maxima
+    PreOp pre_k;
+    int ngroups, nk_wg, nv_units;    // filled by the launcher
+};
+hipError_t launch_prep(const PrepArgs& a, int B, int D, hipStream_t st);
 
-// One-shot path: Q quantizer + V fp16 repack + K-mean group sums in one launch, then the
-// K quantizer that finishes the mean from the group partials itself (partial == null: no
-// smoothing).  Same arithmetic, bit for bit, as the separate launches above.
-hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B, int H, int Nq, int Nkv, int D,
-                             int64_t nq_pad, int64_t nkv_pad, float cmul, int blkq, bool smooth_k,
-                             int8_t* q8, float* qscale, uint16_t* v16, double* partial,
-                             const PreOp& pre_q, const PreOp& pre_k, hipStream_t st);
-hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
-                               const double* partial, float* kmean, int8_t* codes, float* scales,
-                               const PreOp& pre, hipStream_t st);
+// Launch 2: per (b,h,channel) K mean and balancing factor, V scale.
+struct FinalArgs {
+    int64_t total;                   // B*H*D
+    int D, ngroups, kept, flags;     // kept = number of keys that count; flags: bit 0 smoothing, bit 1 balancing
+    float cmul;                      // fp32(scale*log2(e))
+    const double* kpart_sum;         // null: no K statistics (mean 0, factor 1)
+    const float* kpart_mm;
+    float *kmean, *qmul, *kmul;      // [B,H,D] each; kmean null: K outputs are skipped
+    const float* vpart;
+    float* vscale;                   // null: V output is skipped
+};
+hipError_t launch_stats_final(const FinalArgs& a, hipStream_t st);
 
-hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t n_pad,
-                              uint16_t* v16, hipStream_t st);
-
-hipError_t launch_quant_v_fp8(const View& v, int B, int H, int N, int D, int64_t n_pad,
-                              uint8_t* v8, float* vscale, hipStream_t st);
+// Launch 3: the encoders.  q8 / k8 / v8 null: that role is skipped.
+struct QuantArgs {
+    View q, k, v;
+    int H, Nq, Nkv;
+    int64_t nq_pad, nkv_pad;
+    KeyMask km;
+    int blkq, blkk;
+    float cmul;
+    const float *kmean, *qmul, *kmul, *vscale;
+    int8_t* q8;
+    float* qscale;
+    float* rowdot;                   // [B,H,nq_pad] <f32(q)*cmul, kmean>, or null
+    int8_t* k8;
+    float* kscale;
+    uint8_t* v8;
+    PreOp pre_q, pre_k;
+    int nq_blk, nk_blk, nv_tile;     // filled by the launcher
+};
+hipError_t launch_quant(const QuantArgs& a, int B, int D, hipStream_t st);
 
 // ---- attention kernel (sage_attn.hip) --------------------------------------
 struct AttnArgs {
@@ -69,6 +95,7 @@ struct AttnArgs {
     const int8_t* k8;  const float* kscale;  int blkk;
     const void* vq;    const float* vscale;  const float* qshift;  // qshift [B,H,nq_pad], stats only
     int variant;
+    KeyMask km;
     int B, H, Nq, Nkv, kv_valid, D;
     int64_t nq_pad, nkv_pad;
     uint16_t* o; int64_t osb, osh, osn;

@@ -1,10 +1,16 @@
-// sage_quant.hip — HBM-bound kernels of the quantized-SDPA path (gfx950):
-//   * per-block INT8 quantization of Q (pre-scaled) and K (mean-smoothed),
-//   * the K mean over tokens (deterministic summation tree in fp64),
-//   * V repack to tiled fp16, V quantization to tiled e4m3 with per-channel scales.
+// sage_quant.hip — HBM-bound kernels of the quantized-SDPA path (gfx950), three launches:
 //
-// Every fp32 step that decides a code is a single IEEE operation (true divide,
-// round-half-to-even), so the codes and scales are reproducible bit-for-bit.
+//   prep_kernel         per (b,h), workgroup roles:  V repack to tiled fp16  |  V channel
+//                       maxima per 256-token group (e4m3 variant)  |  K channel sums (fp64),
+//                       minima and maxima per 256-token group
+//   stats_final_kernel  per (b,h,channel): K mean, balancing factor -> kmean, qmul, kmul;
+//                       V maxima -> vscale
+//   quant_kernel        per (b,h), workgroup roles:  Q blocks -> int8 + scale  |  K blocks ->
+//                       int8 + scale  |  V tiles -> e4m3 (e4m3 variant)
+//
+// Every fp32 step that decides a code is a single IEEE operation (true divide, IEEE sqrt,
+// round-half-to-even) and every reduction either has a fixed order (the fp64 sums) or is
+// order-free (max / min), so codes, scales and statistics are reproducible bit for bit.
 // All kernels read bf16 rows with 16-byte loads (8 channels per lane).
 #include "sage_internal.h"
 
@@ -25,6 +31,13 @@ __device__ __forceinline__ void unpack8(const u32x4& w, float* x) {
     x[6] = bf16_lo(w.w); x[7] = bf16_hi(w.w);
 }
 
+__device__ __forceinline__ void load8(const float* p, float* x) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
@@ -39,24 +52,32 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
 }
 __device__ __forceinline__ float round_to_bf16(float f) { return __uint_as_float(f32_to_bf16_rne(f) << 16); }
 
+__device__ __forceinline__ bool key_kept(int s, int N, const KeyMask& m) { return s < N && !(s >= m.lo && s < m.hi); }
+
 // RMSNorm (+ RoPE) of one row, spread over the D/8 consecutive lanes that hold its 16-byte
 // chunks: x[0..7] are channels col..col+7.  Every lane of the group must call this (it
 // exchanges partial sums); `valid` false = a padding row, which stays zero.
 // Arithmetic, step for step (all fp32, no fused multiply-add):
-//   squares added left to right inside the chunk, chunk sums combined pairwise, neighbours
-//   first; inv = 1/sqrt(sum/D + eps); y = bf16((x*inv)*gain); rotation of (y[2i], y[2i+1]) by
+//   the squares are added in the order of serenitymojo/ops/norm.mojo:56-72 — a 256-slot array
+//   folded in halves, far pairs first: channel t with t+64 (D = 128), then strides 32, 16 and
+//   8, which pair lanes of the row, then 4, 2, 1 inside the lane;
+//   inv = 1/sqrt(sum/D + eps); y = bf16((x*inv)*gain); rotation of (y[2i], y[2i+1]) by
 //   the table angle with both products rounded before the subtract / add; result bf16.
 template <int D>
 __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, int row, int col, bool valid, float* x) {
     constexpr int CPR = D / 8;
-    float a = 0.0f;
+    float sq[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-        const float sq = x[e] * x[e];
-        a = a + sq;
-    }
+    for (int e = 0; e < 8; e++) sq[e] = x[e] * x[e];
 #pragma unroll
-    for (int off = 1; off < CPR; off <<= 1) a = a + __shfl_xor(a, off, 64);
+    for (int off = CPR / 2; off > 0; off >>= 1)
+#pragma unroll
+        for (int e = 0; e < 8; e++) sq[e] = sq[e] + __shfl_xor(sq[e], off, 64);
+#pragma unroll
+    for (int e = 0; e < 4; e++) sq[e] = sq[e] + sq[e + 4];
+    sq[0] = sq[0] + sq[2];
+    sq[1] = sq[1] + sq[3];
+    const float a = sq[0] + sq[1];
     const float mean = a / (float)D;
     const float inv = 1.0f / sqrtf(mean + p.eps);
     const u32x4 gw = *reinterpret_cast<const u32x4*>(p.gain + col);
@@ -94,9 +115,9 @@ __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, i
 }
 
 // ---------------------------------------------------------------------------
-// Per-block INT8 quantization.  One workgroup (256 threads) per (block, h, b);
-// the block's BLK x D tile lives in registers between the absmax pass and the
-// encode pass, so HBM sees one read of bf16 and one write of int8.
+// Per-block INT8 quantization.  One workgroup (256 threads) per block of BLK tokens of one
+// (b,h); the BLK x D tile lives in registers between the absmax pass and the encode pass, so
+// HBM sees one read of bf16 and one write of int8.
 // ---------------------------------------------------------------------------
 // rint(x / sc) for |x / sc| <= ~127 without paying a full IEEE divide per element: x * (1/sc)
 // is within 2^-15 of the correctly rounded quotient (both below 128), so whenever it lies at
@@ -110,68 +131,68 @@ __device__ __forceinline__ float rint_quotient(float x, float sc, float rinv, bo
     return n;
 }
 
-struct NoHook {
-    __device__ __forceinline__ void operator()() const {}
-};
-
-// `mean` points at the D means of this (b,h) (global or LDS), or is null.  `hook` runs after
-// the tile's loads are issued and before anything reads `mean` (it may compute the mean into
-// LDS; it must end with a barrier if it does).
-template <int D, int BLK, bool IS_K, bool PRE, typename Hook = NoHook>
+// Q (IS_K false): x = f32(q) * chmul[d].  K (IS_K true): x = (f32(k) - mean[d]) * chmul[d];
+// tokens that are masked or beyond N count for nothing and get code 0.
+// rowdot (Q only, may be null): <f32(q) * cmul, mean> per row.
+template <int D, int BLK, bool IS_K, bool PRE>
 __device__ __forceinline__ void quant_i8_block(
     int t, int h, int b, const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, float cmul, const float* mean,
+    int N, int H, int64_t n_pad, const KeyMask& km, const float* __restrict__ mean,
+    const float* __restrict__ chmul, float cmul,
     int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, float* red,
-    const PreOp& pre, Hook hook = Hook()) {
+    const PreOp& pre) {
     constexpr int CPR = D / 8;                 // 16-byte chunks per row
     constexpr int NCH = BLK * CPR / 256;       // chunks per thread
     static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
+    static_assert(256 % CPR == 0, "a thread keeps one column group for all its chunks");
     const int tid = threadIdx.x;
     const int r0 = t * BLK;
+    const int col = (tid % CPR) * 8;
     const int64_t bh = (int64_t)b * H + h;
     const uint16_t* src = x + b * sb + h * sh;
 
     u32x4 raw[NCH];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        const int c = i * 256 + tid;
-        const int row = r0 + c / CPR, col = (c % CPR) * 8;
+        const int row = r0 + (i * 256 + tid) / CPR;
         raw[i] = u32x4{0u, 0u, 0u, 0u};
         if (row < N) raw[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
     }
-    hook();
+    float mul[8], mu[8];
+    load8(chmul + col, mul);
+    if (IS_K || rowdot != nullptr) load8(mean + col, mu);
 
     float v[NCH][8];
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        const int c = i * 256 + tid;
-        const int row = r0 + c / CPR, col = (c % CPR) * 8;
+        const int row = r0 + (i * 256 + tid) / CPR;
         unpack8(raw[i], v[i]);
         if constexpr (PRE) pre_apply<D>(pre, b, h, H, row, col, row < N, v[i]);
+        bool counts;
         if (IS_K) {
-            if (mean != nullptr) {
-                const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
-                const float4 m1 = *reinterpret_cast<const float4*>(mean + col + 4);
-                v[i][0] -= m0.x; v[i][1] -= m0.y; v[i][2] -= m0.z; v[i][3] -= m0.w;
-                v[i][4] -= m1.x; v[i][5] -= m1.y; v[i][6] -= m1.z; v[i][7] -= m1.w;
+            counts = key_kept(row, N, km);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float d = v[i][e] - mu[e];
+                v[i][e] = d * mul[e];
             }
         } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[i][e] *= cmul;
+            counts = row < N;
             if (rowdot != nullptr) {
                 // <pre-scaled query row, K mean>: the amount K smoothing lowers every score
                 // of this row by; the CPR lanes that share a row are adjacent in the wave.
-                const float4 m0 = *reinterpret_cast<const float4*>(mean + col);
-                const float4 m1 = *reinterpret_cast<const float4*>(mean + col + 4);
-                float dot = v[i][0] * m0.x + v[i][1] * m0.y + v[i][2] * m0.z + v[i][3] * m0.w +
-                            v[i][4] * m1.x + v[i][5] * m1.y + v[i][6] * m1.z + v[i][7] * m1.w;
+                float dot = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) dot += (v[i][e] * cmul) * mu[e];
 #pragma unroll
                 for (int off = CPR / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
                 if ((tid % CPR) == 0) rowdot[bh * n_pad + row] = dot;
             }
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[i][e] *= mul[e];
         }
-        if (row < N) {
+        if (counts) {
 #pragma unroll
             for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[i][e]));
         }
@@ -182,18 +203,16 @@ __device__ __forceinline__ void quant_i8_block(
     __syncthreads();
     amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 
-    const bool real_block = r0 < N;
-    const float sc = (real_block && amax > 0.0f) ? amax / 127.0f : 1.0f;
+    const float sc = amax > 0.0f ? amax / 127.0f : 1.0f;      // blocks without a counting token: amax == 0
     if (tid == 0) scales[bh * (n_pad / BLK) + t] = sc;
     const bool fast = sc >= 0x1p-100f && sc <= 0x1p100f;
     const float rinv = 1.0f / sc;
 
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        const int c = i * 256 + tid;
-        const int row = r0 + c / CPR, col = (c % CPR) * 8;
+        const int row = r0 + (i * 256 + tid) / CPR;
         uint32_t pk[2] = {0u, 0u};
-        if (row < N) {
+        if (IS_K ? key_kept(row, N, km) : row < N) {
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 float r = rint_quotient(v[i][e], sc, rinv, fast);
@@ -206,67 +225,26 @@ __device__ __forceinline__ void quant_i8_block(
     }
 }
 
-template <int D, int BLK, bool IS_K, bool PRE>
-__global__ __launch_bounds__(256) void quant_i8_kernel(
-    const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, float cmul, const float* __restrict__ mean,
-    int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, PreOp pre) {
-    __shared__ float red[4];
-    const int h = blockIdx.y, b = blockIdx.z;
-    quant_i8_block<D, BLK, IS_K, PRE>(blockIdx.x, h, b, x, sb, sh, sn, N, H, n_pad, cmul,
-                                 mean ? mean + ((int64_t)b * H + h) * D : nullptr, codes, scales, rowdot, red, pre);
-}
-
-template <int D, bool IS_K>
-static hipError_t launch_quant_i8_d(const View& x, int B, int H, int N, int64_t n_pad, int blk,
-                                    float cmul, const float* mean, int8_t* codes, float* scales,
-                                    float* rowdot, const PreOp& pre, hipStream_t st) {
-    dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
-#define SAGE_LAUNCH_Q(BLK)                                                                          \
-    do {                                                                                           \
-        if (pre.gain != nullptr)                                                                   \
-            hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K, true>), grid, block, 0, st, x.p, x.sb, \
-                               x.sh, x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot, pre);   \
-        else                                                                                       \
-            hipLaunchKernelGGL((quant_i8_kernel<D, BLK, IS_K, false>), grid, block, 0, st, x.p, x.sb, \
-                               x.sh, x.sn, N, H, n_pad, cmul, mean, codes, scales, rowdot, pre);   \
-    } while (0)
-    switch (blk) {
-        case 32: SAGE_LAUNCH_Q(32); break;
-        case 64: SAGE_LAUNCH_Q(64); break;
-        case 128: SAGE_LAUNCH_Q(128); break;
-        default: return hipErrorInvalidValue;
-    }
-#undef SAGE_LAUNCH_Q
-    return hipGetLastError();
-}
-
-hipError_t launch_quant_i8(const View& x, int B, int H, int N, int D, int64_t n_pad, int blk,
-                           bool is_k, float cmul, const float* mean, int8_t* codes,
-                           float* scales, float* rowdot, const PreOp& pre, hipStream_t st) {
-    if (n_pad % blk != 0) return hipErrorInvalidValue;
-    if (D == 128)
-        return is_k ? launch_quant_i8_d<128, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st)
-                    : launch_quant_i8_d<128, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st);
-    if (D == 64)
-        return is_k ? launch_quant_i8_d<64, true>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st)
-                    : launch_quant_i8_d<64, false>(x, B, H, N, n_pad, blk, cmul, mean, codes, scales, rowdot, pre, st);
-    return hipErrorInvalidValue;
-}
-
 // ---------------------------------------------------------------------------
-// K mean.  Summation tree (all in fp64, every order fixed):
+// K channel statistics of one group of 256 tokens.  Sums follow a fixed tree, all in fp64:
 //   leaf  = 16 consecutive tokens, added in ascending order by one lane
 //   group = 16 consecutive leaves, added in ascending order
-//   total = groups added in ascending order;  mean = fp32(total / N)
-// Kernel 1: one workgroup per (group, h, b); lane (leaf, 8-channel chunk).
-// Kernel 2: one thread per (b, h, channel).
+//   total = groups added in ascending order (stats_final_kernel)
+// Tokens that are masked or beyond N add +0.0 and take no part in the minimum / maximum.
+// Executed by 16*(D/8) consecutive threads; `tid` is the index among them; g < 0: idle.
 // ---------------------------------------------------------------------------
-// Executed by 16*(D/8) consecutive threads; `tid` is the index among them.
+template <int D>
+struct KGroupSmem {
+    double leafsum[16][D + 2];
+    float leafmin[16][D + 1];
+    float leafmax[16][D + 1];
+};
+
 template <int D, bool PRE>
-__device__ __forceinline__ void kmean_group_body(
+__device__ __forceinline__ void kstats_group_body(
     int g, int h, int b, int tid, const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int ngroups, double* __restrict__ partial, double (*leafsum)[D + 2], const PreOp& pre) {
+    int N, int H, int ngroups, const KeyMask& km, double* __restrict__ part_sum, float* __restrict__ part_mm,
+    KGroupSmem<D>& sm, const PreOp& pre) {
     constexpr int CPR = D / 8;
     const int leaf = tid / CPR, col = (tid % CPR) * 8;
     const uint16_t* src = k + b * sb + h * sh + col;
@@ -276,89 +254,53 @@ __device__ __forceinline__ void kmean_group_body(
 #pragma unroll
     for (int i = 0; i < kLeaf; i++) {
         w[i] = u32x4{0u, 0u, 0u, 0u};
-        if (g >= 0 && s0 + i < N) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)(s0 + i) * sn);
+        if (g >= 0 && key_kept(s0 + i, N, km)) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)(s0 + i) * sn);
     }
     double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    float mn[8], mx[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) { mn[e] = INFINITY; mx[e] = -INFINITY; }
 #pragma unroll
     for (int i = 0; i < kLeaf; i++) {
         float x[8];
         unpack8(w[i], x);
-        if constexpr (PRE) pre_apply<D>(pre, b, h, H, s0 + i, col, g >= 0 && s0 + i < N, x);
-        // rows past N contribute +0.0, which leaves a double sum unchanged
+        const bool kept = g >= 0 && key_kept(s0 + i, N, km);
+        if constexpr (PRE) pre_apply<D>(pre, b, h, H, s0 + i, col, kept, x);
+        // tokens that do not count are +0.0 here, which leaves a double sum unchanged
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += (double)x[e];
-    }
-
+        if (kept) {
 #pragma unroll
-    for (int e = 0; e < 8; e++) leafsum[leaf][col + e] = acc[e];
+            for (int e = 0; e < 8; e++) { mn[e] = fminf(mn[e], x[e]); mx[e] = fmaxf(mx[e], x[e]); }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        sm.leafsum[leaf][col + e] = acc[e];
+        sm.leafmin[leaf][col + e] = mn[e];
+        sm.leafmax[leaf][col + e] = mx[e];
+    }
     __syncthreads();
     if (tid < D && g >= 0) {
         double gsum = 0.0;
+        float gmn = INFINITY, gmx = -INFINITY;
 #pragma unroll
-        for (int u = 0; u < 16; u++) gsum += leafsum[u][tid];
-        partial[(((int64_t)b * H + h) * ngroups + g) * D + tid] = gsum;
+        for (int u = 0; u < 16; u++) {
+            gsum += sm.leafsum[u][tid];
+            gmn = fminf(gmn, sm.leafmin[u][tid]);
+            gmx = fmaxf(gmx, sm.leafmax[u][tid]);
+        }
+        const int64_t o = (((int64_t)b * H + h) * ngroups + g) * D + tid;
+        part_sum[o] = gsum;
+        part_mm[2 * o] = gmn;
+        part_mm[2 * o + 1] = gmx;
     }
-}
-
-template <int D, bool PRE>
-__global__ __launch_bounds__(16 * (D / 8)) void kmean_group_kernel(
-    const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int ngroups, double* __restrict__ partial, PreOp pre) {
-    __shared__ double leafsum[16][D + 2];
-    kmean_group_body<D, PRE>(blockIdx.x, blockIdx.y, blockIdx.z, threadIdx.x, k, sb, sh, sn, N, H, ngroups, partial, leafsum, pre);
-}
-
-__global__ __launch_bounds__(256) void kmean_final_kernel(
-    const double* __restrict__ partial, int ngroups, int D, int N, int64_t total,
-    float* __restrict__ kmean) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;      // (bh, d)
-    if (i >= total) return;
-    const int64_t bh = i / D;
-    const int d = (int)(i % D);
-    const double* p = partial + bh * ngroups * D + d;
-    double sum = 0.0;
-    for (int g0 = 0; g0 < ngroups; g0 += 8) {
-        double v[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = p[(int64_t)(g0 + j < ngroups ? g0 + j : ngroups - 1) * D];
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-            if (g0 + j < ngroups) sum += v[j];
-    }
-    kmean[i] = (float)(sum / (double)N);
-}
-
-hipError_t launch_kmean(const View& k, int B, int H, int N, int D, double* partial,
-                        float* kmean, const PreOp& pre, hipStream_t st) {
-    const int ngroups = (N + kGroup - 1) / kGroup;
-    dim3 grid((unsigned)ngroups, (unsigned)H, (unsigned)B);
-    const bool has_pre = pre.gain != nullptr;
-    if (D == 128 && has_pre)
-        hipLaunchKernelGGL((kmean_group_kernel<128, true>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
-                           N, H, ngroups, partial, pre);
-    else if (D == 128)
-        hipLaunchKernelGGL((kmean_group_kernel<128, false>), grid, dim3(256), 0, st, k.p, k.sb, k.sh, k.sn,
-                           N, H, ngroups, partial, pre);
-    else if (D == 64 && has_pre)
-        hipLaunchKernelGGL((kmean_group_kernel<64, true>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
-                           N, H, ngroups, partial, pre);
-    else if (D == 64)
-        hipLaunchKernelGGL((kmean_group_kernel<64, false>), grid, dim3(128), 0, st, k.p, k.sb, k.sh, k.sn,
-                           N, H, ngroups, partial, pre);
-    else
-        return hipErrorInvalidValue;
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    const int64_t total = (int64_t)B * H * D;
-    hipLaunchKernelGGL(kmean_final_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                       partial, ngroups, D, N, total, kmean);
-    return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
-// V repack: bf16 [.., N, D] -> fp16 tiles [.., N/64, D, 64]; key k of a tile
-// goes to slot v_slot_f16(k).  One workgroup per (tile, h, b): rows are read
-// coalesced, staged in LDS and written back channel-major in 16-byte runs.
+// V repack: bf16 [.., N, D] -> fp16 tiles [.., N/64, D, 64]; key k of a tile goes to slot
+// v_slot_f16(k).  One workgroup per (tile, h, b): rows are read coalesced, staged in LDS and
+// written back channel-major in 16-byte runs.  Rows that are masked or beyond N become 0.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ uint16_t f32_to_f16_sat(float x) {
     x = fminf(fmaxf(x, -65504.0f), 65504.0f);
@@ -376,7 +318,7 @@ __device__ __forceinline__ int v_tile_chunk(int slot, int chunk) {
 template <int D>
 __device__ __forceinline__ void quant_v_f16_body(
     int t, int h, int b, const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, uint16_t* __restrict__ out, uint16_t* tile) {
+    int N, int H, int64_t n_pad, const KeyMask& km, uint16_t* __restrict__ out, uint16_t* tile) {
     constexpr int CPR = D / 8;
     const int tid = threadIdx.x;
     const uint16_t* src = v + b * sb + h * sh;
@@ -387,7 +329,7 @@ __device__ __forceinline__ void quant_v_f16_body(
         const int key = c / CPR, col = (c % CPR) * 8;
         const int row = t * 64 + key;
         raw[i] = u32x4{0u, 0u, 0u, 0u};
-        if (row < N) raw[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+        if (key_kept(row, N, km)) raw[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
     }
 #pragma unroll
     for (int i = 0; i < 64 * CPR / 256; i++) {
@@ -425,213 +367,23 @@ __device__ __forceinline__ void quant_v_f16_body(
     }
 }
 
-template <int D>
-__global__ __launch_bounds__(256) void quant_v_f16_kernel(
-    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, uint16_t* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * D];
-    quant_v_f16_body<D>(blockIdx.x, blockIdx.y, blockIdx.z, v, sb, sh, sn, N, H, n_pad, out, tile);
-}
-
-hipError_t launch_quant_v_f16(const View& v, int B, int H, int N, int D, int64_t n_pad,
-                              uint16_t* v16, hipStream_t st) {
-    dim3 grid((unsigned)(n_pad / 64), (unsigned)H, (unsigned)B);
-    if (D == 128)
-        hipLaunchKernelGGL((quant_v_f16_kernel<128>), grid, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, v16);
-    else if (D == 64)
-        hipLaunchKernelGGL((quant_v_f16_kernel<64>), grid, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, v16);
-    else
-        return hipErrorInvalidValue;
-    return hipGetLastError();
-}
-
 // ---------------------------------------------------------------------------
-// Fused launches of the one-shot path.  The Q quantizer, the V repack and the K-mean
-// group sums are independent of each other: one launch runs all three as workgroup roles
-// (saves two launch gaps and fills the chip while each role alone is too short to).  The
-// K quantizer then takes its mean straight from the group partials (added in group
-// order, the same arithmetic as kmean_final_kernel) while its tile loads are in flight,
-// which removes the separate final-mean launch.
-// ---------------------------------------------------------------------------
-struct PrepArgs {
-    View q, k, v;
-    int H, Nq, Nkv;
-    int64_t nq_pad, nkv_pad;
-    float cmul;
-    int8_t* q8; float* qscale; uint16_t* v16; double* partial;
-    int nq_blk, nv_tile, nk_wg, ngroups;      // per (b,h): Q blocks, V tiles, K-mean workgroups; K groups
-    PreOp pre_q, pre_k;
-};
-
-template <int D, int BLKQ, bool PRE>
-__global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
-    constexpr int GPW = 256 / (16 * (D / 8));             // K-mean groups per workgroup
-    union Smem {
-        float red[4];
-        uint16_t tile[64 * D];
-        double leafsum[GPW][16][D + 2];
-    };
-    __shared__ __attribute__((aligned(16))) Smem sm;
-    const int per_bh = a.nq_blk + a.nv_tile + a.nk_wg;
-    const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
-    const int b = bh / a.H, h = bh % a.H;
-    if (r < a.nq_blk) {
-        quant_i8_block<D, BLKQ, false, PRE>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, a.cmul, nullptr,
-                                       a.q8, a.qscale, nullptr, sm.red, a.pre_q);
-    } else if (r < a.nq_blk + a.nv_tile) {
-        quant_v_f16_body<D>(r - a.nq_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.v16, sm.tile);
-    } else {
-        const int sub = threadIdx.x / (16 * (D / 8));
-        const int g = (r - a.nq_blk - a.nv_tile) * GPW + sub;
-        // groups past the end still take part in the barrier inside; they read nothing and
-        // their sum is not stored
-        kmean_group_body<D, PRE>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh, a.k.sn,
-                            a.Nkv, a.H, a.ngroups, a.partial, sm.leafsum[sub], a.pre_k);
-    }
-}
-
-template <int D>
-struct MeanFromPartials {
-    const double* partial;      // this (b,h)'s [ngroups][D] group sums, or null
-    int ngroups, N;
-    float* mean_s;              // LDS, D floats
-    float* kmean_out;           // where to publish the mean, or null
-    __device__ __forceinline__ void operator()() const {
-        if (partial == nullptr) return;
-        if (threadIdx.x < D) {
-            // loads eight at a time (independent, all in flight together); adds strictly in
-            // group order
-            double sum = 0.0;
-            for (int g0 = 0; g0 < ngroups; g0 += 8) {
-                double p[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const int g = g0 + j < ngroups ? g0 + j : ngroups - 1;
-                    p[j] = partial[(int64_t)g * D + threadIdx.x];
-                }
-#pragma unroll
-                for (int j = 0; j < 8; j++)
-                    if (g0 + j < ngroups) sum += p[j];
-            }
-            const float m = (float)(sum / (double)N);
-            mean_s[threadIdx.x] = m;
-            if (kmean_out != nullptr) kmean_out[threadIdx.x] = m;
-        }
-        __syncthreads();
-    }
-};
-
-template <int D, int BLK, bool PRE>
-__global__ __launch_bounds__(256) void kquant_fused_kernel(
-    const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, const double* __restrict__ partial, int ngroups,
-    float* __restrict__ kmean, int8_t* __restrict__ codes, float* __restrict__ scales, PreOp pre) {
-    __shared__ float mean_s[D];
-    __shared__ float red[4];
-    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int64_t bh = (int64_t)b * H + h;
-    const bool smooth = partial != nullptr;
-    MeanFromPartials<D> hook{smooth ? partial + bh * ngroups * D : nullptr, ngroups, N, mean_s,
-                             (smooth && t == 0) ? kmean + bh * D : nullptr};
-    quant_i8_block<D, BLK, true, PRE>(t, h, b, k, sb, sh, sn, N, H, n_pad, 0.0f, smooth ? mean_s : nullptr,
-                                 codes, scales, nullptr, red, pre, hook);
-}
-
-template <int D>
-static hipError_t launch_prep_d(const PrepArgs& a, int B, int blkq, hipStream_t st) {
-    dim3 grid((unsigned)((int64_t)B * a.H * (a.nq_blk + a.nv_tile + a.nk_wg))), block(256);
-    const bool has_pre = a.pre_q.gain != nullptr;
-#define SAGE_LAUNCH_PREP(BLKQ)                                                                \
-    do {                                                                                      \
-        if (has_pre) hipLaunchKernelGGL((prep_kernel<D, BLKQ, true>), grid, block, 0, st, a); \
-        else hipLaunchKernelGGL((prep_kernel<D, BLKQ, false>), grid, block, 0, st, a);        \
-    } while (0)
-    switch (blkq) {
-        case 32: SAGE_LAUNCH_PREP(32); break;
-        case 64: SAGE_LAUNCH_PREP(64); break;
-        case 128: SAGE_LAUNCH_PREP(128); break;
-        default: return hipErrorInvalidValue;
-    }
-#undef SAGE_LAUNCH_PREP
-    return hipGetLastError();
-}
-
-hipError_t launch_prep_fused(const View& q, const View& k, const View& v, int B, int H, int Nq, int Nkv, int D,
-                             int64_t nq_pad, int64_t nkv_pad, float cmul, int blkq, bool smooth_k,
-                             int8_t* q8, float* qscale, uint16_t* v16, double* partial,
-                             const PreOp& pre_q, const PreOp& pre_k, hipStream_t st) {
-    PrepArgs a{};
-    a.pre_q = pre_q; a.pre_k = pre_k;
-    a.q = q; a.k = k; a.v = v; a.H = H; a.Nq = Nq; a.Nkv = Nkv; a.nq_pad = nq_pad; a.nkv_pad = nkv_pad;
-    a.cmul = cmul; a.q8 = q8; a.qscale = qscale; a.v16 = v16; a.partial = partial;
-    a.nq_blk = (int)(nq_pad / blkq);
-    a.nv_tile = (int)(nkv_pad / 64);
-    a.ngroups = (Nkv + kGroup - 1) / kGroup;
-    const int gpw = D == 128 ? 1 : 2;
-    a.nk_wg = smooth_k ? (a.ngroups + gpw - 1) / gpw : 0;
-    if (D == 128) return launch_prep_d<128>(a, B, blkq, st);
-    if (D == 64) return launch_prep_d<64>(a, B, blkq, st);
-    return hipErrorInvalidValue;
-}
-
-hipError_t launch_kquant_fused(const View& k, int B, int H, int N, int D, int64_t n_pad, int blk,
-                               const double* partial, float* kmean, int8_t* codes, float* scales,
-                               const PreOp& pre, hipStream_t st) {
-    const int ngroups = (N + kGroup - 1) / kGroup;
-    dim3 grid((unsigned)(n_pad / blk), (unsigned)H, (unsigned)B), block(256);
-#define SAGE_LAUNCH_KQ(DD, BLK)                                                                      \
-    do {                                                                                             \
-        if (pre.gain != nullptr)                                                                     \
-            hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK, true>), grid, block, 0, st, k.p, k.sb,  \
-                               k.sh, k.sn, N, H, n_pad, partial, ngroups, kmean, codes, scales, pre); \
-        else                                                                                         \
-            hipLaunchKernelGGL((kquant_fused_kernel<DD, BLK, false>), grid, block, 0, st, k.p, k.sb, \
-                               k.sh, k.sn, N, H, n_pad, partial, ngroups, kmean, codes, scales, pre); \
-    } while (0)
-    if (D == 128) {
-        switch (blk) {
-            case 32: SAGE_LAUNCH_KQ(128, 32); break;
-            case 64: SAGE_LAUNCH_KQ(128, 64); break;
-            case 128: SAGE_LAUNCH_KQ(128, 128); break;
-            default: return hipErrorInvalidValue;
-        }
-    } else if (D == 64) {
-        switch (blk) {
-            case 32: SAGE_LAUNCH_KQ(64, 32); break;
-            case 64: SAGE_LAUNCH_KQ(64, 64); break;
-            case 128: SAGE_LAUNCH_KQ(64, 128); break;
-            default: return hipErrorInvalidValue;
-        }
-    } else {
-        return hipErrorInvalidValue;
-    }
-#undef SAGE_LAUNCH_KQ
-    return hipGetLastError();
-}
-
-// ---------------------------------------------------------------------------
-// V e4m3 quantization with one scale per (b, h, channel).
-// Kernel 1: channel absmax over tokens (max is order-free; fp32 bit patterns of
-//           non-negative values order like unsigned integers, so atomicMax on
-//           the bits is exact).  vscale holds the amax bits until kernel 2.
-// Kernel 2: amax -> scale in place.  Kernel 3: encode into the tiled layout.
+// V channel maxima of one group of 256 tokens (e4m3 variant; max is order-free).
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void v_absmax_kernel(
-    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, uint32_t* __restrict__ amax_bits) {
+__device__ __forceinline__ void v_absmax_group_body(
+    int g, int h, int b, const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int ngroups, const KeyMask& km, float* __restrict__ part, float (*red)[D + 1]) {
     constexpr int CPR = D / 8;
     constexpr int ROWS = 256 / CPR;                        // rows covered per step
-    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x;
     const int col = (tid % CPR) * 8, r = tid / CPR;
     const uint16_t* src = v + b * sb + h * sh + col;
     float m[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    // 256 tokens per workgroup
 #pragma unroll 4
-    for (int i = 0; i < 256 / ROWS; i++) {
-        const int row = t * 256 + i * ROWS + r;
-        if (row < N) {
+    for (int i = 0; i < kGroup / ROWS; i++) {
+        const int row = g * kGroup + i * ROWS + r;
+        if (key_kept(row, N, km)) {
             u32x4 w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn);
             float x[8];
             unpack8(w, x);
@@ -639,29 +391,14 @@ __global__ __launch_bounds__(256) void v_absmax_kernel(
             for (int e = 0; e < 8; e++) m[e] = fmaxf(m[e], fabsf(x[e]));
         }
     }
-    __shared__ float red[ROWS][D + 1];
 #pragma unroll
     for (int e = 0; e < 8; e++) red[r][col + e] = m[e];
     __syncthreads();
     if (tid < D) {
         float mm = 0.0f;
         for (int i = 0; i < ROWS; i++) mm = fmaxf(mm, red[i][tid]);
-        atomicMax(amax_bits + ((int64_t)b * H + h) * D + tid, __float_as_uint(mm));
+        part[(((int64_t)b * H + h) * ngroups + g) * D + tid] = mm;
     }
-}
-
-// Clears the amax accumulator with a kernel (not hipMemsetAsync) so that a caller can
-// capture the whole sequence into a HIP graph.
-__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* __restrict__ p, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < total) p[i] = 0u;
-}
-
-__global__ __launch_bounds__(256) void v_scale_kernel(float* __restrict__ vscale, int64_t total) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const float amax = vscale[i];                          // bits written by atomicMax
-    vscale[i] = amax > 0.0f ? amax / 448.0f : 1.0f;
 }
 
 // fp32 -> e4m3fn, round-to-nearest-even, saturating at +-448, NaN -> +-0.
@@ -685,14 +422,14 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
     return byte | sign;
 }
 
+// V tile -> e4m3 with the per-channel scales, tiled layout (slot order v_slot_fp8).
 template <int D>
-__global__ __launch_bounds__(256) void quant_v_fp8_kernel(
-    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
-    int N, int H, int64_t n_pad, const float* __restrict__ vscale, uint8_t* __restrict__ out) {
+__device__ __forceinline__ void quant_v_fp8_body(
+    int t, int h, int b, const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
+    int N, int H, int64_t n_pad, const KeyMask& km, const float* __restrict__ vscale,
+    uint8_t* __restrict__ out, uint8_t* tile) {
     constexpr int CPR = D / 8;
     constexpr int LD = D + 16;                             // padded row (bytes)
-    __shared__ __attribute__((aligned(16))) uint8_t tile[64 * LD];
-    const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int tid = threadIdx.x;
     const int64_t bh = (int64_t)b * H + h;
     const uint16_t* src = v + b * sb + h * sh;
@@ -702,12 +439,10 @@ __global__ __launch_bounds__(256) void quant_v_fp8_kernel(
         const int key = c / CPR, col = (c % CPR) * 8;
         const int row = t * 64 + key;
         u32x4 w = {0u, 0u, 0u, 0u};
-        if (row < N) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
-        float x[8];
+        if (key_kept(row, N, km)) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+        float x[8], sc[8];
         unpack8(w, x);
-        const float4 s0 = *reinterpret_cast<const float4*>(vscale + bh * D + col);
-        const float4 s1 = *reinterpret_cast<const float4*>(vscale + bh * D + col + 4);
-        const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        load8(vscale + bh * D + col, sc);
         uint32_t pk[2] = {0u, 0u};
 #pragma unroll
         for (int e = 0; e < 8; e++) pk[e >> 2] |= f32_to_e4m3(x[e] / sc[e]) << ((e & 3) * 8);
@@ -727,26 +462,169 @@ __global__ __launch_bounds__(256) void quant_v_fp8_kernel(
     }
 }
 
-hipError_t launch_quant_v_fp8(const View& v, int B, int H, int N, int D, int64_t n_pad,
-                              uint8_t* v8, float* vscale, hipStream_t st) {
-    const int64_t total = (int64_t)B * H * D;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                       reinterpret_cast<uint32_t*>(vscale), total);
-    dim3 g1((unsigned)((N + 255) / 256), (unsigned)H, (unsigned)B);
-    dim3 g3((unsigned)(n_pad / 64), (unsigned)H, (unsigned)B);
-    if (D == 128) {
-        hipLaunchKernelGGL((v_absmax_kernel<128>), g1, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H,
-                           reinterpret_cast<uint32_t*>(vscale));
-        hipLaunchKernelGGL(v_scale_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, vscale, total);
-        hipLaunchKernelGGL((quant_v_fp8_kernel<128>), g3, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, vscale, v8);
-    } else if (D == 64) {
-        hipLaunchKernelGGL((v_absmax_kernel<64>), g1, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H,
-                           reinterpret_cast<uint32_t*>(vscale));
-        hipLaunchKernelGGL(v_scale_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, vscale, total);
-        hipLaunchKernelGGL((quant_v_fp8_kernel<64>), g3, dim3(256), 0, st, v.p, v.sb, v.sh, v.sn, N, H, n_pad, vscale, v8);
+// ---------------------------------------------------------------------------
+// Launch 1: independent passes over V and K as workgroup roles of one grid (one launch fills
+// the chip where each pass alone is too short to).
+// ---------------------------------------------------------------------------
+template <int D, bool PRE>
+__global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
+    constexpr int GPW = 256 / (16 * (D / 8));             // K groups per workgroup
+    union Smem {
+        uint16_t tile[64 * D];
+        float red[256 / (D / 8)][D + 1];
+        KGroupSmem<D> kg[GPW];
+    };
+    __shared__ __attribute__((aligned(16))) Smem sm;
+    const int per_bh = a.nv_units + a.nk_wg;
+    const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
+    const int b = bh / a.H, h = bh % a.H;
+    if (r < a.nv_units) {
+        if (a.vmode == 0)
+            quant_v_f16_body<D>(r, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km, a.v16, sm.tile);
+        else
+            v_absmax_group_body<D>(r, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.ngroups, a.km, a.vpart, sm.red);
     } else {
-        return hipErrorInvalidValue;
+        const int sub = threadIdx.x / (16 * (D / 8));
+        const int g = (r - a.nv_units) * GPW + sub;
+        // groups past the end still take part in the barrier inside; they read nothing and
+        // store nothing
+        kstats_group_body<D, PRE>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh,
+                                  a.k.sn, a.Nkv, a.H, a.ngroups, a.km, a.kpart_sum, a.kpart_mm, sm.kg[sub], a.pre_k);
     }
+}
+
+hipError_t launch_prep(const PrepArgs& a_in, int B, int D, hipStream_t st) {
+    PrepArgs a = a_in;
+    a.ngroups = (a.Nkv + kGroup - 1) / kGroup;
+    const int gpw = D == 128 ? 1 : 2;
+    a.nk_wg = a.kpart_sum != nullptr ? (a.ngroups + gpw - 1) / gpw : 0;
+    a.nv_units = a.vmode == 0 ? (int)(a.nkv_pad / 64) : (a.vmode == 1 ? a.ngroups : 0);
+    const int64_t total = (int64_t)B * a.H * (a.nv_units + a.nk_wg);
+    if (total == 0) return hipSuccess;
+    if (total > 0x7FFFFFFF) return hipErrorInvalidValue;
+    dim3 grid((unsigned)total), block(256);
+    const bool has_pre = a.pre_k.gain != nullptr;
+    if (D == 128 && has_pre) hipLaunchKernelGGL((prep_kernel<128, true>), grid, block, 0, st, a);
+    else if (D == 128) hipLaunchKernelGGL((prep_kernel<128, false>), grid, block, 0, st, a);
+    else if (D == 64 && has_pre) hipLaunchKernelGGL((prep_kernel<64, true>), grid, block, 0, st, a);
+    else if (D == 64) hipLaunchKernelGGL((prep_kernel<64, false>), grid, block, 0, st, a);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Launch 2: one thread per (b, h, channel).
+//   K: sum of the group sums in group order -> mean = fp32(sum / kept) (0 without smoothing);
+//      amax = max(|kmax - mean|, |kmin - mean|) — rounding is monotone, so this IS the largest
+//      |k - mean| over the kept keys; s = sqrt(amax) (1 when amax is 0 or without balancing);
+//      kmul = 1/s, qmul = cmul*s.
+//   V: vscale = amax/448 (1 when 0).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void stats_final_kernel(FinalArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;      // (bh, d)
+    if (i >= a.total) return;
+    const int64_t bh = i / a.D;
+    const int d = (int)(i % a.D);
+    if (a.kmean != nullptr) {
+        float mean = 0.0f, s = 1.0f;
+        if (a.kpart_sum != nullptr) {
+            const double* p = a.kpart_sum + bh * a.ngroups * a.D + d;
+            const float* q = a.kpart_mm + 2 * (bh * a.ngroups * a.D + d);
+            double sum = 0.0;
+            float mn = INFINITY, mx = -INFINITY;
+            for (int g0 = 0; g0 < a.ngroups; g0 += 8) {
+                double v[8];
+                float lo[8], hi[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int64_t g = g0 + j < a.ngroups ? g0 + j : a.ngroups - 1;
+                    v[j] = p[g * a.D];
+                    lo[j] = q[2 * g * a.D];
+                    hi[j] = q[2 * g * a.D + 1];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (g0 + j < a.ngroups) { sum += v[j]; mn = fminf(mn, lo[j]); mx = fmaxf(mx, hi[j]); }
+            }
+            if (a.flags & 1) mean = (float)(sum / (double)a.kept);
+            if (a.flags & 2) {
+                const float amax = fmaxf(fabsf(mx - mean), fabsf(mn - mean));
+                if (amax > 0.0f) s = sqrtf(amax);
+            }
+        }
+        a.kmean[i] = mean;
+        a.kmul[i] = 1.0f / s;
+        a.qmul[i] = a.cmul * s;
+    }
+    if (a.vscale != nullptr) {
+        const float* p = a.vpart + bh * a.ngroups * a.D + d;
+        float amax = 0.0f;
+        for (int g = 0; g < a.ngroups; g++) amax = fmaxf(amax, p[(int64_t)g * a.D]);
+        a.vscale[i] = amax > 0.0f ? amax / 448.0f : 1.0f;
+    }
+}
+
+hipError_t launch_stats_final(const FinalArgs& a, hipStream_t st) {
+    if (a.total <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(stats_final_kernel, dim3((unsigned)((a.total + 255) / 256)), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Launch 3: Q blocks, K blocks and (e4m3 variant) V tiles as workgroup roles.
+// ---------------------------------------------------------------------------
+template <int D, bool PRE>
+__global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
+    union Smem {
+        float red[4];
+        uint8_t tile8[64 * (D + 16)];
+    };
+    __shared__ __attribute__((aligned(16))) Smem sm;
+    const int per_bh = a.nq_blk + a.nk_blk + a.nv_tile;
+    const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
+    const int b = bh / a.H, h = bh % a.H;
+    const KeyMask none{0, 0};
+    if (r < a.nq_blk) {
+        const float* mul = a.qmul + (int64_t)bh * D;
+        const float* mean = a.kmean + (int64_t)bh * D;
+#define SAGE_Q(BLK) quant_i8_block<D, BLK, false, PRE>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, none, \
+                                                       mean, mul, a.cmul, a.q8, a.qscale, a.rowdot, sm.red, a.pre_q)
+        if (a.blkq == 128) SAGE_Q(128);
+        else if (a.blkq == 64) SAGE_Q(64);
+        else SAGE_Q(32);
+#undef SAGE_Q
+    } else if (r < a.nq_blk + a.nk_blk) {
+        const int t = r - a.nq_blk;
+        const float* mul = a.kmul + (int64_t)bh * D;
+        const float* mean = a.kmean + (int64_t)bh * D;
+#define SAGE_K(BLK) quant_i8_block<D, BLK, true, PRE>(t, h, b, a.k.p, a.k.sb, a.k.sh, a.k.sn, a.Nkv, a.H, a.nkv_pad, a.km, \
+                                                      mean, mul, 0.0f, a.k8, a.kscale, nullptr, sm.red, a.pre_k)
+        if (a.blkk == 128) SAGE_K(128);
+        else if (a.blkk == 64) SAGE_K(64);
+        else SAGE_K(32);
+#undef SAGE_K
+    } else {
+        quant_v_fp8_body<D>(r - a.nq_blk - a.nk_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km,
+                            a.vscale, a.v8, sm.tile8);
+    }
+}
+
+hipError_t launch_quant(const QuantArgs& a_in, int B, int D, hipStream_t st) {
+    QuantArgs a = a_in;
+    a.nq_blk = a.q8 != nullptr ? (int)(a.nq_pad / a.blkq) : 0;
+    a.nk_blk = a.k8 != nullptr ? (int)(a.nkv_pad / a.blkk) : 0;
+    a.nv_tile = a.v8 != nullptr ? (int)(a.nkv_pad / 64) : 0;
+    if (a.q8 != nullptr && a.nq_pad % a.blkq != 0) return hipErrorInvalidValue;
+    if (a.k8 != nullptr && a.nkv_pad % a.blkk != 0) return hipErrorInvalidValue;
+    const int64_t total = (int64_t)B * a.H * (a.nq_blk + a.nk_blk + a.nv_tile);
+    if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
+    dim3 grid((unsigned)total), block(256);
+    const bool has_pre = a.pre_q.gain != nullptr;
+    if (D == 128 && has_pre) hipLaunchKernelGGL((quant_kernel<128, true>), grid, block, 0, st, a);
+    else if (D == 128) hipLaunchKernelGGL((quant_kernel<128, false>), grid, block, 0, st, a);
+    else if (D == 64 && has_pre) hipLaunchKernelGGL((quant_kernel<64, true>), grid, block, 0, st, a);
+    else if (D == 64) hipLaunchKernelGGL((quant_kernel<64, false>), grid, block, 0, st, a);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 

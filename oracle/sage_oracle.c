@@ -551,8 +551,8 @@ int sage_oracle_quant_k(const uint16_t* k, int B, int H, int N, int D,
     return sage_oracle_quant_k_ch(k, B, H, N, D, st, kmean, NULL, 0, 0, blkk, npad_mult, k8, kscale);
 }
 
-int sage_oracle_quant_v_f16(const uint16_t* v, int B, int H, int N, int D,
-                            const int64_t* st, int npad_mult, uint16_t* v16) {
+int sage_oracle_quant_v_f16_masked(const uint16_t* v, int B, int H, int N, int D,
+                                   const int64_t* st, int mask_lo, int mask_hi, int npad_mult, uint16_t* v16) {
     if (bad_quant_args(v, B, H, N, D, st, 1, npad_mult) || !v16) return -1;
     int64_t npad = sage_oracle_pad(N, npad_mult);
     memset(v16, 0, (size_t)B * H * npad * D * 2);
@@ -564,9 +564,15 @@ int sage_oracle_quant_v_f16(const uint16_t* v, int B, int H, int N, int D,
         int b = (int)(w / ((int64_t)N * H));
         const uint16_t* src = v + b * st[0] + h * st[1] + (int64_t)s * st[2];
         uint16_t* dst = v16 + (((int64_t)b * H + h) * npad + s) * D;
+        if (!key_kept(s, N, mask_lo, mask_hi)) continue;          /* masked rows stay 0 */
         for (int d = 0; d < D; d++) dst[d] = sage_oracle_f32_to_f16(sage_oracle_bf16_to_f32(src[d * st[3]]));
     }
     return 0;
+}
+
+int sage_oracle_quant_v_f16(const uint16_t* v, int B, int H, int N, int D,
+                            const int64_t* st, int npad_mult, uint16_t* v16) {
+    return sage_oracle_quant_v_f16_masked(v, B, H, N, D, st, 0, 0, npad_mult, v16);
 }
 
 int sage_oracle_quant_v_fp8_masked(const uint16_t* v, int B, int H, int N, int D,
@@ -593,7 +599,7 @@ int sage_oracle_quant_v_fp8_masked(const uint16_t* v, int B, int H, int N, int D
         for (int s = 0; s < N; s++) {
             const uint16_t* src = v + b * st[0] + h * st[1] + (int64_t)s * st[2];
             uint8_t* dst = v8 + ((int64_t)w * npad + s) * D;
-            /* masked rows are encoded too (saturating): their probabilities are zero */
+            if (!key_kept(s, N, mask_lo, mask_hi)) continue;      /* masked rows stay 0 */
             for (int d = 0; d < D; d++)
                 dst[d] = sage_oracle_f32_to_e4m3(sage_oracle_bf16_to_f32(src[d * st[3]]) / vscale[w * D + d]);
         }
@@ -676,10 +682,13 @@ int sage_oracle_attn_ex(const int8_t* q8, const float* qscale, int blkq, int64_t
             for (int d = 0; d < D; d++) acc[d] = 0.0f;
             for (int j = 0; j < Nkv; j++) {
                 float p = exp2f(sc[j] - mref);
-                l += (double)p;
                 float pq = variant == 0
                     ? sage_oracle_f16_to_f32(sage_oracle_f32_to_f16(p))
                     : sage_oracle_e4m3_to_f32(sage_oracle_f32_to_e4m3(p * 448.0f));
+                /* The e4m3 variant normalises by the sum of the ROUNDED probabilities (the weights
+                 * the product really uses): a row dominated by one key then returns that key's V
+                 * exactly, whatever the rounding of its probability. */
+                l += variant == 0 ? (double)p : (double)pq / 448.0;
                 if (pq == 0.0f) continue;
                 const float* vr = vf + (bh * NkvPad + j) * D;
                 for (int d = 0; d < D; d++) acc[d] += pq * vr[d];
@@ -761,7 +770,7 @@ int sage_oracle_sdpa_bf16_ex(const uint16_t* q, const uint16_t* k, const uint16_
         if (!rc) rc = sage_oracle_quant_q_ch(q, B, H, Nq, D, qs, scale, qmul, blkq, blkq, q8, qsc);
         if (!rc) rc = sage_oracle_quant_k_ch(k, B, H, Nkv, D, ks, mu, kmul, mask_lo, mask_hi, blkk, blkk, k8, ksc);
         if (!rc) rc = variant == 0
-            ? sage_oracle_quant_v_f16(v, B, H, Nkv, D, vs, blkk, (uint16_t*)vq)
+            ? sage_oracle_quant_v_f16_masked(v, B, H, Nkv, D, vs, mask_lo, mask_hi, blkk, (uint16_t*)vq)
             : sage_oracle_quant_v_fp8_masked(v, B, H, Nkv, D, vs, mask_lo, mask_hi, blkk, (uint8_t*)vq, vsc);
         if (!rc && stats) rowdot_q(q, B, H, Nq, D, qs, scale, mu, nqp, shift);
         if (!rc) rc = sage_oracle_attn_ex(q8, qsc, blkq, nqp, k8, ksc, blkk, nkp, vq, vsc, variant,

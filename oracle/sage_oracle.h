@@ -161,7 +161,11 @@ int sage_oracle_quant_v_fp8(const uint16_t* v, int B, int H, int N, int D,
                             const int64_t* strides, int npad_mult,
                             uint8_t* v8, float* vscale);
 
-/* The same with the channel maximum taken over the kept keys only. */
+/* The same with masked rows (mask_lo <= s < mask_hi) left 0. */
+int sage_oracle_quant_v_f16_masked(const uint16_t* v, int B, int H, int N, int D,
+                                   const int64_t* strides, int mask_lo, int mask_hi, int npad_mult, uint16_t* v16);
+
+/* The same with the channel maximum taken over the kept keys only and masked rows left 0. */
 int sage_oracle_quant_v_fp8_masked(const uint16_t* v, int B, int H, int N, int D,
                                    const int64_t* strides, int mask_lo, int mask_hi, int npad_mult,
                                    uint8_t* v8, float* vscale);
@@ -169,7 +173,7 @@ int sage_oracle_quant_v_fp8_masked(const uint16_t* v, int B, int H, int N, int D
 /* ---- quantized attention ------------------------------------------------ */
 /* s[i,j] = float(sum_d q8*k8) * (qscale*kscale)   (log2 domain)
  * variant 0: p = exp2(s - max_j s), P16 = f16(p), O = sum P16*V16 / sum p
- * variant 1: p = exp2(s - ceil(max_j s)), P8 = e4m3(p*448), O = sum P8*V8 * vscale / (448 * sum p)
+ * variant 1: p = exp2(s - ceil(max_j s)), P8 = e4m3(p*448), O = sum P8*V8 * vscale / sum P8
  *            (an integer reference: shifting it by a whole number only moves the exponent of
  *            every probability, so their e4m3 significands do not depend on which integer an
  *            implementation that walks the keys in tiles happens to hold)

@@ -70,6 +70,9 @@ def lib():
         L.sage_oracle_quant_k_ch.restype = ctypes.c_int
         L.sage_oracle_quant_k_ch.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p, ctypes.c_void_p] + [
                                              ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_quant_v_f16_masked.restype = ctypes.c_int
+        L.sage_oracle_quant_v_f16_masked.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p] + [ctypes.c_int] * 3 + [
+                                                     ctypes.c_void_p]
         L.sage_oracle_quant_v_fp8_masked.restype = ctypes.c_int
         L.sage_oracle_quant_v_fp8_masked.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p] + [ctypes.c_int] * 3 + [
                                                      ctypes.c_void_p, ctypes.c_void_p]
@@ -321,12 +324,12 @@ def quant_k(k_bf16, mu, blkk, npad_mult=None):
     return k8, sc
 
 
-def quant_v_f16(v_bf16, npad_mult):
+def quant_v_f16(v_bf16, npad_mult, mask_lo=0, mask_hi=0):
     v = np.ascontiguousarray(v_bf16, dtype=np.uint16)
     B, S, H, D = v.shape
     v16 = np.empty((B, H, pad(S, npad_mult), D), np.uint16)
-    _chk(lib().sage_oracle_quant_v_f16(_p(v), B, H, S, D, strides_bshd(S, H, D), npad_mult, _p(v16)),
-         "quant_v_f16")
+    _chk(lib().sage_oracle_quant_v_f16_masked(_p(v), B, H, S, D, strides_bshd(S, H, D), mask_lo, mask_hi,
+                                              npad_mult, _p(v16)), "quant_v_f16")
     return v16
 
 

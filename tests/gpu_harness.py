@@ -46,7 +46,7 @@ def tile_v(v_plain, variant):
 
 
 def quant_qk(q_bits, k_bits, scale, blkq, blkk, smooth_k, strides_q=None, strides_k=None,
-             q_off=0, k_off=0, shape=None):
+             q_off=0, k_off=0, shape=None, balance=True, mask=(0, 0)):
     """q_bits/k_bits: uint16 [B,S,H,D] (or any buffer when shape/strides are given).
     Returns dict of numpy arrays in the padded device layouts."""
     L = _lib.lib()
@@ -63,40 +63,60 @@ def quant_qk(q_bits, k_bits, scale, blkq, blkk, smooth_k, strides_q=None, stride
     k8 = torch.full((B, H, nkp, D), 77, dtype=torch.int8, device="cuda")
     qs = torch.full((B, H, nqp // blkq), -1.0, dtype=torch.float32, device="cuda")
     ks = torch.full((B, H, nkp // blkk), -1.0, dtype=torch.float32, device="cuda")
-    km = torch.full((B, H, D), -1.0, dtype=torch.float32, device="cuda")
+    km, qm, kmu = (torch.full((B, H, D), -1.0, dtype=torch.float32, device="cuda") for _ in range(3))
     nscr = L.mi355_sage_quant_scratch_bytes(B, H, Skv, D)
-    scr = torch.empty(max(nscr, 8), dtype=torch.uint8, device="cuda")
+    scr = torch.full((max(nscr, 8),), 0xAB, dtype=torch.uint8, device="cuda")
+    flags = (_lib.K_SMOOTH if smooth_k else 0) | (_lib.K_BALANCE if balance else 0)
     rc = L.mi355_sage_quant_qk_bf16(qd.data_ptr(), kd.data_ptr(), B, H, Sq, Skv, D, scale,
-                                    strides_q, strides_k, q_off, k_off, blkq, blkk, int(smooth_k),
+                                    strides_q, strides_k, q_off, k_off, blkq, blkk, flags, mask[0], mask[1],
                                     q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(),
-                                    km.data_ptr() if smooth_k else None, scr.data_ptr(), scr.numel(), stream())
+                                    km.data_ptr(), qm.data_ptr(), kmu.data_ptr(), scr.data_ptr(), scr.numel(), stream())
     assert rc == 0, rc
     torch.cuda.synchronize()
     return dict(q8=q8.cpu().numpy(), qscale=qs.cpu().numpy(), k8=k8.cpu().numpy(), kscale=ks.cpu().numpy(),
-                kmean=km.cpu().numpy(), dev=dict(q8=q8, qscale=qs, k8=k8, kscale=ks, kmean=km))
+                kmean=km.cpu().numpy(), qmul=qm.cpu().numpy(), kmul=kmu.cpu().numpy(),
+                dev=dict(q8=q8, qscale=qs, k8=k8, kscale=ks, kmean=km, qmul=qm, kmul=kmu))
 
 
-def quant_v(v_bits, variant):
+def oracle_quant_qk(oracle, q_bits, k_bits, scale, blkq, blkk, smooth_k=True, balance=True, mask=(0, 0)):
+    """The CPU checker's statistics and codes in the device's padded layouts."""
     L = _lib.lib()
-    B, S, H, D = v_bits.shape
+    flags = (1 if smooth_k else 0) | (2 if balance else 0)
+    mu, qmul, kmul = oracle.kstats(k_bits, scale, flags, *mask)
+    q8, qs = oracle.quant_q_ch(q_bits, scale, qmul, blkq, int(L.mi355_sage_pad_q(1)))
+    k8, ks = oracle.quant_k_ch(k_bits, mu, kmul, blkk, 128, *mask)
+    return dict(q8=q8, qscale=qs, k8=k8, kscale=ks, kmean=mu, qmul=qmul, kmul=kmul)
+
+
+def quant_v(v_bits, variant, mask=(0, 0), strides=None, v_off=0, shape=None):
+    L = _lib.lib()
+    if shape is None:
+        B, S, H, D = v_bits.shape
+        st = _lib.strides_bhnd(S, H, D)
+    else:
+        B, H, S, D = shape
+        st = strides
     vd = dev_bf16(v_bits)
     nkp = L.mi355_sage_pad_kv(S)
-    st = _lib.strides_bhnd(S, H, D)
     if variant == 0:
         out = torch.full((B, H, nkp // 64, D, 64), 0x7E00, dtype=torch.int16, device="cuda")
-        rc = L.mi355_sage_quant_v_f16(vd.data_ptr(), B, H, S, D, st, 0, out.data_ptr(), stream())
+        rc = L.mi355_sage_quant_v_f16(vd.data_ptr(), B, H, S, D, st, v_off, mask[0], mask[1], out.data_ptr(), stream())
         assert rc == 0, rc
         torch.cuda.synchronize()
         return dict(vq=out.cpu().numpy().view(np.uint16), vscale=None, dev=dict(vq=out, vscale=None))
     out = torch.full((B, H, nkp // 64, D, 64), 0x7F, dtype=torch.uint8, device="cuda")
     vs = torch.full((B, H, D), -1.0, dtype=torch.float32, device="cuda")
-    rc = L.mi355_sage_quant_v_fp8(vd.data_ptr(), B, H, S, D, st, 0, out.data_ptr(), vs.data_ptr(), stream())
+    nscr = L.mi355_sage_quant_scratch_bytes(B, H, S, D)
+    scr = torch.full((max(nscr, 8),), 0xAB, dtype=torch.uint8, device="cuda")
+    rc = L.mi355_sage_quant_v_fp8(vd.data_ptr(), B, H, S, D, st, v_off, mask[0], mask[1], out.data_ptr(), vs.data_ptr(),
+                                  scr.data_ptr(), scr.numel(), stream())
     assert rc == 0, rc
     torch.cuda.synchronize()
     return dict(vq=out.cpu().numpy(), vscale=vs.cpu().numpy(), dev=dict(vq=out, vscale=vs))
 
 
-def attn_fwd(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv, kv_valid=None, want_stats=False):
+def attn_fwd(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv, kv_valid=None, want_stats=False,
+             mask=(0, 0), qshift=None):
     """Device tensors in the device layouts.  Returns (o bits uint16 [B,Sq,H,D], stats or None)."""
     L = _lib.lib()
     B, H, _, D = q8.shape
@@ -104,7 +124,8 @@ def attn_fwd(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv, k
     stats = torch.zeros((B, H, Sq), dtype=torch.float32, device="cuda") if want_stats else None
     rc = L.mi355_sage_attn_fwd(q8.data_ptr(), qscale.data_ptr(), blkq, k8.data_ptr(), kscale.data_ptr(), blkk,
                                vq.data_ptr(), vscale.data_ptr() if vscale is not None else None, variant,
-                               B, H, Sq, Skv, kv_valid or Skv, D, o.data_ptr(), _lib.strides_bhnd(Sq, H, D), 0,
+                               B, H, Sq, Skv, kv_valid or Skv, mask[0], mask[1], D, o.data_ptr(),
+                               _lib.strides_bhnd(Sq, H, D), 0, qshift.data_ptr() if qshift is not None else None,
                                stats.data_ptr() if want_stats else None, stream())
     assert rc == 0, rc
     torch.cuda.synchronize()

@@ -129,8 +129,9 @@ def _pad_tokens(x, npad_mult):
     return out
 
 
-def quant_v_f16(v_bits_bshd, npad_mult):
+def quant_v_f16(v_bits_bshd, npad_mult, mask_lo=0, mask_hi=0):
     x = bf16_to_f32(v_bits_bshd).transpose(0, 2, 1, 3)
+    x = np.where(keep_mask(x.shape[2], mask_lo, mask_hi)[None, None, :, None], x, np.float32(0.0))
     with np.errstate(over="ignore"):
         h = np.clip(x, -65504.0, 65504.0).astype(np.float16)
     return _pad_tokens(h.view(np.uint16), npad_mult)
@@ -140,17 +141,19 @@ def quant_v_fp8(v_bits_bshd, npad_mult, mask_lo=0, mask_hi=0):
     x = bf16_to_f32(v_bits_bshd).transpose(0, 2, 1, 3)
     amax = np.abs(x[:, :, keep_mask(x.shape[2], mask_lo, mask_hi), :]).max(axis=2).astype(np.float32)
     sc = np.where(amax > 0, amax / np.float32(448.0), np.float32(1.0)).astype(np.float32)
-    y = np.clip((x / sc[:, :, None, :]).astype(np.float32), -448.0, 448.0)     # masked rows may exceed the scale
+    y = (x / sc[:, :, None, :]).astype(np.float32)
+    y = np.where(keep_mask(x.shape[2], mask_lo, mask_hi)[None, None, :, None], y, np.float32(0.0))   # masked rows stay 0
     b = torch.from_numpy(np.ascontiguousarray(y)).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
     return _pad_tokens(b, npad_mult), sc
 
 
 def attn_float64(q8, qs, blkq, k8, ks, blkk, v_f32, Sq, Skv, p_codec, integer_reference=False,
-                 mask_lo=0, mask_hi=0, addmask=None):
+                 mask_lo=0, mask_hi=0, addmask=None, normalise_by_rounded=False):
     """Quantized attention in float64 from the quantized tensors.
     v_f32: decoded V [B,H,Skv_pad,D] (already multiplied by any per-channel scale).
     p_codec: function rounding p (float32 array in [0,1]) to the P*V operand grid.
     integer_reference: exponentials against ceil(row maximum) instead of the row maximum.
+    normalise_by_rounded: divide by the sum of the rounded probabilities instead of the exact ones.
     addmask: [B,H,Sq,Skv] natural-log bias."""
     B, H, _, D = q8.shape
     out = np.zeros((B, Sq, H, D))
@@ -168,8 +171,9 @@ def attn_float64(q8, qs, blkq, k8, ks, blkk, v_f32, Sq, Skv, p_codec, integer_re
             if integer_reference:
                 ref = np.ceil(ref)
             p = np.exp2((s - ref).astype(np.float32)).astype(np.float32)
-            l = p.astype(np.float64).sum(axis=1, keepdims=True)
-            out[b, :, h, :] = (p_codec(p).astype(np.float64) @ v_f32[b, h, :Skv].astype(np.float64)) / l
+            pr = p_codec(p).astype(np.float64)
+            l = (pr if normalise_by_rounded else p.astype(np.float64)).sum(axis=1, keepdims=True)
+            out[b, :, h, :] = (pr @ v_f32[b, h, :Skv].astype(np.float64)) / l
     return out
 
 

@@ -94,3 +94,11 @@ def test_host_mirror_error_strings():
         A.sdpa_flash_fwd_padmask(qb, qb, qb, 0, 0.1)
     with pytest.raises(A.Error, match="no CPU fallback"):
         A.sdpa_nomask(qb, qb, qb, 0.1)
+    with pytest.raises(A.Error, match="sdpa_nomask_tiled: q/k/v dtype mismatch"):
+        A.sdpa_nomask_tiled(q, qb, q, 0.1)
+    with pytest.raises(A.Error, match="sdpa_qwen_keymask: real_txt_len out of range"):
+        A.sdpa_qwen_keymask(qb, qb, qb, 64, 65, 0.1)
+    with pytest.raises(A.Error, match="sdpa_qwen_keymask: N_TXT must be <= S"):
+        A.sdpa_qwen_keymask(qb, qb, qb, 129, 5, 0.1)
+    with pytest.raises(A.Error, match="sdpa_qwen_keymask: k/v shape mismatch"):
+        A.sdpa_qwen_keymask(qb, qb[:, :64], qb, 64, 5, 0.1)

@@ -13,27 +13,30 @@ MAX_ABS = 2e-2
 COS = 0.999
 
 
-def _oracle_quantized(oracle, q, k, v, w, variant):
-    q8, qs = oracle.quant_q(q, w.scale, w.blkq, int(_lib.lib().mi355_sage_pad_q(1)))
-    k8, ks = oracle.quant_k(k, oracle.kmean(k), w.blkk, 128)
+def _oracle_quantized(oracle, q, k, v, w, variant, mask=(0, 0)):
+    import gpu_harness as H
+    g = H.oracle_quant_qk(oracle, q, k, w.scale, w.blkq, w.blkk, True, True, mask)
     if variant == 0:
-        vq, vs = oracle.quant_v_f16(v, 128), None
+        vq, vs = oracle.quant_v_f16(v, 128, *mask), None
     else:
-        vq, vs = oracle.quant_v_fp8(v, 128)
-    return q8, qs, k8, ks, vq, vs
+        vq, vs = oracle.quant_v_fp8(v, 128, *mask)
+    return g["q8"], g["qscale"], g["k8"], g["kscale"], vq, vs
 
 
-@pytest.mark.parametrize("wid,variant,S", [(1, 0, 1024), (2, 0, 640), (2, 0, 200), (3, 0, 333), (4, 1, 640),
-                                           (2, 1, 200), (1, 1, 1024)])
-def test_attn_kernel_on_checker_quantized_tensors(oracle, wid, variant, S):
+@pytest.mark.parametrize("wid,variant,S,mask", [(1, 0, 1024, (0, 0)), (2, 0, 640, (0, 0)), (2, 0, 200, (0, 0)),
+                                                (3, 0, 333, (0, 0)), (4, 1, 640, (0, 0)), (2, 1, 200, (0, 0)),
+                                                (1, 1, 1024, (0, 0)), (2, 0, 640, (100, 300)), (4, 1, 333, (0, 70)),
+                                                (2, 0, 700, (128, 512)), (2, 1, 200, (150, 200))])
+def test_attn_kernel_on_checker_quantized_tensors(oracle, wid, variant, S, mask):
     """Feeds the kernel the CPU checker's own quantized tensors, so only the
-    attention arithmetic differs."""
+    attention arithmetic differs.  Masked key ranges start inside, cover whole, and end
+    inside 64-key tiles, including the first tile and the ragged last one."""
     import torch
     import gpu_harness as H
     w = WORKLOADS[wid].scaled(B=1, H=2, S=S)
     q, k, v = make_inputs(w)
-    q8, qs, k8, ks, vq, vs = _oracle_quantized(oracle, q, k, v, w, variant)
-    want16, want32 = oracle.attn(q8, qs, w.blkq, k8, ks, w.blkk, vq, vs, variant, S, S)
+    q8, qs, k8, ks, vq, vs = _oracle_quantized(oracle, q, k, v, w, variant, mask)
+    want16, want32 = oracle.attn(q8, qs, w.blkq, k8, ks, w.blkk, vq, vs, variant, S, S, *mask)
     L = _lib.lib()
     nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
     def padded(x, n, fill):
@@ -47,14 +50,14 @@ def test_attn_kernel_on_checker_quantized_tensors(oracle, wid, variant, S):
     vt = H.tile_v(padded(vq, nkp, 0), variant)
     dv = torch.from_numpy(vt.view(np.int16) if variant == 0 else vt).cuda()
     dvs = torch.from_numpy(vs).cuda() if vs is not None else None
-    got, _ = H.attn_fwd(dq8, dqs, w.blkq, dk8, dks, w.blkk, dv, dvs, variant, S, S)
+    got, _ = H.attn_fwd(dq8, dqs, w.blkq, dk8, dks, w.blkk, dv, dvs, variant, S, S, mask=mask)
     cos, mx = H.cos_maxabs(bf16_bits_to_f32(got), want32)
-    # e4m3 P carries 2^-4 relative rounding noise, and the kernel rounds p relative to the
-    # running maximum while the checker rounds relative to the final one
-    assert mx <= MAX_ABS and cos >= (0.9999 if variant == 0 else 0.999), (cos, mx)
+    # both variants round every probability to the same significand as the checker (the e4m3
+    # variant through its whole-number reference), so they agree far inside the 2e-2 bar
+    assert mx <= MAX_ABS and cos >= 0.9999, (cos, mx)
 
 
-def _one_shot(q, k, v, scale, variant, blkq=None, blkk=64, smooth=True):
+def _one_shot(q, k, v, scale, variant, blkq=None, blkk=64, smooth=True, balance=True):
     import torch
     import gpu_harness as H
     L = _lib.lib()
@@ -69,7 +72,7 @@ def _one_shot(q, k, v, scale, variant, blkq=None, blkk=64, smooth=True):
     else:
         rc = L.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), B, Hh, Sq, Skv, D,
                                        scale, qs, ks, ks, qs, 0, 0, 0, 0, 0, H.stream(), variant, blkq, blkk,
-                                       int(smooth), None, 0)
+                                       (1 if smooth else 0) | (2 if balance else 0), None, 0)
     assert rc == 0, rc
     torch.cuda.synchronize()
     return H.to_bits(o)
@@ -87,30 +90,29 @@ def test_one_shot_matches_checker_and_referee(oracle, wid, S):
     assert mx <= MAX_ABS, (cos, mx)
     ref = oracle.sdpa_f32(bf16_bits_to_f32(q), bf16_bits_to_f32(k), bf16_bits_to_f32(v), w.scale)
     cos_ref, mx_ref = H.cos_maxabs(bf16_bits_to_f32(got), ref)
-    # workload 3's zero-mean outlier channels put the recipe itself at ~0.9986 (see the CPU test)
-    assert cos_ref >= (0.998 if wid == 3 else COS), (cos_ref, mx_ref)
+    assert cos_ref >= COS, (cos_ref, mx_ref)
 
 
 @pytest.mark.parametrize("wid,S,smooth", [(2, 1100, True), (1, 1024, True), (3, 333, False), (1, 77, True)])
 def test_one_shot_equals_stage_pipeline(wid, S, smooth):
-    """The one-shot call runs fused launches (Q quantize + V repack + K-mean sums in one kernel,
-    K mean + K quantize in another); the stage entry points run them separately.  The stage
-    outputs are proven bit-exact against the CPU checker, so bit-equal O from both routes
-    carries that proof over to the fused kernels."""
+    """The one-shot call runs the V passes and the K statistics as roles of one launch and the
+    three encoders as roles of another; the stage entry points run subsets of those roles.  The
+    stage outputs are proven bit-exact against the CPU checker, so bit-equal O from both routes
+    carries that proof over to the one-shot call."""
     import torch
     import gpu_harness as H
     w = WORKLOADS[wid]
     w = w.scaled(B=2, H=3, S=S)
     q, k, v = make_inputs(w)
-    got = _one_shot(q, k, v, w.scale, 0, w.blkq, w.blkk, smooth)
-    g = H.quant_qk(q, k, w.scale, w.blkq, w.blkk, smooth)["dev"]
+    got = _one_shot(q, k, v, w.scale, 0, w.blkq, w.blkk, smooth, balance=(wid != 1))
+    g = H.quant_qk(q, k, w.scale, w.blkq, w.blkk, smooth, balance=(wid != 1))["dev"]
     gv = H.quant_v(v, 0)["dev"]
     staged, _ = H.attn_fwd(g["q8"], g["qscale"], w.blkq, g["k8"], g["kscale"], w.blkk, gv["vq"], None, 0, S, S)
     np.testing.assert_array_equal(got, staged)
 
 
 def test_default_recipe_entry_point(oracle):
-    """mi355_sage_sdpa_bf16 without the recipe arguments: blkq 128 / blkk 64 / smoothing on."""
+    """mi355_sage_sdpa_bf16 without the recipe arguments: blkq 128 / blkk 64 / smoothing and balancing on."""
     import gpu_harness as H
     w = WORKLOADS[2].scaled(B=2, H=2, S=384)
     q, k, v = make_inputs(w)
@@ -154,7 +156,17 @@ def test_reference_maximum_keeps_rising(oracle, variant):
     """Keys grow along the sequence, so the row maximum rises from tile to tile by far more
     than the kernel's lazy-refresh margin: every path that repairs a stale reference
     maximum (refresh + accumulator rescale, redo of an optimistic tile) is exercised, in
-    interior tiles, repeatedly.  The second case puts one huge key in the middle."""
+    interior tiles, repeatedly.  The second case puts one huge key in the middle.
+
+    Nearly every row here is dominated by one or two keys.  The fp16 variant stays inside the
+    2e-2 bar everywhere.  For the e4m3 variant kernel and checker follow the same rule (whole-
+    number reference, normaliser over the rounded probabilities), but they evaluate exp2 with
+    different last bits, so a probability within ~1e-4 (relative) of an e4m3 rounding boundary
+    is rounded the other way by one of them: one weight moves by one e4m3 step (2^-3 .. 2^-4
+    relative), which in a row carried by two keys a and b shows as up to 2^-4 |v_a - v_b|.  (The
+    scores here are ~25 times larger than on real inputs and the last bits of the exponent
+    argument scale with them, so such flips are ~100 times more frequent than usual.)  The
+    test therefore holds 99 % of the elements to the 2e-2 bar and all of them to that bound."""
     import gpu_harness as H
     w = WORKLOADS[2].scaled(B=1, H=2, S=1024, k_offset_std=0.0)
     q, k, v = make_inputs(w)
@@ -168,9 +180,14 @@ def test_reference_maximum_keeps_rising(oracle, variant):
         got = _one_shot(q, kk, v, w.scale, variant, 128, 64, smooth=False)
         _, want32 = oracle.sdpa_bf16(q, kk, v, w.scale, variant=variant, blkq=128, blkk=64, smooth_k=False)
         cos, mx = H.cos_maxabs(bf16_bits_to_f32(got), want32)
-        # here the softmax is nearly one-hot and |O| reaches |V| ~ 4, so the 2^-4 relative rounding of an
-        # e4m3 probability shows up as up to ~0.1 absolute; the fp16 variant stays inside the 2e-2 bar
-        assert mx <= (MAX_ABS if variant == 0 else 1e-1) and cos >= (0.9999 if variant == 0 else 0.999), (cos, mx)
+        assert cos >= 0.9999, (cos, mx)
+        if variant == 0:
+            assert mx <= MAX_ABS, (cos, mx)
+        else:
+            diff = np.abs(bf16_bits_to_f32(got).astype(np.float64) - want32)
+            vf = bf16_bits_to_f32(v)
+            assert np.quantile(diff, 0.99) <= MAX_ABS, np.quantile(diff, 0.99)
+            assert mx <= 2.0 ** -4 * (vf.max() - vf.min()), (mx, vf.max() - vf.min())
         assert np.isfinite(bf16_bits_to_f32(got)).all()
 
 
@@ -198,6 +215,156 @@ def test_train_fwd_stats_and_padmask(oracle):
     ref = oracle.sdpa_f32(qf[:, :real], kf[:, :real], vf[:, :real], w.scale)
     cos, mx = H.cos_maxabs(pm.o.float().cpu().numpy()[:, :real], ref)
     assert cos >= COS, (cos, mx)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_stats_rect_f32_and_both_variants(oracle, variant):
+    """sdpa_flash_train_fwd_rect (Sq != Skv, with Stats) and sdpa_flash_train_fwd_f32, for the
+    fp16 and the e4m3 variant: O against the CPU checker, Stats against the checker's and against
+    the log-sum-exp of the fp32 referee."""
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    w = WORKLOADS[2].scaled(B=2, H=2, S=320)
+    q, k, v = make_inputs(w)
+    q = np.ascontiguousarray(q[:, :200])                               # Sq = 200, Skv = 320
+    qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
+    fwd = A.sdpa_flash_train_fwd_rect(qd, kd, vd, w.scale, variant)
+    torch.cuda.synchronize()
+    assert fwd.stats.shape == (w.B, w.H, 200, 1) and fwd.o.shape == qd.shape
+    blkq = 128 if variant == 0 else 32
+    _, want32, want_stats = oracle.sdpa_bf16(q, k, v, w.scale, variant=variant, blkq=blkq, blkk=64, want_stats=True)
+    cos, mx = H.cos_maxabs(fwd.o.float().cpu().numpy(), want32)
+    assert mx <= MAX_ABS and cos >= 0.9999, (cos, mx)
+    # (e4m3: the normaliser sums rounded probabilities, a few of which round the other way in the checker)
+    np.testing.assert_allclose(fwd.stats.cpu().numpy()[..., 0], want_stats, atol=2e-3 if variant == 0 else 1e-2)
+    qf, kf, vf = (bf16_bits_to_f32(x) for x in (q, k, v))
+    ref, lse = oracle.sdpa_f32(qf, kf, vf, w.scale, want_stats=True)
+    np.testing.assert_allclose(fwd.stats.cpu().numpy()[..., 0], lse, atol=3e-2)
+    cos, mx = H.cos_maxabs(fwd.o.float().cpu().numpy(), ref)
+    assert cos >= COS, (cos, mx)
+    # F32 activations: cast to bf16 at the boundary, attend, cast back
+    sq = qd[:, :, :, :].float()
+    att, fwd32 = A.sdpa_flash_train_fwd_f32(kd.float(), kd.float(), vd.float(), w.scale, variant)
+    same = A.sdpa_flash_train_fwd(kd, kd, vd, w.scale, variant)
+    torch.cuda.synchronize()
+    assert att.dtype == torch.float32 and sq.dtype == torch.float32
+    np.testing.assert_array_equal(att.cpu().numpy(), same.o.float().cpu().numpy())
+    np.testing.assert_array_equal(fwd32.stats.cpu().numpy(), same.stats.cpu().numpy())
+
+
+@pytest.mark.parametrize("variant,S,n_txt,real", [(0, 600, 256, 100), (1, 600, 256, 100), (0, 333, 128, 0),
+                                                  (0, 520, 200, 200), (1, 450, 450, 77)])
+def test_qwen_keymask(oracle, variant, S, n_txt, real):
+    """sdpa_qwen_keymask: text keys [real, n_txt) masked, image keys kept.  Against the CPU
+    checker with the same mask, against the checker on the tensors with the masked keys removed
+    (same result whenever the cut falls on block boundaries; always within the bar), and
+    against the fp32 referee.  real == n_txt is no mask at all."""
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    w = WORKLOADS[2].scaled(B=1, H=2, S=S)
+    q, k, v = make_inputs(w)
+    # what sits in the padded text rows must not matter: make it large
+    kx, vx = bf16_bits_to_f32(k), bf16_bits_to_f32(v)
+    kx[:, real:n_txt] *= 30.0
+    vx[:, real:n_txt] += 100.0
+    k, v = f32_to_bf16_bits(kx), f32_to_bf16_bits(vx)
+    qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
+    got = A.sdpa_qwen_keymask(qd, kd, vd, n_txt, real, w.scale, variant)
+    torch.cuda.synchronize()
+    gotf = got.float().cpu().numpy()
+    blkq = 128 if variant == 0 else 32
+    _, want32 = oracle.sdpa_bf16(q, k, v, w.scale, variant=variant, blkq=blkq, blkk=64, mask_lo=real, mask_hi=n_txt)
+    cos, mx = H.cos_maxabs(gotf, want32)
+    assert mx <= MAX_ABS and cos >= 0.9999, (cos, mx)
+    keep = np.r_[0:real, n_txt:S]
+    ref = oracle.sdpa_f32(bf16_bits_to_f32(q), bf16_bits_to_f32(k)[:, keep], bf16_bits_to_f32(v)[:, keep], w.scale)
+    cos, mx = H.cos_maxabs(gotf, ref)
+    # (few keys make a peaked softmax, where single e4m3 probabilities show)
+    assert cos >= COS and mx <= (4e-2 if variant == 0 else 8e-2), (cos, mx)
+    if real == n_txt:
+        np.testing.assert_array_equal(H.to_bits(got), H.to_bits(A.sdpa_nomask(qd, kd, vd, w.scale, variant)))
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_one_shot_bhsd_memory_and_offsets_for_every_tensor(oracle, variant):
+    """Q, K, V and O all in head-major [B,H,S,D] memory at non-zero element offsets inside
+    larger buffers, Stats at an offset too: same bits as the plain BSHD call."""
+    import ctypes
+    import torch
+    import gpu_harness as H
+    L = _lib.lib()
+    w = WORKLOADS[2].scaled(B=2, H=3, S=300)
+    q, k, v = make_inputs(w)
+    want = _one_shot(q, k, v, w.scale, variant)
+    B, S, Hh, D = w.B, w.S, w.H, w.D
+    offs = dict(q=64, k=128, v=8, o=200)
+
+    def bhsd_buf(x, off):
+        flat = torch.zeros(off + x.size + 64, dtype=torch.bfloat16, device="cuda")
+        flat[off:off + x.size] = H.dev_bf16(np.ascontiguousarray(x.transpose(0, 2, 1, 3))).reshape(-1)
+        return flat
+    qb, kb, vb = bhsd_buf(q, offs["q"]), bhsd_buf(k, offs["k"]), bhsd_buf(v, offs["v"])
+    ob = torch.zeros(offs["o"] + q.size + 64, dtype=torch.bfloat16, device="cuda")
+    stats = torch.zeros(16 + B * Hh * S, dtype=torch.float32, device="cuda")
+    st = (ctypes.c_int64 * 4)(Hh * S * D, S * D, D, 1)
+    rc = L.mi355_sage_sdpa_bf16_train_fwd(qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(), stats.data_ptr(),
+                                          B, Hh, S, S, D, w.scale, st, st, st, st, offs["q"], offs["k"], offs["v"],
+                                          offs["o"], 16, 0, S, S, H.stream(), variant, None, 0)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    got = ob[offs["o"]:offs["o"] + q.size].reshape(B, Hh, S, D).permute(0, 2, 1, 3)
+    np.testing.assert_array_equal(H.to_bits(got), want)
+    assert not ob[:offs["o"]].any() and not ob[offs["o"] + q.size:].any()      # nothing written outside O
+    assert not stats[:16].any() and stats[16:].abs().min() > 0
+    # rows that are not 16-byte aligned are refused before anything is launched
+    assert L.mi355_sage_sdpa_bf16_train_fwd(qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(), stats.data_ptr(),
+                                            B, Hh, S, S, D, w.scale, st, st, st, st, offs["q"], offs["k"], 3,
+                                            offs["o"], 16, 0, S, S, H.stream(), variant, None, 0) == -2
+    bad = (ctypes.c_int64 * 4)(Hh * S * D, S * D, D + 4, 1)
+    assert L.mi355_sage_sdpa_bf16_train_fwd(qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), ob.data_ptr(), stats.data_ptr(),
+                                            B, Hh, S, S, D, w.scale, st, st, st, bad, offs["q"], offs["k"], offs["v"],
+                                            offs["o"], 16, 0, S, S, H.stream(), variant, None, 0) == -2
+
+
+def test_internal_workspace_is_per_stream():
+    """workspace == NULL on two streams: the calls get separate buffers, so the interleaved
+    results equal the single-stream ones bit for bit; growth inside a capture is refused."""
+    import torch
+    import gpu_harness as H
+    L = _lib.lib()
+    w = WORKLOADS[2].scaled(B=1, H=2, S=512)
+    q, k, v = (H.dev_bf16(x) for x in make_inputs(w))
+    q2, k2, v2 = q.flip(1).contiguous(), k.flip(1).contiguous(), v.flip(1).contiguous()
+    st = _lib.strides_bhnd(w.S, w.H, w.D)
+
+    def call(qq, kk, vv, out, stream, S=w.S, strides=st):
+        return L.mi355_sage_sdpa_bf16(qq.data_ptr(), kk.data_ptr(), vv.data_ptr(), out.data_ptr(), w.B, w.H, S, S, w.D,
+                                      w.scale, strides, strides, strides, strides, 0, 0, 0, 0, 0, stream, 0, None, 0)
+    ref1, ref2 = torch.empty_like(q), torch.empty_like(q)
+    assert call(q, k, v, ref1, H.stream()) == 0 and call(q2, k2, v2, ref2, H.stream()) == 0
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    o1, o2 = torch.empty_like(q), torch.empty_like(q)
+    for _ in range(8):
+        assert call(q, k, v, o1, s1.cuda_stream) == 0
+        assert call(q2, k2, v2, o2, s2.cuda_stream) == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(H.to_bits(o1), H.to_bits(ref1))
+    np.testing.assert_array_equal(H.to_bits(o2), H.to_bits(ref2))
+    # a stream that is being captured cannot grow its buffer: -3, and the capture stays usable
+    s3 = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s3):
+        big = torch.zeros((1, 2048, w.H, w.D), dtype=torch.bfloat16, device="cuda")
+        obig = torch.empty_like(big)
+        stb = _lib.strides_bhnd(2048, w.H, w.D)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=s3):
+            rc = call(big, big, big, obig, torch.cuda.current_stream().cuda_stream, 2048, stb)
+            obig.zero_()
+    assert rc == -3, rc
 
 
 def test_host_mirror_dtypes_and_workspace_reuse(oracle):
@@ -283,7 +450,7 @@ def _one_shot_dev(q, k, v, w):
     st = _lib.strides_bhnd(w.S, w.H, w.D)
     rc = L.mi355_sage_sdpa_bf16_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), w.B, w.H, w.S, w.S, w.D,
                                    w.scale, st, st, st, st, 0, 0, 0, 0, 0, H.stream(), w.variant, w.blkq, w.blkk,
-                                   1, None, 0)
+                                   _lib.K_SMOOTH | _lib.K_BALANCE, None, 0)
     assert rc == 0, rc
     torch.cuda.synchronize()
     return o
@@ -317,11 +484,9 @@ def test_full_size_properties(wid):
         worst_cos = min(worst_cos, cos)
         worst_abs = max(worst_abs, (got - ref).abs().max().item())
     # Against fp32 (not against the quantized checker) the error is the recipe's own quantization
-    # noise: c3's zero-mean outlier channels are the worst case for per-block INT8 (see
-    # test_oracle_attn), the e4m3 probabilities of c4/c5 come next.
-    bar = 0.998 if wid == 3 else COS
-    abs_bar = {3: 8e-2, 4: 4e-2, 5: 4e-2}[wid]
-    assert worst_cos >= bar and worst_abs <= abs_bar, (worst_cos, worst_abs)
+    # noise, largest for single elements of the e4m3 probabilities of c4/c5 and of c3's outlier
+    # channels.
+    assert worst_cos >= COS and worst_abs <= 4e-2, (worst_cos, worst_abs)
     # constant V
     vc = v[:, :1].expand(-1, w.S, -1, -1).contiguous()
     oc = _one_shot_dev(q, k, vc, w)
@@ -334,7 +499,7 @@ def test_full_size_properties(wid):
     k2 = (k.float() + off).to(torch.bfloat16)
     o2 = _one_shot_dev(q, k2, v, w)
     cos = torch.nn.functional.cosine_similarity(o.float().flatten(), o2.float().flatten(), dim=0).item()
-    assert cos >= (0.998 if wid == 3 else 0.999), cos
+    assert cos >= 0.999, cos
 
 
 @pytest.mark.parametrize("variant", [0, 1])

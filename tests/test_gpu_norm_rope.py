@@ -1,5 +1,5 @@
 """GPU parity of the quantizers with RMSNorm + interleaved RoPE fused in front: the INT8 codes,
-scales and the K mean must be bit-identical with what the CPU checker gets by running its
+scales and the K statistics must be bit-identical with what the CPU checker gets by running its
 norm/rope restatement first and its quantizers on the result; the one-shot call must agree with
 the unfused pipeline."""
 import numpy as np
@@ -36,18 +36,19 @@ def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_row
     k8 = torch.full((B, Hh, nkp, D), 77, dtype=torch.int8, device="cuda")
     qs = torch.full((B, Hh, nqp // blkq), -1.0, dtype=torch.float32, device="cuda")
     ks = torch.full((B, Hh, nkp // blkk), -1.0, dtype=torch.float32, device="cuda")
-    km = torch.full((B, Hh, D), -1.0, dtype=torch.float32, device="cuda")
+    km, qm, kmu = (torch.full((B, Hh, D), -1.0, dtype=torch.float32, device="cuda") for _ in range(3))
     scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, Hh, S, D), 8), dtype=torch.uint8, device="cuda")
     st = _lib.strides_bhnd(S, Hh, D)
     rc = L.mi355_sage_quant_qk_norm_rope_bf16(
         qd.data_ptr(), kd.data_ptr(), B, Hh, S, S, D, scale, st, st, 0, 0,
         gqd.data_ptr(), gkd.data_ptr(), eps, cd.data_ptr() if cd is not None else None,
-        sd.data_ptr() if sd is not None else None, batch_rows, blkq, blkk, int(smooth),
-        q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr() if smooth else None,
+        sd.data_ptr() if sd is not None else None, batch_rows, blkq, blkk, (1 if smooth else 0) | 2,
+        q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
         scr.data_ptr(), scr.numel(), H.stream())
     assert rc == 0, rc
     torch.cuda.synchronize()
-    return q8.cpu().numpy(), qs.cpu().numpy(), k8.cpu().numpy(), ks.cpu().numpy(), km.cpu().numpy()
+    return dict(q8=q8.cpu().numpy(), qscale=qs.cpu().numpy(), k8=k8.cpu().numpy(), kscale=ks.cpu().numpy(),
+                kmean=km.cpu().numpy(), qmul=qm.cpu().numpy(), kmul=kmu.cpu().numpy())
 
 
 @pytest.mark.parametrize("D,S,blkq,blkk,smooth,rope,per_batch", [
@@ -68,15 +69,15 @@ def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_
     got = _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows)
     qn = oracle.norm_rope_bf16(q, gq, eps, cos, sin, batch_rows)
     kn = oracle.norm_rope_bf16(k, gk, eps, cos, sin, batch_rows)
-    q8, qs = oracle.quant_q(qn, scale, blkq, int(_lib.lib().mi355_sage_pad_q(1)))
-    mu = oracle.kmean(kn) if smooth else None
-    k8, ks = oracle.quant_k(kn, mu, blkk, 128)
-    if smooth:
-        np.testing.assert_array_equal(got[4].view(np.uint32), mu.view(np.uint32))
-    np.testing.assert_array_equal(got[1][:, :, :qs.shape[2]].view(np.uint32), qs.view(np.uint32))
-    np.testing.assert_array_equal(got[3][:, :, :ks.shape[2]].view(np.uint32), ks.view(np.uint32))
-    np.testing.assert_array_equal(got[0], q8)
-    np.testing.assert_array_equal(got[2], k8)
+    import gpu_harness as H
+    want = H.oracle_quant_qk(oracle, qn, kn, scale, blkq, blkk, smooth, True)
+    for name in ("kmean", "qmul", "kmul"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    nqb, nkb = want["qscale"].shape[2], want["kscale"].shape[2]
+    np.testing.assert_array_equal(got["qscale"][:, :, :nqb].view(np.uint32), want["qscale"].view(np.uint32))
+    np.testing.assert_array_equal(got["kscale"][:, :, :nkb].view(np.uint32), want["kscale"].view(np.uint32))
+    np.testing.assert_array_equal(got["q8"], want["q8"])
+    np.testing.assert_array_equal(got["k8"], want["k8"])
 
 
 @pytest.mark.parametrize("variant,wid", [(0, 2), (1, 2), (0, 1)])
@@ -104,7 +105,7 @@ def test_one_shot_equals_unfused_pipeline(oracle, variant, wid):
     qnd, knd = H.dev_bf16(qn), H.dev_bf16(kn)
     rc = _lib.lib().mi355_sage_sdpa_bf16_ex(qnd.data_ptr(), knd.data_ptr(), vd.data_ptr(), want.data_ptr(),
                                             w.B, w.H, w.S, w.S, w.D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, H.stream(),
-                                            variant, w.blkq, w.blkk, 1, None, 0)
+                                            variant, w.blkq, w.blkk, 3, None, 0)
     assert rc == 0, rc
     torch.cuda.synchronize()
     np.testing.assert_array_equal(H.to_bits(got), H.to_bits(want))
@@ -139,6 +140,18 @@ def test_argument_errors():
                                           st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 1,
                                           g.data_ptr() + 2, g.data_ptr(), 1e-6, None, None, 0, None, 0)
     assert rc == -2
+    # the table has one row per position, shared by Q and K: N_q != N_kv is refused (-2), norm only is fine
+    t = torch.zeros((64 * 2, 64), dtype=torch.float32, device="cuda")
+    st32 = _lib.strides_bhnd(32, 2, 128)
+    rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 32, 64, 128, 0.1,
+                                          st32, st, st, st32, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
+                                          g.data_ptr(), g.data_ptr(), 1e-6, t.data_ptr(), t.data_ptr(), 0, None, 0)
+    assert rc == -2
+    rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 32, 64, 128, 0.1,
+                                          st32, st, st, st32, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
+                                          g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, None, 0)
+    assert rc == 0
+    torch.cuda.synchronize()
 
 
 def test_fused_train_fwd_stats(oracle):

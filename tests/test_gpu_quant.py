@@ -1,6 +1,6 @@
 """GPU parity of the quantize kernels, through the C ABI, against the CPU
-checker: INT8 codes, fp32 scales, the K mean, fp16 / e4m3 V and V scales must
-be bit-identical."""
+checker: INT8 codes, fp32 scales, the K statistics (mean, channel multipliers),
+fp16 / e4m3 V and V scales must be bit-identical."""
 import ctypes
 
 import numpy as np
@@ -12,14 +12,12 @@ from mojodiffusion_amd.workloads import WORKLOADS, make_inputs, f32_to_bf16_bits
 pytestmark = pytest.mark.gpu
 
 
-def _check_qk(oracle, H, q, k, scale, blkq, blkk, smooth):
-    g = H.quant_qk(q, k, scale, blkq, blkk, smooth)
-    Sq, Skv = q.shape[1], k.shape[1]
-    q8, qs = oracle.quant_q(q, scale, blkq, int(_lib.lib().mi355_sage_pad_q(1)))
-    mu = oracle.kmean(k) if smooth else None
-    k8, ks = oracle.quant_k(k, mu, blkk, 128)
-    if smooth:
-        np.testing.assert_array_equal(g["kmean"].view(np.uint32), mu.view(np.uint32))
+def _check_qk(oracle, H, q, k, scale, blkq, blkk, smooth, balance=True, mask=(0, 0)):
+    g = H.quant_qk(q, k, scale, blkq, blkk, smooth, balance=balance, mask=mask)
+    want = H.oracle_quant_qk(oracle, q, k, scale, blkq, blkk, smooth, balance, mask)
+    q8, qs, k8, ks = want["q8"], want["qscale"], want["k8"], want["kscale"]
+    for name in ("kmean", "qmul", "kmul"):
+        np.testing.assert_array_equal(g[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
     nqb, nkb = qs.shape[2], ks.shape[2]
     np.testing.assert_array_equal(g["qscale"][:, :, :nqb].view(np.uint32), qs.view(np.uint32))
     np.testing.assert_array_equal(g["kscale"][:, :, :nkb].view(np.uint32), ks.view(np.uint32))
@@ -36,6 +34,48 @@ def test_quant_qk_bit_exact_workload_stats(oracle, wid):
     w = w if wid == 1 else w.scaled(B=w.B, H=3, S=1100)      # ragged: 1100 = 8*128 + 76 = 17*64 + 12
     q, k, _ = make_inputs(w)
     _check_qk(oracle, H, q, k, w.scale, w.blkq, w.blkk, True)
+    _check_qk(oracle, H, q, k, w.scale, w.blkq, w.blkk, True, balance=False)
+
+
+@pytest.mark.parametrize("wid", [2, 3, 4, 5])
+def test_quant_bit_exact_at_full_sequence_length(oracle, wid):
+    """Every workload at its real sequence length (c5: S = 32760 = 511*64 + 56, a ragged last
+    block in every tensor) on two heads: statistics, INT8 codes and scales of Q and K, and for
+    the e4m3 workloads the V bytes and scales, bit for bit."""
+    import gpu_harness as H
+    w = WORKLOADS[wid].scaled(B=1, H=2)
+    q, k, v = make_inputs(w)
+    _check_qk(oracle, H, q, k, w.scale, w.blkq, w.blkk, True)
+    g = H.quant_v(v, w.variant)
+    if w.variant == 0:
+        np.testing.assert_array_equal(H.untile_v(g["vq"], 0), oracle.quant_v_f16(v, 128))
+    else:
+        v8, vs = oracle.quant_v_fp8(v, 128)
+        np.testing.assert_array_equal(g["vscale"].view(np.uint32), vs.view(np.uint32))
+        np.testing.assert_array_equal(H.untile_v(g["vq"], 1), v8)
+
+
+@pytest.mark.parametrize("D,S,mask,smooth,balance", [(128, 700, (300, 512), True, True), (128, 333, (0, 64), True, True),
+                                                     (64, 520, (500, 520), True, False), (128, 200, (17, 150), False, True)])
+def test_quant_with_masked_key_range(oracle, D, S, mask, smooth, balance):
+    """Keys [lo, hi) take no part: not in the K statistics, not in their scale blocks (code 0),
+    not in the V scales (bytes 0) — also when the range cuts through blocks and groups."""
+    import gpu_harness as H
+    rng = np.random.default_rng(S + D)
+    q = f32_to_bf16_bits(rng.standard_normal((2, S, 2, D)).astype(np.float32))
+    kx = (rng.standard_normal((2, S, 2, D)) * 2 + rng.standard_normal((2, 1, 2, D)) * 3).astype(np.float32)
+    vx = rng.standard_normal((2, S, 2, D)).astype(np.float32)
+    kx[:, mask[0]:mask[1]] *= 50.0                       # would dominate every statistic if it counted
+    vx[:, mask[0]:mask[1]] *= 50.0
+    k, v = f32_to_bf16_bits(kx), f32_to_bf16_bits(vx)
+    g = _check_qk(oracle, H, q, k, 0.09, 128, 64, smooth, balance, mask)
+    assert not g["k8"][:, :, mask[0]:mask[1]].any()
+    g0 = H.quant_v(v, 0, mask)
+    np.testing.assert_array_equal(H.untile_v(g0["vq"], 0), oracle.quant_v_f16(v, 128, *mask))
+    g1 = H.quant_v(v, 1, mask)
+    v8, vs = oracle.quant_v_fp8(v, 128, *mask)
+    np.testing.assert_array_equal(g1["vscale"].view(np.uint32), vs.view(np.uint32))
+    np.testing.assert_array_equal(H.untile_v(g1["vq"], 1), v8)
 
 
 @pytest.mark.parametrize("D,blkq,blkk,S,smooth", [
@@ -47,6 +87,7 @@ def test_quant_qk_bit_exact_shapes(oracle, D, blkq, blkk, S, smooth):
     q = f32_to_bf16_bits(rng.standard_normal((2, S, 2, D)).astype(np.float32))
     k = f32_to_bf16_bits((rng.standard_normal((2, S, 2, D)) * 3 + rng.standard_normal((2, 1, 2, D)) * 5).astype(np.float32))
     _check_qk(oracle, H, q, k, 0.2, blkq, blkk, smooth)
+    _check_qk(oracle, H, q, k, 0.2, blkq, blkk, smooth, balance=False)
 
 
 def test_quant_qk_ties_zero_blocks_and_extremes(oracle):
@@ -62,7 +103,12 @@ def test_quant_qk_ties_zero_blocks_and_extremes(oracle):
     x[0, 192:256] = np.random.default_rng(6).standard_normal((64, 1, D)) * 1e30       # block 3: huge values
     k = f32_to_bf16_bits(x)
     q = f32_to_bf16_bits(np.random.default_rng(7).standard_normal((1, S, 1, D)).astype(np.float32))
-    g = _check_qk(oracle, H, q, k, 1.0, 64, 64, False)
+    g = _check_qk(oracle, H, q, k, 1.0, 64, 64, False, balance=False)
+    # balanced, with a spread the channel factors can carry without leaving the normal fp32 range
+    # (values below 2^-126 are where a GPU that flushes subnormals and the CPU stop agreeing)
+    x[0, 128:192] *= 1e18
+    x[0, 192:256] *= 1e-18
+    _check_qk(oracle, H, q, f32_to_bf16_bits(x), 1.0, 64, 64, False)
     assert g["kscale"][0, 0, 0] == 1.0 and g["kscale"][0, 0, 1] == 1.0
     np.testing.assert_array_equal(g["k8"][0, 0, 0, :len(ties)],
                                   np.int8([127, 0, 2, 2, 0, -2, -2, 64, 64, -126, 126, 0, 1, -1]))
@@ -85,8 +131,16 @@ def test_quant_qk_bhsd_strides_and_offsets(oracle):
     st = (ctypes.c_int64 * 4)(Hh * S * D, S * D, D, 1)
     got = H.quant_qk(bhsd_buf(q), bhsd_buf(k), 0.1, 128, 64, True, strides_q=st, strides_k=st,
                      q_off=off, k_off=off, shape=(B, Hh, S, S, D))
-    for name in ("q8", "qscale", "k8", "kscale", "kmean"):
+    for name in ("q8", "qscale", "k8", "kscale", "kmean", "qmul", "kmul"):
         np.testing.assert_array_equal(got[name], ref[name])
+    # V presented the same way: BHSD memory at a non-zero offset
+    v = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32) * 2.0)
+    for variant in (0, 1):
+        a = H.quant_v(v, variant)
+        b = H.quant_v(bhsd_buf(v), variant, strides=st, v_off=off, shape=(B, Hh, S, D))
+        np.testing.assert_array_equal(a["vq"], b["vq"])
+        if variant == 1:
+            np.testing.assert_array_equal(a["vscale"], b["vscale"])
 
 
 @pytest.mark.parametrize("D,S", [(128, 1100), (64, 1024), (128, 64), (64, 7)])
@@ -113,7 +167,7 @@ def test_quant_full_size_properties():
     import gpu_harness as H
     w = WORKLOADS[2]
     q, k, _ = make_inputs(w)
-    g = H.quant_qk(q, k, w.scale, w.blkq, w.blkk, True)
+    g = H.quant_qk(q, k, w.scale, w.blkq, w.blkk, True, balance=False)
     q8, k8 = g["q8"].astype(np.int32), g["k8"].astype(np.int32)
     # every block's absmax code is exactly 127 and -128 never appears
     assert np.all(np.abs(q8).reshape(w.B, w.H, -1, w.blkq * w.D).max(-1) == 127)

@@ -45,7 +45,8 @@ def test_attn_matches_float64_restatement(oracle, wid, variant, mask):
         v_f32 = oracle.e4m3_to_f32(vq) * vs[:, :, None, :]
         codec = _e4m3_codec_448
     o16, o32 = oracle.attn(q8, qs, w.blkq, k8, ks, w.blkk, vq, vs, variant, w.S, w.S, *mask)
-    want = R.attn_float64(q8, qs, w.blkq, k8, ks, w.blkk, v_f32, w.S, w.S, codec, variant == 1, *mask)
+    want = R.attn_float64(q8, qs, w.blkq, k8, ks, w.blkk, v_f32, w.S, w.S, codec, variant == 1, *mask,
+                          normalise_by_rounded=(variant == 1))
     # exp2f (libm) and np.exp2 may differ in the last ulp, which can flip one P rounding
     np.testing.assert_allclose(o32, want, atol=2e-4, rtol=1e-4)
     # bf16 epilogue is RNE of the fp32 value
@@ -133,6 +134,21 @@ def test_additive_mask(oracle):
     _, o32c = oracle.sdpa_bf16(q, k, v, w.scale, addmask=rowc)
     _, o32z = oracle.sdpa_bf16(q, k, v, w.scale)
     np.testing.assert_allclose(o32c, o32z, atol=2e-3)
+
+
+def test_e4m3_variant_returns_a_dominant_key_exactly(oracle):
+    """One key far above the rest: the softmax is one-hot and O must be that key's V (to the
+    precision of V's own e4m3 code), although the key's probability 2^(s - ceil(s)) is not an
+    e4m3 number — the normaliser sums the rounded probabilities."""
+    w = WORKLOADS[2].scaled(B=1, H=1, S=128, k_offset_std=0.0)
+    q, k, v = make_inputs(w)
+    kf = bf16_bits_to_f32(k)
+    kf[:, 77] = bf16_bits_to_f32(q)[:, 5] * 6.0          # aligned with query 5: score ~ 6*|q|^2*scale
+    from mojodiffusion_amd.workloads import f32_to_bf16_bits
+    _, o32 = oracle.sdpa_bf16(q, f32_to_bf16_bits(kf), v, w.scale, variant=1, blkq=32, blkk=64)
+    v8, vs = oracle.quant_v_fp8(v, 64)
+    v_deq = oracle.e4m3_to_f32(v8)[0, 0, 77] * vs[0, 0]
+    np.testing.assert_allclose(o32[0, 5, 0], v_deq, rtol=1e-5, atol=1e-6)
 
 
 def test_k_smoothing_rescues_offset_keys(oracle):

@@ -176,14 +176,17 @@ def test_quant_v(oracle):
     # the channel absmax maps to +-448 exactly
     dec = oracle.e4m3_to_f32(v8)
     assert np.all(np.abs(dec[:, :, :150]).max(axis=2)[vs != 1.0] == 448.0)
-    # channel maximum over the kept keys only; a masked row beyond it saturates
+    # channel maximum over the kept keys only; masked rows stay 0
     v[:, 20:40] = f32_to_bf16_bits(np.full((2, 20, 3, 32), 50.0, np.float32))
     v8m, vsm = oracle.quant_v_fp8(v, 64, 20, 40)
     v8mn, vsmn = R.quant_v_fp8(v, 64, 20, 40)
     np.testing.assert_array_equal(vsm, vsmn)
     np.testing.assert_array_equal(v8m, v8mn)
     np.testing.assert_array_equal(vsm, oracle.quant_v_fp8(np.delete(v, np.s_[20:40], axis=1), 64)[1])
-    assert np.all(oracle.e4m3_to_f32(v8m[:, :, 20:40])[(vsm != 1.0)[:, :, None, :].repeat(20, 2)] == 448.0)
+    assert not v8m[:, :, 20:40].any()
+    v16m = oracle.quant_v_f16(v, 64, 20, 40)
+    np.testing.assert_array_equal(v16m, R.quant_v_f16(v, 64, 20, 40))
+    assert not v16m[:, :, 20:40].any() and v16m[:, :, :20].any()
 
 
 def test_bad_args(oracle):
