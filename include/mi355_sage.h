@@ -78,6 +78,26 @@ int mi355_sage_sdpa_bf16(
     void* stream,
     int variant, void* workspace, size_t workspace_bytes);
 
+/* mi355_sage_sdpa_bf16 for callers that cannot allocate device memory and hold no workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments and result as mi355_sage_sdpa_bf16; the
+ * intermediate tensors live in a buffer of mi355_sage_static_scratch_bytes() bytes (16 MiB) that is
+ * part of the loaded library on every GPU, so the call allocates nothing.  A problem whose
+ * workspace (mi355_sage_workspace_bytes) exceeds that returns -3.  All calls on one GPU share the
+ * buffer: calls that overlap in time on one GPU (different streams, or threads) race. */
+int mi355_sage_sdpa_bf16_static(
+    const void* Q, const void* K, const void* V, void* O,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t o_offset_elems,
+    int causal,
+    void* stream,
+    int variant);
+size_t mi355_sage_static_scratch_bytes(void);
+
 /* Same with the quantization recipe spelled out: blkq / blkk = tokens per Q / K
  * scale block (32, 64 or 128 each), k_flags = MI355_SAGE_K_SMOOTH | MI355_SAGE_K_BALANCE
  * or a subset. */

@@ -15,6 +15,9 @@ _i64 = ctypes.c_int64
 SIGNATURES = {
     "mi355_sage_sdpa_bf16": (_int, [_vp] * 4 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [_i64] * 4
                              + [_int, _vp, _int, _vp, ctypes.c_size_t]),
+    "mi355_sage_sdpa_bf16_static": (_int, [_vp] * 4 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [_i64] * 4
+                                    + [_int, _vp, _int]),
+    "mi355_sage_static_scratch_bytes": (ctypes.c_size_t, []),
     "mi355_sage_sdpa_bf16_ex": (_int, [_vp] * 4 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [_i64] * 4
                                 + [_int, _vp, _int, _int, _int, _int, _vp, ctypes.c_size_t]),
     "mi355_sage_sdpa_bf16_train_fwd": (_int, [_vp] * 5 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [_i64] * 5
@@ -57,6 +60,10 @@ def lib():
             raise RuntimeError(
                 "libmi355_sage.so is not built (%s). Build it with `make -C mojodiffusion_amd/csrc` "
                 "or `python -c 'import __graft_entry__ as g; g.build()'`; there is no fallback path." % LIB_PATH)
+        # torch ships its own copy of the HIP runtime.  It has to be in the process before this
+        # library is loaded, so that the library binds to that same copy: two HIP runtimes in one
+        # process cannot both initialise the device (the second reports "no ROCm-capable device").
+        import torch  # noqa: F401
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)          # AttributeError if a declared symbol is not exported

@@ -9,6 +9,13 @@
 
 using namespace sage;
 
+// Scratch of mi355_sage_sdpa_bf16_static: device memory that belongs to the loaded library, so
+// that entry point never allocates.  Each GPU the library runs on holds its own copy of the
+// array, at its own address, until the process ends.  In host code the array's NAME is only a
+// handle for hipGetSymbolAddress; the address that call returns is what kernels are given.
+constexpr size_t kStaticScratchBytes = 16u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 constexpr size_t kAlign = 256;
@@ -164,6 +171,25 @@ int make_pre(const void* q_gain, const void* k_gain, float eps, const void* rope
                    static_cast<const float*>(rope_sin), rope_batch_rows};
     out->k = out->q;
     out->k.gain = static_cast<const uint16_t*>(k_gain);
+    return 0;
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+std::mutex g_static_mutex;
+void* g_static_ptr[64] = {};
+
+int static_scratch(void** out) {
+    int dev = 0;
+    SAGE_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return MI355_SAGE_EUNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (g_static_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        SAGE_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & (kAlign - 1))) return MI355_SAGE_EUNSUPPORTED;
+        g_static_ptr[dev] = p;
+    }
+    *out = g_static_ptr[dev];
     return 0;
 }
 
@@ -348,6 +374,32 @@ int mi355_sage_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
                      o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, default_blkq(variant), 64,
                      kDefaultFlags, workspace, workspace_bytes);
 }
+
+int mi355_sage_sdpa_bf16_static(const void* Q, const void* K, const void* V, void* O,
+                                int B, int H, int N_q, int N_kv, int D, float scale,
+                                const int64_t* q_strides, const int64_t* k_strides,
+                                const int64_t* v_strides, const int64_t* o_strides,
+                                int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off,
+                                int causal, void* stream, int variant) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
+    if (!dims_ok(D) || (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8)) return MI355_SAGE_EUNSUPPORTED;
+    const size_t need = carve(B, H, N_q, N_kv, D, variant).total;
+    if (need > kStaticScratchBytes) {
+        SAGE_LOG("mi355_sage_sdpa_bf16_static: this problem needs %zu bytes of scratch, the built-in buffer holds %zu; "
+                 "use mi355_sage_sdpa_bf16 with a workspace", need, kStaticScratchBytes);
+        return MI355_SAGE_EWORKSPACE;
+    }
+    // Nothing in the buffer has to start at zero: every byte a kernel of the path reads was
+    // written by an earlier kernel of the same call (pad rows and pad blocks included).
+    void* p = nullptr;
+    int rc;
+    if ((rc = static_scratch(&p))) return rc;
+    return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                     o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, default_blkq(variant), 64,
+                     kDefaultFlags, p, kStaticScratchBytes);
+}
+
+size_t mi355_sage_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int mi355_sage_sdpa_bf16_ex(const void* Q, const void* K, const void* V, void* O,
                             int B, int H, int N_q, int N_kv, int D, float scale,
