@@ -176,6 +176,24 @@ int mi355_sage_sdpa_bf16_keymask(
     void* stream,
     int variant, void* workspace, size_t workspace_bytes);
 
+/* Attention with an additive score bias: the native path behind sdpa / sdpa_chunked
+ * (serenitymojo/ops/attention.mojo:1596-1647, :1650-1687; mask [B,H,S,S]) and sdpa_cross_masked
+ * (:1897-1936; mask [B,H,Sq,Skv]).  Mask: bf16 (the dtype of q, as the reference requires),
+ * logical [B,H,N_q,N_kv] through four element strides — the key stride must be 1, rows 8-byte
+ * aligned; a stride of 0 broadcasts over batch or head.  The bias is in the units of the scaled
+ * scores (softmax(scale * q.k + mask)); -inf (or the reference's -1e4) removes a key for a row.
+ * Default recipe of mi355_sage_sdpa_bf16; the K statistics do not look at the mask. */
+int mi355_sage_sdpa_bf16_mask(
+    const void* Q, const void* K, const void* V, const void* Mask, void* O,
+    int B, int H, int N_q, int N_kv, int D,
+    float scale,
+    const int64_t* q_strides, const int64_t* k_strides,
+    const int64_t* v_strides, const int64_t* mask_strides, const int64_t* o_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems,
+    int64_t v_offset_elems, int64_t mask_offset_elems, int64_t o_offset_elems,
+    void* stream,
+    int variant, void* workspace, size_t workspace_bytes);
+
 /* mi355_sage_sdpa_bf16_train_fwd on the pre-norm projections (default recipe: Q blocks of 128
  * tokens, 32 for the e4m3 variant; K blocks of 64; K smoothing and balancing on), for the blocks that run
  * rms_norm / rope_interleaved in front of sdpa_flash_train_fwd

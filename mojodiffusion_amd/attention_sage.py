@@ -4,8 +4,10 @@ bound to libmi355_sage.so.
 Function names, argument meaning and error behaviour follow
 serenitymojo/ops/attention_flash.mojo (sdpa_flash_train_fwd :149-202, _rect
 :205-264, sdpa_flash_fwd_padmask :267-342, sdpa_flash_train_fwd_f32 :457-475) and
-serenitymojo/ops/attention.mojo (sdpa_nomask :1690-1718, sdpa_nomask_tiled
-:1762-1787, sdpa_qwen_keymask :1790-1857, sdpa_cross_nomask :1860-1894).  Tensors are [B, S, H, Dh]; torch is
+serenitymojo/ops/attention.mojo (sdpa :1596-1647, sdpa_chunked :1650-1687,
+sdpa_nomask :1690-1718, sdpa_nomask_tiled :1762-1787, sdpa_qwen_keymask :1790-1857,
+sdpa_cross_nomask :1860-1894, sdpa_cross_masked :1897-1936, sdpa_nomask_slab
+:2144-2169).  Tensors are [B, S, H, Dh]; torch is
 used only to own device memory and the stream.  What differs from the cuDNN path:
 no 128-padding copies are needed (ragged S is handled in the kernels), so the
 `*_pad` members of the result alias the caller's tensors.
@@ -213,6 +215,119 @@ def sdpa_cross_nomask(q, k, v, scale, variant=PV_FP16):
     o = _call_train_fwd("sdpa_cross_nomask", q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16),
                         scale, q.shape[1], k.shape[1], variant, False)[0]
     return o.to(q.dtype)
+
+
+def _masked(name, q, k, v, mask, scale, variant, square):
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise Error("%s: q/k/v dtype mismatch" % name)
+    if q.dtype != mask.dtype:
+        raise Error("%s: q/mask dtype mismatch" % name)
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise Error("%s: q must be rank-4 [B,S,H,Dh]" % name if square else "%s: q/k/v must be rank-4 [B,S,H,Dh]" % name)
+    _check_shapes(name, q, k, v, square)
+    B, Sq, H, Dh = q.shape
+    Skv = k.shape[1]
+    if tuple(mask.shape) != (B, H, Sq, Skv):
+        raise Error("%s: mask must be [B,H,S,S]" % name if square else "%s: mask must be [B,H,Sq,Skv]" % name)
+    _require_cuda(name, q, k, v)
+    if not mask.is_cuda:
+        raise Error("%s: tensors must live on the GPU (no CPU fallback exists)" % name)
+    out_dtype = q.dtype
+    if q.dtype != torch.bfloat16:
+        q, k, v, mask = (t.to(torch.bfloat16) for t in (q, k, v, mask))
+    if mask.stride(3) != 1 or any(st % 4 for st in mask.stride()[:3]):
+        mask = mask.contiguous()
+        if Skv % 4:                                   # rows of the bias must start 8-byte aligned
+            padded = torch.zeros((B, H, Sq, (Skv + 3) // 4 * 4), dtype=mask.dtype, device=mask.device)
+            padded[..., :Skv] = mask
+            mask = padded
+    L = _lib.lib()
+    o = torch.empty_like(q)
+    ws = _workspace(max(L.mi355_sage_workspace_bytes(B, H, Sq, Skv, Dh, variant), 256), q.device)
+    qs, ks = _lib.strides_bhnd(Sq, H, Dh), _lib.strides_bhnd(Skv, H, Dh)
+    ms = (_lib.ctypes.c_int64 * 4)(*mask.stride())
+    rc = L.mi355_sage_sdpa_bf16_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), o.data_ptr(),
+                                     B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, ms, qs, 0, 0, 0, 0, 0,
+                                     torch.cuda.current_stream(q.device).cuda_stream, variant, ws.data_ptr(), ws.numel())
+    if rc != 0:
+        raise Error("%s: shim rc=%d (B=%d Sq=%d Skv=%d H=%d Dh=%d)" % (name, rc, B, Sq, Skv, H, Dh))
+    return o.to(out_dtype)
+
+
+def sdpa(q, k, v, mask, scale, variant=PV_FP16):
+    """attention.mojo:1596-1647: full attention with an additive score bias.  q, k, v:
+    [B,S,H,Dh]; mask: [B,H,S,S] of q's dtype (zeros = full attention); returns [B,S,H,Dh] in
+    q's dtype."""
+    return _masked("sdpa", q, k, v, mask, scale, variant, True)
+
+
+def sdpa_chunked(q, k, v, mask, scale, variant=PV_FP16):
+    """attention.mojo:1650-1687: the reference's head-chunked variant of `sdpa` (same result,
+    smaller score slab).  This kernel never holds a score slab, so it is the same call."""
+    return _masked("sdpa_chunked", q, k, v, mask, scale, variant, True)
+
+
+def sdpa_cross_masked(q, k, v, mask, scale, variant=PV_FP16):
+    """attention.mojo:1897-1936: rectangular attention with an additive bias [B,H,Sq,Skv]."""
+    return _masked("sdpa_cross_masked", q, k, v, mask, scale, variant, False)
+
+
+class StepSlab:
+    """Counterpart of serenitymojo/autograd_v2/step_slab.mojo:39-90: a bump allocator over one
+    device buffer owned by the caller's step.  alloc() hands out 256-byte-aligned views and never
+    touches the device allocator; reset() rewinds (host bookkeeping only)."""
+
+    def __init__(self, slab_bytes, device="cuda", alignment=256):
+        self.buf = torch.empty(int(slab_bytes), dtype=torch.uint8, device=device)
+        self.alignment = alignment
+        self.used = 0
+        self.peak = 0
+        self.n_allocs = 0
+
+    def alloc(self, nbytes):
+        base = self.buf.data_ptr()
+        start = (base + self.used + self.alignment - 1) // self.alignment * self.alignment - base
+        if start + nbytes > self.buf.numel():
+            raise Error("StepSlab: out of space (%d + %d > %d)" % (start, nbytes, self.buf.numel()))
+        self.used = start + nbytes
+        self.peak = max(self.peak, self.used)
+        self.n_allocs += 1
+        return self.buf[start:start + nbytes]
+
+    def reset(self):
+        self.used = 0
+
+    def peak_bytes(self):
+        return self.peak
+
+    def capacity_bytes(self):
+        return self.buf.numel()
+
+    def used_bytes(self):
+        return self.used
+
+
+def sdpa_nomask_slab(q, k, v, scale, slab, variant=PV_FP16):
+    """attention.mojo:2144-2169: `sdpa_nomask` with every allocation (the output and the
+    intermediates) taken from the caller's StepSlab instead of the device allocator — the form a
+    captured step uses.  BF16 only (the reference's slab path converts nothing either)."""
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise Error("sdpa_nomask: q/k/v dtype mismatch")
+    _check_shapes("sdpa_nomask", q, k, v, True)
+    _require_bf16("sdpa_nomask_slab", q, k, v)
+    _require_cuda("sdpa_nomask", q, k, v)
+    B, S, H, Dh = q.shape
+    L = _lib.lib()
+    o = slab.alloc(q.numel() * 2).view(torch.bfloat16).view(q.shape)
+    nws = max(L.mi355_sage_workspace_bytes(B, H, S, S, Dh, variant), 256)
+    ws = slab.alloc(nws)
+    st = _lib.strides_bhnd(S, H, Dh)
+    rc = L.mi355_sage_sdpa_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, S, S, Dh, float(scale),
+                                st, st, st, st, 0, 0, 0, 0, 0, torch.cuda.current_stream(q.device).cuda_stream,
+                                variant, ws.data_ptr(), nws)
+    if rc != 0:
+        raise Error("sdpa_nomask: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (rc, B, S, H, Dh))
+    return o
 
 
 def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin):

@@ -250,7 +250,10 @@ int quantize(const View& q, const View& k, const View* v, int B, int H, int Nq, 
 }
 
 struct MaskArgs {
-    int lo = 0, hi = 0;        // keys lo <= s < hi are masked
+    int lo = 0, hi = 0;                // keys lo <= s < hi are masked
+    const void* add = nullptr;         // additive bias, bf16, logical [B,H,N_q,N_kv]
+    const int64_t* add_strides = nullptr;
+    int64_t add_off = 0;
 };
 
 int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
@@ -277,6 +280,15 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if (pre.q.gain != nullptr && pre.q.cos != nullptr && N_q != N_kv) {
         SAGE_LOG("fused RoPE uses one table row per position of Q and K alike: N_q must equal N_kv");
         return MI355_SAGE_EUNSUPPORTED;
+    }
+    if (mask.add != nullptr) {
+        const int64_t* ms = mask.add_strides;
+        if (!ms) return MI355_SAGE_EINVAL;
+        const uintptr_t a = reinterpret_cast<uintptr_t>(mask.add) + (uintptr_t)(mask.add_off * 2);
+        if (ms[3] != 1 || (a & 7) || (ms[0] & 3) || (ms[1] & 3) || (ms[2] & 3)) {
+            SAGE_LOG("mask: key stride must be 1 and every row 8-byte aligned");
+            return MI355_SAGE_EUNSUPPORTED;
+        }
     }
     // Keys past the real length are excluded from the statistics and the scores alike:
     // the quantizers see only the first kv tokens.
@@ -331,6 +343,10 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(kv, kPadKV);
     a.o = static_cast<uint16_t*>(O) + o_off; a.osb = os[0]; a.osh = os[1]; a.osn = os[2];
     a.stats = Stats ? static_cast<float*>(Stats) + stats_off : nullptr;
+    if (mask.add != nullptr) {
+        a.amask = static_cast<const uint16_t*>(mask.add) + mask.add_off;
+        a.amb = mask.add_strides[0]; a.amh = mask.add_strides[1]; a.amn = mask.add_strides[2];
+    }
     SAGE_HIP(launch_attn(a, st));
     return MI355_SAGE_OK;
 }
@@ -440,6 +456,20 @@ int mi355_sage_sdpa_bf16_keymask(const void* Q, const void* K, const void* V, vo
     m.lo = mask_lo; m.hi = mask_hi;
     return sdpa_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, stats_off, 0, 0, stream, variant,
+                     default_blkq(variant), 64, kDefaultFlags, workspace, workspace_bytes, Pre{}, m);
+}
+
+int mi355_sage_sdpa_bf16_mask(const void* Q, const void* K, const void* V, const void* Mask, void* O,
+                              int B, int H, int N_q, int N_kv, int D, float scale,
+                              const int64_t* q_strides, const int64_t* k_strides,
+                              const int64_t* v_strides, const int64_t* mask_strides, const int64_t* o_strides,
+                              int64_t q_off, int64_t k_off, int64_t v_off, int64_t mask_off, int64_t o_off,
+                              void* stream, int variant, void* workspace, size_t workspace_bytes) {
+    if (!Mask || !mask_strides) return MI355_SAGE_EINVAL;
+    MaskArgs m;
+    m.add = Mask; m.add_strides = mask_strides; m.add_off = mask_off;
+    return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                     o_strides, q_off, k_off, v_off, o_off, 0, 0, 0, stream, variant,
                      default_blkq(variant), 64, kDefaultFlags, workspace, workspace_bytes, Pre{}, m);
 }
 

@@ -115,7 +115,12 @@ template <int VARIANT> struct Lazy {
     static constexpr bool integer_ref = VARIANT == 1;
 };
 
-template <int D, int VARIANT, bool STATS>
+// ADDMASK: an additive score bias (natural-log units, bf16, logical [B,H,Nq,Nkv] through element
+// strides with the key stride 1) is added to the dequantised scores.  That instantiation looks
+// for every tile's maximum on the biased scores (no optimistic tiles) and lets its ordinary
+// global loads share the vector-memory counter with the tile copies, i.e. it waits for all of
+// them at the midpoint: it is bound by the N_q x N_kv bias it has to read, not by the copies.
+template <int D, int VARIANT, bool STATS, bool ADDMASK>
 __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
@@ -123,7 +128,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const float* __restrict__ qshift,
     int H, int Nq, int kv_valid, int mask_lo, int mask_hi, int64_t nq_pad, int64_t nkv_pad,
     uint16_t* __restrict__ o, int64_t osb, int64_t osh, int64_t osn,
-    float* __restrict__ stats, int n_qtiles, int total_wg) {
+    float* __restrict__ stats, int n_qtiles, int total_wg,
+    const uint16_t* __restrict__ amask, int64_t amb, int64_t amh, int64_t amn) {
     constexpr int VB = (VARIANT == 0) ? 2 : 1;          // bytes per V element
     constexpr int KSTEPS = D / 32;                      // int8 MFMA steps over the head dim
     constexpr int DB = D / 32;                          // 32-channel output blocks
@@ -177,6 +183,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         for (int s = 0; s < KSTEPS; s++) qf[s] = *reinterpret_cast<const v4i*>(qp + s * 32);
     }
     const float sq = qscale[bh * (nq_pad / blkq) + qrow / blkq] * kMagicUnit;
+    // this lane's row of the additive bias (padding rows read the last real row; their output is dropped)
+    const uint16_t* mrow = ADDMASK ? amask + b * amb + h * amh + (int64_t)min(qrow, Nq - 1) * amn : nullptr;
 
     // K scales of this head are staged in LDS once: a global load inside the main loop
     // would make the compiler wait for ALL outstanding vector-memory operations, i.e. for the
@@ -309,7 +317,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     auto iteration = [&](int t, auto x_tag, auto first_tag) {
         constexpr int X = decltype(x_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
-        constexpr bool OPT = VARIANT == 0 && !FIRST;
+        constexpr bool OPT = VARIANT == 0 && !FIRST && !ADDMASK;
         const int slot_vprev = (t + NSV - 1) % NSV, slot_knext = (t + 1) % NSK;
 
         // ---- S^T = K(t) . Q^T : two 32-key blocks
@@ -338,11 +346,45 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
                     if (key >= kv_valid || (key >= mask_lo && key < mask_hi)) s[kb][i] = (int)0xFF800000;
                 }
         }
+        // biased scores in the log2 domain, without the reference maximum (ADDMASK only)
+        float xs[2][ADDMASK ? 16 : 1];
+        if constexpr (ADDMASK) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const float base = -(kMagicF * f[kb]);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int key = key0 + kb * 32 + g * 8 + half * 4;
+                    uint32_t w0 = 0u, w1 = 0u;
+                    if (key + 4 <= kv_valid) {
+                        const u32x2 w = *reinterpret_cast<const u32x2*>(mrow + key);
+                        w0 = w.x; w1 = w.y;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (key + e < kv_valid) (e < 2 ? w0 : w1) |= (uint32_t)mrow[key + e] << ((e & 1) * 16);
+                    }
+                    const float mv[4] = {__uint_as_float(w0 << 16), __uint_as_float(w0 & 0xFFFF0000u),
+                                         __uint_as_float(w1 << 16), __uint_as_float(w1 & 0xFFFF0000u)};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float sdq = fmaf(__int_as_float(s[kb][g * 4 + e]), f[kb], base);
+                        xs[kb][g * 4 + e] = fmaf(mv[e], 1.4426950408889634f, sdq);
+                    }
+                }
+            }
+        }
         float corr = 1.0f;
         bool refresh = false;
         // tile maximum on the raw accumulators (monotone in the score since f > 0), refresh decision
         auto decide = [&](float tau) {
             float mt = -INFINITY;
+            if constexpr (ADDMASK) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) mt = fmaxf(mt, xs[kb][i]);
+            } else
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
                 int ma = max(max(s[kb][0], s[kb][1]), s[kb][2]);
@@ -373,8 +415,15 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         // Exponentials of scores n, n+1 of this lane (n counts through kb, then i).
         auto exp_pair = [&](int n) {
             const int kb = n >> 4, i = n & 15;
-            float p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
-            float p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
+            float p0, p1;
+            if constexpr (ADDMASK) {
+                const float mref = m_used - Lazy<VARIANT>::log2_pscale;
+                p0 = __builtin_amdgcn_exp2f(xs[kb][i] - mref);
+                p1 = __builtin_amdgcn_exp2f(xs[kb][i + 1] - mref);
+            } else {
+                p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
+                p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
+            }
             if constexpr (VARIANT == 0) {
                 const v2h pr = {(_Float16)p0, (_Float16)p1};
                 const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
@@ -401,7 +450,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         // it read are free: publish K(t+1)/V(t), start the copies of K(t+2) and V(t+1), and
         // fetch the fragments of K(t+1).
         auto midpoint = [&]() {
-            dma_wait<(LEAD - 1) * (K_CH + V_CH)>();
+            dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
             __syncthreads();
             dma_k(min(t + LEAD + 1, last), (t + LEAD + 1) % NSK);
             dma_v(min(t + LEAD, last), (t + LEAD) % NSV);
@@ -514,14 +563,19 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
     dim3 grid((unsigned)total), block(512);
-    if (a.stats != nullptr)
-        hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, true>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
-                           a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
-                           a.kv_valid, a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
-    else
-        hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, false>), grid, block, 0, st, a.q8, a.qscale, a.blkq,
-                           a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq,
-                           a.kv_valid, a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles, (int)total);
+#define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                                                                          \
+    hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
+                       a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,   \
+                       a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,        \
+                       (int)total, a.amask, a.amb, a.amh, a.amn)
+    if (a.amask != nullptr) {
+        if (a.stats != nullptr) SAGE_LAUNCH_ATTN(true, true);
+        else SAGE_LAUNCH_ATTN(false, true);
+    } else {
+        if (a.stats != nullptr) SAGE_LAUNCH_ATTN(true, false);
+        else SAGE_LAUNCH_ATTN(false, false);
+    }
+#undef SAGE_LAUNCH_ATTN
     return hipGetLastError();
 }
 

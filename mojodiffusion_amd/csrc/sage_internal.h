@@ -100,6 +100,8 @@ struct AttnArgs {
     int64_t nq_pad, nkv_pad;
     uint16_t* o; int64_t osb, osh, osn;
     float* stats;            // [B,H,Nq] or null
+    const uint16_t* amask;   // additive bias, bf16, base + offset; null = none
+    int64_t amb, amh, amn;   // its element strides for batch, head, query (key stride 1)
 };
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st);
 

@@ -96,6 +96,14 @@ def test_host_mirror_error_strings():
         A.sdpa_nomask(qb, qb, qb, 0.1)
     with pytest.raises(A.Error, match="sdpa_nomask_tiled: q/k/v dtype mismatch"):
         A.sdpa_nomask_tiled(q, qb, q, 0.1)
+    with pytest.raises(A.Error, match="sdpa: q/mask dtype mismatch"):
+        A.sdpa(qb, qb, qb, torch.zeros((1, 2, 128, 128)), 0.1)
+    with pytest.raises(A.Error, match=r"sdpa: mask must be \[B,H,S,S\]"):
+        A.sdpa(qb, qb, qb, torch.zeros((1, 2, 128, 64), dtype=torch.bfloat16), 0.1)
+    with pytest.raises(A.Error, match=r"sdpa_cross_masked: mask must be \[B,H,Sq,Skv\]"):
+        A.sdpa_cross_masked(qb[:, :64], qb, qb, torch.zeros((1, 2, 128, 128), dtype=torch.bfloat16), 0.1)
+    with pytest.raises(A.Error, match="sdpa_chunked: q/k/v dtype mismatch"):
+        A.sdpa_chunked(q, qb, q, torch.zeros((1, 2, 128, 128)), 0.1)
     with pytest.raises(A.Error, match="sdpa_qwen_keymask: real_txt_len out of range"):
         A.sdpa_qwen_keymask(qb, qb, qb, 64, 65, 0.1)
     with pytest.raises(A.Error, match="sdpa_qwen_keymask: N_TXT must be <= S"):

@@ -328,6 +328,110 @@ def test_one_shot_bhsd_memory_and_offsets_for_every_tensor(oracle, variant):
                                             offs["o"], 16, 0, S, S, H.stream(), variant, None, 0) == -2
 
 
+@pytest.mark.parametrize("variant,Sq,Skv", [(0, 320, 320), (1, 320, 320), (0, 130, 333), (0, 256, 70)])
+def test_additive_mask_entry_points(oracle, variant, Sq, Skv):
+    """sdpa / sdpa_chunked / sdpa_cross_masked: an additive bias on the scaled scores.  Against
+    the CPU checker with the same bias (2e-2) and the biased fp32 referee (cosine 0.999); a -1e4
+    block behaves like the key-range mask; a zero bias reproduces the unmasked call;
+    a bias broadcast over heads through a zero stride gives the same as its materialised copy."""
+    import ctypes
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    w = WORKLOADS[2].scaled(B=2, H=2, S=max(Sq, Skv))
+    q, k, v = make_inputs(w)
+    q, k, v = np.ascontiguousarray(q[:, :Sq]), np.ascontiguousarray(k[:, :Skv]), np.ascontiguousarray(v[:, :Skv])
+    rng = np.random.default_rng(Sq + Skv)
+    bias = f32_to_bf16_bits(rng.standard_normal((w.B, w.H, Sq, Skv)).astype(np.float32) * 1.5)
+    bias_f = bf16_bits_to_f32(bias)
+    bias_f[:, :, :, 5:9] = -np.inf                                   # a few keys removed outright
+    bias_f[0, 1, 7, :] = -1e4                                        # one row biased uniformly (cancels)
+    bias = f32_to_bf16_bits(np.nan_to_num(bias_f, neginf=-3e38))
+    bias_f = bf16_bits_to_f32(bias)
+    qd, kd, vd, md = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v), H.dev_bf16(bias)
+    fn = A.sdpa if Sq == Skv else A.sdpa_cross_masked
+    got = fn(qd, kd, vd, md, w.scale, variant)
+    torch.cuda.synchronize()
+    gotf = got.float().cpu().numpy()
+    blkq = 128 if variant == 0 else 32
+    _, want32 = oracle.sdpa_bf16(q, k, v, w.scale, variant=variant, blkq=blkq, blkk=64, addmask=bias_f)
+    cos, mx = H.cos_maxabs(gotf, want32)
+    assert mx <= MAX_ABS and cos >= 0.9999, (cos, mx)
+    ref = oracle.sdpa_f32(bf16_bits_to_f32(q), bf16_bits_to_f32(k), bf16_bits_to_f32(v), w.scale, addmask=bias_f)
+    cos, mx = H.cos_maxabs(gotf, ref)
+    assert cos >= COS, (cos, mx)
+    if Sq == Skv:
+        np.testing.assert_array_equal(H.to_bits(A.sdpa_chunked(qd, kd, vd, md, w.scale, variant)), H.to_bits(got))
+        zero = torch.zeros_like(md)
+        # (the biased instantiation takes every tile's maximum on the biased scores, the plain one
+        # is lazy about it: same function, last-bit differences)
+        cz, mz = H.cos_maxabs(A.sdpa(qd, kd, vd, zero, w.scale, variant).float().cpu().numpy(),
+                              A.sdpa_nomask(qd, kd, vd, w.scale, variant).float().cpu().numpy())
+        assert cz >= 0.99999 and mz <= (4e-3 if variant == 0 else MAX_ABS), (cz, mz)
+        # F32 storage: cast at the boundary, result in F32
+        o32 = A.sdpa(qd.float(), kd.float(), vd.float(), md.float(), w.scale, variant)
+        assert o32.dtype == torch.float32
+        np.testing.assert_array_equal(o32.cpu().numpy(), gotf)
+    # broadcast over heads through a zero stride, straight through the C ABI
+    L = _lib.lib()
+    one_head = md[:, :1].contiguous()
+    if Skv % 4 == 0:
+        ms = (ctypes.c_int64 * 4)(Sq * Skv, 0, Skv, 1)
+        o1 = torch.empty_like(qd)
+        qs, ks = _lib.strides_bhnd(Sq, w.H, w.D), _lib.strides_bhnd(Skv, w.H, w.D)
+        rc = L.mi355_sage_sdpa_bf16_mask(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), one_head.data_ptr(), o1.data_ptr(),
+                                         w.B, w.H, Sq, Skv, w.D, w.scale, qs, ks, ks, ms, qs, 0, 0, 0, 0, 0, H.stream(),
+                                         variant, None, 0)
+        assert rc == 0, rc
+        o2 = fn(qd, kd, vd, one_head.expand(-1, w.H, -1, -1).contiguous(), w.scale, variant)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(H.to_bits(o1), H.to_bits(o2))
+        bad = (ctypes.c_int64 * 4)(Sq * Skv, 0, Skv + 2, 1)
+        assert L.mi355_sage_sdpa_bf16_mask(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), one_head.data_ptr(), o1.data_ptr(),
+                                           w.B, w.H, Sq, Skv, w.D, w.scale, qs, ks, ks, bad, qs, 0, 0, 0, 0, 0, H.stream(),
+                                           variant, None, 0) == -2
+
+
+def test_minus_1e4_block_equals_the_key_range_mask(oracle):
+    """What sdpa_qwen_keymask does with its -1e4 bias (attention.mojo:804-870), done through the
+    additive-mask call: same output as the key-range call to within the quantization of the
+    statistics (the range call also keeps the masked keys out of the K statistics)."""
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    w = WORKLOADS[2].scaled(B=1, H=2, S=384)
+    q, k, v = (H.dev_bf16(x) for x in make_inputs(w))
+    mask = torch.zeros((1, 2, w.S, w.S), dtype=torch.bfloat16, device="cuda")
+    mask[..., 100:256] = -1e4
+    a = A.sdpa(q, k, v, mask, w.scale)
+    b = A.sdpa_qwen_keymask(q, k, v, 256, 100, w.scale)
+    torch.cuda.synchronize()
+    cos, mx = H.cos_maxabs(a.float().cpu().numpy(), b.float().cpu().numpy())
+    assert cos >= 0.9995 and mx <= 3e-2, (cos, mx)
+
+
+def test_sdpa_nomask_slab_allocates_from_the_slab():
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    w = WORKLOADS[2].scaled(B=1, H=2, S=300)
+    q, k, v = (H.dev_bf16(x) for x in make_inputs(w))
+    want = A.sdpa_nomask(q, k, v, w.scale)
+    slab = A.StepSlab(8 << 20)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    for _ in range(2):
+        slab.reset()
+        got = A.sdpa_nomask_slab(q, k, v, w.scale, slab)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert got.data_ptr() >= slab.buf.data_ptr() and got.data_ptr() < slab.buf.data_ptr() + slab.capacity_bytes()
+    assert slab.n_allocs == 4 and slab.used_bytes() <= slab.peak_bytes() <= slab.capacity_bytes()
+    np.testing.assert_array_equal(H.to_bits(got), H.to_bits(want))
+    with pytest.raises(A.Error, match="StepSlab: out of space"):
+        A.sdpa_nomask_slab(q, k, v, w.scale, A.StepSlab(1 << 16))
+
+
 def test_internal_workspace_is_per_stream():
     """workspace == NULL on two streams: the calls get separate buffers, so the interleaved
     results equal the single-stream ones bit for bit; growth inside a capture is refused."""
