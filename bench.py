@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2] [--skip-cpu-baseline]
 
-A step is one pass of the whole path (K mean, INT8 Q/K quantization, V repack,
+A step is one pass of the whole path (K statistics, INT8 Q/K quantization, V repack,
 attention, bf16 output) over one synthetic batch that is already resident in
 HBM.  The workload is the Flux/Klein joint text+image attention shape
 B=1, H=24, S=4608, D=128 (INT8 QK^T, FP16 PV).  One JSON line is printed:
@@ -14,7 +14,15 @@ B=1, H=24, S=4608, D=128 (INT8 QK^T, FP16 PV).  One JSON line is printed:
   cpu_baseline   the CPU checker's implementation of the same path, timed on
                  this machine's host cores (a reported baseline, not a target)
 
+  roofline.traffic  HBM bytes per launch of that kernel as measured with rocprofv3 --pmc
+                 (FETCH_SIZE, WRITE_SIZE), read from the summary under profiles/ that
+                 `--summarize-traffic` wrote; null when the kernel's source has changed since
+
 This path runs on a single GPU; --gpus above 1 is refused.
+
+    python bench.py --summarize-traffic FETCH_DIR WRITE_DIR FETCH_COPY_DIR WRITE_COPY_DIR
+        turns the four rocprofv3 --pmc output directories (attention kernel and the 256 MiB
+        calibration copy, one counter each) into the text of profiles/<kernel>_hbm_traffic.txt
 """
 import argparse
 import ctypes
@@ -33,11 +41,131 @@ PEAK_FP8_TOPS = 5000.0       # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0
 K_FLAGS = 3                  # K mean smoothing + per-channel Q/K balancing (the default recipe)
 
-# HBM bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
-# (KiB per dispatch, one run each) scaled by the readings of the same counters for a 256 MiB
-# device copy (--copy-calibration): fetch 54 520 KiB x 2.000, write 76 390 KiB x 1.000.
-# Keyed by (workload id, variant); other workloads have not been measured.
-MEASURED_ATTN_TRAFFIC_BYTES = {(2, 0): int(54520 * 1024 * 2.0 + 76390 * 1024 * 1.0)}
+KERNEL_SOURCES = ("mojodiffusion_amd/csrc/sage_attn.hip", "mojodiffusion_amd/csrc/sage_internal.h")
+
+
+def kernel_source_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def traffic_summary_path(workload_name):
+    return os.path.join(ROOT, "profiles", "attention_%s_hbm_traffic.txt" % workload_name)
+
+
+def measured_traffic(workload_name):
+    """HBM bytes per launch of the attention kernel from the committed counter summary, or None
+    when there is none for this workload or the kernel's source has changed since it was taken."""
+    path = traffic_summary_path(workload_name)
+    if not os.path.exists(path):
+        return None
+    kv = {}
+    for line in open(path):
+        if "=" in line and not line.lstrip().startswith("#"):
+            k, v = line.split("=", 1)
+            kv[k.strip()] = v.strip()
+    if kv.get("kernel_source_digest") != kernel_source_digest():
+        return None
+    return int(kv["traffic_bytes_per_launch"])
+
+
+def summarize_traffic(dirs):
+    """rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE report KiB per dispatch.  The same counters on a
+    plain 256 MiB device copy (which reads and writes exactly 256 MiB) give the scale factors."""
+    import csv
+    import glob
+
+    def avg(d, pattern):
+        f = glob.glob(os.path.join(d, "*counter_collection.csv"))
+        vals = [float(r["Counter_Value"]) for r in csv.DictReader(open(f[0])) if pattern in r["Kernel_Name"]]
+        # the copy kernel is the one whose value is largest (torch launches helpers too)
+        return sum(vals) / len(vals), len(vals)
+
+    def copy_avg(d):
+        f = glob.glob(os.path.join(d, "*counter_collection.csv"))
+        by = {}
+        for r in csv.DictReader(open(f[0])):
+            by.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        name = max(by, key=lambda k: sum(by[k]) / len(by[k]))
+        return sum(by[name]) / len(by[name]), name
+    fetch, n_f = avg(dirs[0], "sage_attn_kernel")
+    write, n_w = avg(dirs[1], "sage_attn_kernel")
+    fetch_copy, cname = copy_avg(dirs[2])
+    write_copy, _ = copy_avg(dirs[3])
+    copy_kib = 256.0 * 1024.0
+    f_scale, w_scale = copy_kib / fetch_copy, copy_kib / write_copy
+    total = int(round((fetch * f_scale + write * w_scale) * 1024.0))
+    print("# HBM traffic of sage_attn_kernel per launch, rocprofv3 --pmc (one counter per run)")
+    print("kernel_source_digest = %s" % kernel_source_digest())
+    print("fetch_size_kib_per_dispatch = %.1f   # %d dispatches" % (fetch, n_f))
+    print("write_size_kib_per_dispatch = %.1f   # %d dispatches" % (write, n_w))
+    print("copy_kernel = %s" % cname.split("(")[0][:80])
+    print("copy_fetch_size_kib = %.1f   # for 262144 KiB read: scale %.4f" % (fetch_copy, f_scale))
+    print("copy_write_size_kib = %.1f   # for 262144 KiB written: scale %.4f" % (write_copy, w_scale))
+    print("traffic_bytes_per_launch = %d" % total)
+
+
+
+def clock_probe(args, L, w, qd, kd, vd, o, st, stream):
+    """The chip lowers its shader clock under this kernel (power management).  The measurement
+    build's attention kernel stamps s_memtime (shader clocks) and s_memrealtime (100 MHz) at its
+    start and end; their ratio is the clock each workgroup ran at."""
+    import numpy as np
+    import torch
+    from mojodiffusion_amd import _lib
+    P = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libmi355_sage_probe.so"))
+    for name in ("mi355_sage_quant_qk_bf16", "mi355_sage_quant_v_f16", "mi355_sage_quant_v_fp8", "mi355_sage_attn_fwd"):
+        getattr(P, name).restype, getattr(P, name).argtypes = _lib.SIGNATURES[name]
+    B, S, H, D = w.B, w.S, w.H, w.D
+    dev = qd.device
+    nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
+    q8 = torch.empty((B, H, nqp, D), dtype=torch.int8, device=dev)
+    k8 = torch.empty((B, H, nkp, D), dtype=torch.int8, device=dev)
+    qs = torch.empty((B, H, nqp // w.blkq), dtype=torch.float32, device=dev)
+    ks = torch.empty((B, H, nkp // w.blkk), dtype=torch.float32, device=dev)
+    km, qm, kmu, vsc = (torch.empty((B, H, D), dtype=torch.float32, device=dev) for _ in range(4))
+    vq = torch.empty((B, H, nkp // 64, D, 64), dtype=torch.int16 if w.variant == 0 else torch.uint8, device=dev)
+    scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, H, S, D), 8), dtype=torch.uint8, device=dev)
+    nwg = (nqp // 256) * B * H
+    stats = torch.zeros(B * H * S + 2 * nwg, dtype=torch.float32, device=dev)      # Stats, then the stamps
+    assert P.mi355_sage_quant_qk_bf16(qd.data_ptr(), kd.data_ptr(), B, H, S, S, D, w.scale, st, st, 0, 0, w.blkq, w.blkk,
+                                      K_FLAGS, 0, 0, q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(),
+                                      km.data_ptr(), qm.data_ptr(), kmu.data_ptr(), scr.data_ptr(), scr.numel(), stream) == 0
+    if w.variant == 0:
+        assert P.mi355_sage_quant_v_f16(vd.data_ptr(), B, H, S, D, st, 0, 0, 0, vq.data_ptr(), stream) == 0
+    else:
+        assert P.mi355_sage_quant_v_fp8(vd.data_ptr(), B, H, S, D, st, 0, 0, 0, vq.data_ptr(), vsc.data_ptr(),
+                                        scr.data_ptr(), scr.numel(), stream) == 0
+
+    def attn():
+        assert P.mi355_sage_attn_fwd(q8.data_ptr(), qs.data_ptr(), w.blkq, k8.data_ptr(), ks.data_ptr(), w.blkk,
+                                     vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, 0, 0, D,
+                                     o.data_ptr(), st, 0, None, stats.data_ptr(), stream) == 0
+    for _ in range(args.warmup + args.steps):               # back to back, as in a sampler's layer loop
+        attn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    attn()
+    b.record()
+    torch.cuda.synchronize()
+    x = stats[B * H * S:].cpu().numpy().reshape(nwg, 2).astype(np.float64)
+    mhz = x[:, 0] / x[:, 1] * 100.0
+    tiles = (S + 63) // 64
+    per_xcd = [round(float(np.median(mhz[i::8])), 1) for i in range(8)]     # consecutive workgroups go to the 8 XCDs in turn
+    print(json.dumps({
+        "workload": w.name, "kernel_ms": round(a.elapsed_time(b), 5), "workgroups": nwg,
+        "shader_clock_mhz": {"mean": round(float(mhz.mean()), 1), "median": round(float(np.median(mhz)), 1),
+                             "p10": round(float(np.quantile(mhz, 0.1)), 1), "p90": round(float(np.quantile(mhz, 0.9)), 1)},
+        "median_shader_clock_mhz_per_xcd": per_xcd,
+        "shader_clocks_per_workgroup": round(float(x[:, 0].mean()), 0),
+        "shader_clocks_per_64_key_tile": round(float(x[:, 0].mean()) / tiles, 1),
+        "matrix_pipe_clocks_per_tile_per_simd": 2 * (8 * 32 + (16 * 32 if w.variant == 0 else 4 * 64)),
+    }))
 
 
 def main():
@@ -47,10 +175,19 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--summarize-traffic", nargs=4, metavar="DIR",
+                    help="print the traffic summary from four rocprofv3 --pmc output directories (no GPU needed)")
+    ap.add_argument("--clock-probe", action="store_true",
+                    help="run the attention kernel of the measurement build (libmi355_sage_probe.so), which records "
+                         "its own shader cycles and elapsed constant-rate time per workgroup, and print the clock "
+                         "the chip sustained under it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain device copy of 256 MiB (read 256 MiB, write 256 MiB) five times: "
                          "the known-size kernel the HBM traffic counters are scaled by")
     args = ap.parse_args()
+    if args.summarize_traffic:
+        summarize_traffic(args.summarize_traffic)
+        return
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this hot path is measured on ONE GPU (heads are independent and would shard "
               "without any exchange); run with --gpus 1", file=sys.stderr)
@@ -104,6 +241,36 @@ def main():
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     tops = w.ops / (ms_per_step * 1e-3) / 1e12
+
+    if args.clock_probe:
+        clock_probe(args, L, w, qd, kd, vd, o, st, stream)
+        return
+
+    # ---- the same step replayed from a HIP graph (launch gaps shrink to the graph's own) -----
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            cap_stream = torch.cuda.current_stream().cuda_stream
+            with torch.cuda.graph(g, stream=side):
+                rc = L.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
+                                               B, H, S, S, D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, cap_stream,
+                                               w.variant, w.blkq, w.blkk, K_FLAGS, ws.data_ptr(), nws)
+            if rc != 0:
+                raise RuntimeError("capture rc=%d" % rc)
+            for _ in range(args.warmup):
+                g.replay()
+            torch.cuda.synchronize()
+            g0 = time.perf_counter()
+            for _ in range(args.steps):
+                g.replay()
+            torch.cuda.synchronize()
+            graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
+    except Exception as e:                                  # reported, never fatal for the headline number
+        print("bench.py: graph replay timing skipped: %r" % (e,), file=sys.stderr)
+    torch.cuda.synchronize()
 
     # ---- stage timings with HIP events on the launch stream -------------------------
     nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
@@ -181,6 +348,7 @@ def main():
             # into two launches, so its quantize share is about ms_per_step - attn)
             "stage_ms": {"quant_qk": round(qk_avg, 5), "quant_v": round(v_avg, 5), "attn": round(at_avg, 5)},
             "one_shot_quant_ms": round(ms_per_step - at_avg, 5),
+            "graph_replay_ms": None if graph_ms is None else round(graph_ms, 5),
             "quant_stage_hbm": {"algorithmic_bytes": quant_bytes, "GB/s": round(quant_gbs, 1),
                                 "frac_of_8TB/s": round(quant_gbs / PEAK_HBM_GBS, 4)},
             "device": torch.cuda.get_device_name(0),
@@ -192,7 +360,7 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(attn_tops / peak, 4),
-            "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, w.variant)),
+            "traffic": measured_traffic(w.name),
             # int8 Q and K read once, V^T tiles (fp16 or e4m3) read once, bf16 O written once
             "algorithmic_bytes_per_launch": 2 * elems + elems * (2 if w.variant == 0 else 1) + 2 * elems,
             "avg_ms": round(at_avg, 5), "median_ms": round(at_med, 5), "min_ms": round(at_min, 5),

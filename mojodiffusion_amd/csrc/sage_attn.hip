@@ -170,6 +170,12 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int64_t bh = wg / n_qtiles;
     const int b = (int)(bh / H), h = (int)(bh % H);
 
+#ifdef SAGE_CLOCK_PROBE
+    // Measurement build only (libmi355_sage_probe.so): shader cycles and constant-rate time of
+    // this workgroup, written behind the [B,H,Nq] Stats output (the caller sizes the buffer).
+    const unsigned long long probe_r0 = __builtin_amdgcn_s_memrealtime();
+    const unsigned long long probe_t0 = __builtin_readcyclecounter();
+#endif
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
@@ -555,6 +561,18 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             stats[bh * Nq + qrow] = (m_used + __builtin_amdgcn_logf(l_tot) - Lazy<VARIANT>::log2_pscale + shift) * 0.6931471805599453f;
         }
     }
+#ifdef SAGE_CLOCK_PROBE
+    if (STATS) {
+        __syncthreads();
+        const unsigned long long probe_t1 = __builtin_readcyclecounter();
+        const unsigned long long probe_r1 = __builtin_amdgcn_s_memrealtime();
+        if (tid == 0) {
+            float* probe = stats + (int64_t)(total_wg / n_qtiles) * Nq + blockIdx.x * 2;
+            probe[0] = (float)(probe_t1 - probe_t0);          // shader clocks
+            probe[1] = (float)(probe_r1 - probe_r0);          // 100 MHz ticks
+        }
+    }
+#endif
 }
 
 template <int D, int VARIANT>

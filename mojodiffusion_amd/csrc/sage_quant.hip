@@ -520,8 +520,8 @@ hipError_t launch_prep(const PrepArgs& a_in, int B, int D, hipStream_t st) {
 //      kmul = 1/s, qmul = cmul*s.
 //   V: vscale = amax/448 (1 when 0).
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void stats_final_kernel(FinalArgs a) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;      // (bh, d)
+__global__ __launch_bounds__(64) void stats_final_kernel(FinalArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;      // (bh, d)
     if (i >= a.total) return;
     const int64_t bh = i / a.D;
     const int d = (int)(i % a.D);
@@ -532,18 +532,20 @@ __global__ __launch_bounds__(256) void stats_final_kernel(FinalArgs a) {
             const float* q = a.kpart_mm + 2 * (bh * a.ngroups * a.D + d);
             double sum = 0.0;
             float mn = INFINITY, mx = -INFINITY;
-            for (int g0 = 0; g0 < a.ngroups; g0 += 8) {
-                double v[8];
-                float lo[8], hi[8];
+            // loads 32 groups at a time (all independent, in flight together); sums strictly in group order
+            constexpr int NB = 32;
+            for (int g0 = 0; g0 < a.ngroups; g0 += NB) {
+                double v[NB];
+                float lo[NB], hi[NB];
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
+                for (int j = 0; j < NB; j++) {
                     const int64_t g = g0 + j < a.ngroups ? g0 + j : a.ngroups - 1;
                     v[j] = p[g * a.D];
                     lo[j] = q[2 * g * a.D];
                     hi[j] = q[2 * g * a.D + 1];
                 }
 #pragma unroll
-                for (int j = 0; j < 8; j++)
+                for (int j = 0; j < NB; j++)
                     if (g0 + j < a.ngroups) { sum += v[j]; mn = fminf(mn, lo[j]); mx = fmaxf(mx, hi[j]); }
             }
             if (a.flags & 1) mean = (float)(sum / (double)a.kept);
@@ -566,7 +568,7 @@ __global__ __launch_bounds__(256) void stats_final_kernel(FinalArgs a) {
 
 hipError_t launch_stats_final(const FinalArgs& a, hipStream_t st) {
     if (a.total <= 0) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(stats_final_kernel, dim3((unsigned)((a.total + 255) / 256)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(stats_final_kernel, dim3((unsigned)((a.total + 63) / 64)), dim3(64), 0, st, a);
     return hipGetLastError();
 }
 
