@@ -256,6 +256,106 @@ int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, 
     return err ? -1 : 0;
 }
 
+/* ---- backward of the full-precision SDPA ---------------------------------- */
+/* The decomposed backward of serenitymojo/ops/attention_backward.mojo:12-19,
+ *   attn = softmax(Q K^T * scale);  dV = attn^T dO;  dA = dO V^T;
+ *   dS = attn * (dA - rowsum(dA * attn));  dQ = dS K * scale;  dK = dS^T Q * scale,
+ * in double precision on one (b,h) at a time.  With `o` and `stats` NULL the probabilities
+ * are recomputed from q and k (what torch.autograd does to ops/parity/sdpa_bwd_oracle.py:56-63);
+ * with both given (the flash interface of ops/cshim/cudnn_sdpa_bwd.cpp:325-347) they are
+ * attn = exp(score - stats[row]) with the caller's log-sum-exp, and rowsum(dA * attn) is taken as
+ * rowsum(dO * O) — equal in exact arithmetic, and what a kernel that never holds a whole row has
+ * to use.  Query rows >= real_nq and keys >= real_nkv are padding: they take no part and their
+ * gradient rows are zero (cudnn_sdpa_bwd.cpp:344 real_N_q / real_N_kv). */
+int sage_oracle_sdpa_bwd_f32(const float* q, const float* k, const float* v, const float* o,
+                             const float* dout, const float* stats,
+                             float* dq, float* dk, float* dv,
+                             int B, int H, int Nq, int Nkv, int D, float scale,
+                             const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                             const int64_t* dos, const int64_t* dqs, const int64_t* dks, const int64_t* dvs,
+                             int real_nq, int real_nkv) {
+    if (!q || !k || !v || !dout || !dq || !dk || !dv) return -1;
+    if ((o == NULL) != (stats == NULL)) return -1;
+    if (B <= 0 || H <= 0 || Nq <= 0 || Nkv <= 0 || D <= 0) return -1;
+    if (!qs || !ks || !vs || !dos || !dqs || !dks || !dvs || (o && !os)) return -1;
+    const int nq = real_nq > 0 && real_nq < Nq ? real_nq : Nq;
+    const int nk = real_nkv > 0 && real_nkv < Nkv ? real_nkv : Nkv;
+    double* P = (double*)malloc(sizeof(double) * (size_t)nq * (size_t)nk);
+    double* dS = (double*)malloc(sizeof(double) * (size_t)nq * (size_t)nk);
+    if (!P || !dS) { free(P); free(dS); return -1; }
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < H; h++) {
+            const float* qb = q + b * qs[0] + h * qs[1];
+            const float* kb = k + b * ks[0] + h * ks[1];
+            const float* vb = v + b * vs[0] + h * vs[1];
+            const float* gb = dout + b * dos[0] + h * dos[1];
+#pragma omp parallel for schedule(dynamic, 8)
+            for (int i = 0; i < nq; i++) {
+                const float* qr = qb + i * qs[2];
+                const float* gr = gb + i * dos[2];
+                double* Pr = P + (size_t)i * nk;
+                double* Sr = dS + (size_t)i * nk;
+                double mx = -INFINITY;
+                for (int j = 0; j < nk; j++) {
+                    const float* kr = kb + j * ks[2];
+                    double dot = 0.0;
+                    for (int d = 0; d < D; d++) dot += (double)qr[d * qs[3]] * (double)kr[d * ks[3]];
+                    Pr[j] = dot * (double)scale;
+                    if (Pr[j] > mx) mx = Pr[j];
+                }
+                double delta = 0.0;
+                if (stats) {
+                    const double lse = (double)stats[((int64_t)b * H + h) * Nq + i];
+                    for (int j = 0; j < nk; j++) Pr[j] = exp(Pr[j] - lse);
+                    const float* orow = o + b * os[0] + h * os[1] + i * os[2];
+                    for (int d = 0; d < D; d++) delta += (double)gr[d * dos[3]] * (double)orow[d * os[3]];
+                } else {
+                    double l = 0.0;
+                    for (int j = 0; j < nk; j++) { Pr[j] = exp(Pr[j] - mx); l += Pr[j]; }
+                    for (int j = 0; j < nk; j++) Pr[j] /= l;
+                }
+                for (int j = 0; j < nk; j++) {
+                    const float* vr = vb + j * vs[2];
+                    double da = 0.0;
+                    for (int d = 0; d < D; d++) da += (double)gr[d * dos[3]] * (double)vr[d * vs[3]];
+                    Sr[j] = da;
+                    if (!stats) delta += da * Pr[j];
+                }
+                for (int j = 0; j < nk; j++) Sr[j] = Pr[j] * (Sr[j] - delta);
+                float* dqr = dq + b * dqs[0] + h * dqs[1] + i * dqs[2];
+                for (int d = 0; d < D; d++) {
+                    double a = 0.0;
+                    for (int j = 0; j < nk; j++) a += Sr[j] * (double)kb[j * ks[2] + d * ks[3]];
+                    dqr[d * dqs[3]] = (float)(a * (double)scale);
+                }
+            }
+#pragma omp parallel for schedule(dynamic, 8)
+            for (int j = 0; j < nk; j++) {
+                float* dkr = dk + b * dks[0] + h * dks[1] + j * dks[2];
+                float* dvr = dv + b * dvs[0] + h * dvs[1] + j * dvs[2];
+                for (int d = 0; d < D; d++) {
+                    double ak = 0.0, av = 0.0;
+                    for (int i = 0; i < nq; i++) {
+                        ak += dS[(size_t)i * nk + j] * (double)qb[i * qs[2] + d * qs[3]];
+                        av += P[(size_t)i * nk + j] * (double)gb[i * dos[2] + d * dos[3]];
+                    }
+                    dkr[d * dks[3]] = (float)(ak * (double)scale);
+                    dvr[d * dvs[3]] = (float)av;
+                }
+            }
+            for (int i = nq; i < Nq; i++)
+                for (int d = 0; d < D; d++) dq[b * dqs[0] + h * dqs[1] + i * dqs[2] + d * dqs[3]] = 0.0f;
+            for (int j = nk; j < Nkv; j++)
+                for (int d = 0; d < D; d++) {
+                    dk[b * dks[0] + h * dks[1] + j * dks[2] + d * dks[3]] = 0.0f;
+                    dv[b * dvs[0] + h * dvs[1] + j * dvs[2] + d * dvs[3]] = 0.0f;
+                }
+        }
+    free(P);
+    free(dS);
+    return 0;
+}
+
 /* ------------------------------------------------------------------------ */
 /* quantizers                                                               */
 /* ------------------------------------------------------------------------ */

@@ -80,6 +80,23 @@ int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, 
                                 const int64_t* qs, const int64_t* ks,
                                 const int64_t* vs, const int64_t* os);
 
+/* ---- backward of the full-precision SDPA ------------------------------------ */
+/* Decomposed backward in double precision, restating serenitymojo/ops/attention_backward.mojo:12-19.
+ * o == stats == NULL: probabilities recomputed from q, k (the torch.autograd reference of
+ * ops/parity/sdpa_bwd_oracle.py:56-63).  Both given: the flash interface of
+ * ops/cshim/cudnn_sdpa_bwd.cpp:325-347 — attn = exp(score - stats[row]) and the softmax-backward
+ * row term is rowsum(dO * O).  stats contiguous [B,H,Nq] (natural log).  Rows >= real_nq and keys
+ * >= real_nkv (0: all) are padding; their gradients are zero.  Pinned by the reference's golden
+ * gradients ops/parity/sdpa_bwd_ref.txt, torch.autograd in float64, central differences, and the
+ * invariance of attention to a common shift of all keys (sum over keys of dK is zero). */
+int sage_oracle_sdpa_bwd_f32(const float* q, const float* k, const float* v, const float* o,
+                             const float* dout, const float* stats,
+                             float* dq, float* dk, float* dv,
+                             int B, int H, int Nq, int Nkv, int D, float scale,
+                             const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                             const int64_t* dos, const int64_t* dqs, const int64_t* dks, const int64_t* dvs,
+                             int real_nq, int real_nkv);
+
 /* ---- the two ops in front of the path (fused into the quantizers by the product) ---- */
 /* RMSNorm rows x cols in fp32: serenitymojo/ops/norm.mojo:47-79.  Pinned by the reference's
  * vector serenitymojo/ops_smoke.mojo:78-96 and the closed form of ops_smoke2.mojo:372-403;

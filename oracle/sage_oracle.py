@@ -61,6 +61,9 @@ def lib():
         L.sage_oracle_sdpa_f32_ex.restype = ctypes.c_int
         L.sage_oracle_sdpa_f32_ex.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [
                                               ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        L.sage_oracle_sdpa_bwd_f32.restype = ctypes.c_int
+        L.sage_oracle_sdpa_bwd_f32.argtypes = [ctypes.c_void_p] * 9 + [ctypes.c_int] * 5 + [ctypes.c_float] + [_i64p] * 8 + [
+                                               ctypes.c_int, ctypes.c_int]
         L.sage_oracle_kstats.restype = ctypes.c_int
         L.sage_oracle_kstats.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_float] + [ctypes.c_int] * 3 + [
                                          ctypes.c_void_p] * 3
@@ -208,6 +211,25 @@ def sdpa_f32(q, k, v, scale, online=False, mask_lo=0, mask_hi=0, addmask=None, w
     stats = np.empty((B, H, Sq), np.float32) if want_stats else None
     _chk(lib().sage_oracle_sdpa_f32_ex(*args, mask_lo, mask_hi, _p(addmask), _p(stats)), "sdpa_f32")
     return (o, stats) if want_stats else o
+
+
+def sdpa_bwd_f32(q, k, v, dout, scale, o=None, stats=None, real_nq=0, real_nkv=0):
+    """Gradients (dq, dk, dv), fp32 [B,S,H,D], of softmax(q k^T * scale) v against the upstream
+    gradient dout.  With o [B,Sq,H,D] and stats [B,H,Sq] given, the flash form: probabilities from
+    the caller's log-sum-exp, row term rowsum(dout * o).  real_nq / real_nkv: valid lengths."""
+    q, k, v, dout = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v, dout))
+    B, H, Sq, Skv, D = _dims_bshd(q, k)
+    assert (o is None) == (stats is None)
+    if o is not None:
+        o = np.ascontiguousarray(o, dtype=np.float32)
+        stats = np.ascontiguousarray(stats, dtype=np.float32)
+        assert o.shape == q.shape and stats.shape == (B, H, Sq)
+    dq, dk, dv = np.empty_like(q), np.empty_like(k), np.empty_like(v)
+    sq, sk = strides_bshd(Sq, H, D), strides_bshd(Skv, H, D)
+    _chk(lib().sage_oracle_sdpa_bwd_f32(_p(q), _p(k), _p(v), _p(o), _p(dout), _p(stats), _p(dq), _p(dk), _p(dv),
+                                        B, H, Sq, Skv, D, scale, sq, sk, sk, sq, sq, sq, sk, sk,
+                                        real_nq, real_nkv), "sdpa_bwd_f32")
+    return dq, dk, dv
 
 
 def rms_norm_f32(x, g, eps):

@@ -7,6 +7,8 @@ no reference code is imported or executed.
 Sources (relative to the reference checkout):
   serenitymojo/ops/parity/sdpa_math_ref.txt        tags dh128 [1,8,32,128], dh512 [1,64,1,512]
       inputs are the closed forms of ops/parity/sdpa_math_parity.mojo:32-50
+  serenitymojo/ops/parity/sdpa_bwd_ref.txt         gradients dq/dk/dv for tags dh128 [1,8,32,128], dh64 [1,8,8,64]
+      inputs are the closed forms of ops/parity/sdpa_bwd_parity.mojo:44-65
   serenitymojo/ops_smoke2.mojo:239-278              q/k/v/out literals, [1,4,2,8], scale 0.35355339
   serenitymojo/ops_smoke.mojo:78-96                 rms_norm x[3,6], g[6], eps 1e-6 -> y[3,6]
   serenitymojo/ops_smoke2.mojo:92-120               rope x[3,8], cos/sin[3,4] -> interleaved y[3,8]
@@ -33,6 +35,17 @@ def main():
                 out[parts[0]] = np.array([float(x) for x in parts[1:]], dtype=np.float64)
     assert out["dh128"].size == 1 * 8 * 32 * 128 and out["dh512"].size == 1 * 64 * 1 * 512
     np.savez_compressed(os.path.join(HERE, "sdpa_math_ref.npz"), dh128=out["dh128"], dh512=out["dh512"])
+
+    bwd = {}
+    with open(os.path.join(ref, "serenitymojo/ops/parity/sdpa_bwd_ref.txt")) as f:
+        for line in f:
+            parts = line.split()
+            if parts:
+                bwd[parts[0]] = np.array([float(x) for x in parts[1:]], dtype=np.float64)
+    for tag, n in (("dh128", 1 * 8 * 32 * 128), ("dh64", 1 * 8 * 8 * 64)):
+        for g in ("dq", "dk", "dv"):
+            assert bwd[tag + "_" + g].size == n, (tag, g)
+    np.savez_compressed(os.path.join(HERE, "sdpa_bwd_ref.npz"), **bwd)
 
     with open(os.path.join(ref, "serenitymojo/ops_smoke2.mojo")) as f:
         lines = f.read().split("\n")
