@@ -305,6 +305,35 @@ int mi355_sage_attn_fwd(
     void* O, const int64_t* o_strides, int64_t o_offset_elems,
     const void* qshift, void* stats, void* stream);
 
+/* Backward.  Replaces flame_cudnn_sdpa_bwd_bf16 (serenitymojo/ops/cshim/cudnn_sdpa_bwd.cpp:325-347;
+ * Mojo callers ops/attention_flash.mojo:345-433, :478-535, :538-607): identical parameter list up
+ * to `stream`, then the workspace pair.  Q, K, V, O, dO bf16 and dQ, dK, dV bf16, each a logical
+ * [B,H,N,D] view through 4 element strides + an element offset; Stats fp32 contiguous [B,H,N_q]
+ * (natural-log log-sum-exp, as the train-forward entry points write it).  Computes, without ever
+ * storing an N_q x N_kv matrix,
+ *     P = exp(scale * Q K^T - Stats),  dV = P^T dO,  dS = P * (dO V^T - rowsum(dO * O)),
+ *     dQ = scale * dS K,  dK = scale * dS^T Q
+ * in bf16 matrix instructions with fp32 accumulation (no quantization: gradients keep bf16
+ * operands).  real_N_q / real_N_kv (0 or >= N: all) are the valid lengths; padding rows and keys
+ * take no part and their gradient rows are written as zeros.  causal must be 0.
+ * Workspace: mi355_sage_bwd_workspace_bytes(...) bytes, 256-byte aligned, or NULL for the
+ * library's per-stream buffer (same rules as the forward).  Unlike the log-sum-exp handed to
+ * cuDNN, Stats may come from the quantized forward: the probabilities are then normalised by the
+ * quantized scores' sum, which differs from the bf16 one by the forward's own error. */
+size_t mi355_sage_bwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D);
+int mi355_sage_sdpa_bwd_bf16(
+    const void* Q, const void* K, const void* V, const void* O, const void* dO, const void* Stats,
+    void* dQ, void* dK, void* dV,
+    int B, int H, int N_q, int N_kv, int D, float scale,
+    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+    const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+    const int64_t* dk_strides, const int64_t* dv_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems, int64_t o_offset_elems,
+    int64_t do_offset_elems, int64_t stats_offset_elems, int64_t dq_offset_elems,
+    int64_t dk_offset_elems, int64_t dv_offset_elems,
+    int causal, int real_N_q, int real_N_kv, void* stream,
+    void* workspace, size_t workspace_bytes);
+
 /* Library identification: "mi355_sage <version> gfx950". */
 const char* mi355_sage_version(void);
 

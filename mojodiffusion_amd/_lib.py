@@ -27,6 +27,9 @@ SIGNATURES = {
     "mi355_sage_sdpa_bf16_mask": (_int, [_vp] * 5 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 5 + [_i64] * 5
                                   + [_vp, _int, _vp, ctypes.c_size_t]),
     "mi355_sage_workspace_bytes": (ctypes.c_size_t, [_int] * 6),
+    "mi355_sage_bwd_workspace_bytes": (ctypes.c_size_t, [_int] * 5),
+    "mi355_sage_sdpa_bwd_bf16": (_int, [_vp] * 9 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 8 + [_i64] * 9
+                                 + [_int, _int, _int, _vp, _vp, ctypes.c_size_t]),
     "mi355_sage_pad_q": (_i64, [_i64]),
     "mi355_sage_pad_kv": (_i64, [_i64]),
     "mi355_sage_v_slot": (_int, [_int, _int]),

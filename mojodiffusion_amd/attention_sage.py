@@ -152,6 +152,74 @@ def sdpa_flash_train_fwd_f32(q, k, v, scale, variant=PV_FP16):
     return fwd.o.to(torch.float32), fwd
 
 
+@dataclass
+class SdpaFlashGrads:
+    """serenitymojo/ops/attention_flash.mojo:138-146."""
+    d_q: torch.Tensor
+    d_k: torch.Tensor
+    d_v: torch.Tensor
+
+
+def _call_bwd(name, q, k, v, o, d_out, stats, scale, real_q, real_kv):
+    B, Sq, H, Dh = q.shape
+    Skv = k.shape[1]
+    L = _lib.lib()
+    d_q, d_k, d_v = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ws = _workspace(max(L.mi355_sage_bwd_workspace_bytes(B, H, Sq, Skv, Dh), 256), q.device)
+    qs = _lib.strides_bhnd(Sq, H, Dh)
+    ks = _lib.strides_bhnd(Skv, H, Dh)
+    stream = torch.cuda.current_stream(q.device).cuda_stream
+    rc = L.mi355_sage_sdpa_bwd_bf16(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d_out.data_ptr(), stats.data_ptr(),
+        d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(),
+        B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, qs, qs, ks, ks,
+        0, 0, 0, 0, 0, 0, 0, 0, 0,
+        0, real_q, real_kv, stream, ws.data_ptr(), ws.numel())
+    if rc != 0:
+        raise Error("%s: shim rc=%d (B=%d Sq=%d Skv=%d H=%d Dh=%d)" % (name, rc, B, Sq, Skv, H, Dh))
+    return SdpaFlashGrads(d_q, d_k, d_v)
+
+
+def sdpa_flash_backward(fwd, d_out, scale, real_len=None):
+    """dQ/dK/dV [B,S,H,Dh] BF16 from the saved train-forward set and the upstream d_out
+    (attention_flash.mojo:345-433).  The reference pads the sequence to 128 around its call; the
+    kernels here take any length, so the saved tensors are used as they are.  real_len: the valid
+    length of a sdpa_flash_fwd_padmask forward (rows and keys at and beyond it get zero gradients)."""
+    name = "sdpa_flash_backward"
+    _require_bf16(name, fwd.q_pad, fwd.k_pad, fwd.v_pad, fwd.o_pad)
+    if d_out.dtype != torch.bfloat16:
+        raise Error("%s: d_out must be BF16" % name)
+    if d_out.shape != fwd.o_pad.shape:
+        raise Error("%s: d_out shape does not match the forward output" % name)
+    _require_cuda(name, fwd.q_pad, fwd.k_pad, fwd.v_pad, fwd.o_pad, d_out, fwd.stats)
+    rq = fwd.q_pad.shape[1] if real_len is None else real_len
+    rk = fwd.k_pad.shape[1] if real_len is None else real_len
+    return _call_bwd(name, fwd.q_pad, fwd.k_pad, fwd.v_pad, fwd.o_pad, d_out, fwd.stats, scale, rq, rk)
+
+
+def sdpa_flash_backward_f32(q_bf, k_bf, v_bf, o_bf, stats, d_att, scale):
+    """F32 gradient in and out around the bf16 backward (attention_flash.mojo:478-535): d_att F32
+    -> bf16, dQ/dK/dV bf16 -> F32.  The reference accepts 128-aligned S only on this path."""
+    name = "sdpa_flash_backward_f32"
+    if q_bf.shape[1] % 128 != 0:
+        raise Error("%s: S must be 128-aligned" % name)
+    _require_bf16(name, q_bf, k_bf, v_bf, o_bf)
+    do_bf = d_att.to(torch.bfloat16)
+    _require_cuda(name, q_bf, k_bf, v_bf, o_bf, do_bf, stats)
+    g = _call_bwd(name, q_bf, k_bf, v_bf, o_bf, do_bf, stats, scale, q_bf.shape[1], k_bf.shape[1])
+    return SdpaFlashGrads(g.d_q.to(torch.float32), g.d_k.to(torch.float32), g.d_v.to(torch.float32))
+
+
+def sdpa_flash_backward_raw(q_pad, k_pad, v_pad, o_pad, stats, d_out, scale):
+    """bf16 in and out on the saved set of the graph path (attention_flash.mojo:538-607)."""
+    name = "sdpa_flash_backward_raw"
+    _require_bf16(name, q_pad, k_pad, v_pad, o_pad)
+    if d_out.dtype != torch.bfloat16:
+        raise Error("%s: d_out must be BF16" % name)
+    _require_cuda(name, q_pad, k_pad, v_pad, o_pad, d_out, stats)
+    return _call_bwd(name, q_pad, k_pad, v_pad, o_pad, d_out, stats, scale, q_pad.shape[1], k_pad.shape[1])
+
+
 def sdpa_nomask(q, k, v, scale, variant=PV_FP16):
     """Full attention without a mask tensor (attention.mojo:1690-1718): the entry
     every DiT sampler uses.  Output has q's dtype; F32/F16 storage is cast to

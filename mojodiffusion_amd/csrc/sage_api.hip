@@ -641,4 +641,96 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     return MI355_SAGE_OK;
 }
 
+// ---- backward ---------------------------------------------------------------------------------
+struct BwdCarve { size_t kT, qT, doT, lse2, delta, total; };
+static BwdCarve bwd_carve(int B, int H, int Nq, int Nkv, int D) {
+    const size_t bh = (size_t)B * H;
+    const size_t nqp = (size_t)pad_to(Nq, 64), nkp = (size_t)pad_to(Nkv, 64);
+    BwdCarve c{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
+    c.kT = take(bh * nkp * D * 2);
+    c.qT = take(bh * nqp * D * 2);
+    c.doT = take(bh * nqp * D * 2);
+    c.lse2 = take(bh * nqp * sizeof(float));
+    c.delta = take(bh * nqp * sizeof(float));
+    c.total = off;
+    return c;
+}
+
+size_t mi355_sage_bwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || !dims_ok(D)) return 0;
+    return bwd_carve(B, H, N_q, N_kv, D).total;
+}
+
+int mi355_sage_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                             const void* Stats, void* dQ, void* dK, void* dV,
+                             int B, int H, int N_q, int N_kv, int D, float scale,
+                             const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                             const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                             const int64_t* dk_strides, const int64_t* dv_strides,
+                             int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                             int64_t stats_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                             int causal, int real_N_q, int real_N_kv, void* stream,
+                             void* workspace, size_t workspace_bytes) {
+    // same order as serenitymojo/ops/cshim/cudnn_sdpa_bwd.cpp:348-352
+    if (!Q || !K || !V || !O || !dO || !Stats) return MI355_SAGE_EINVAL;
+    if (!dQ || !dK || !dV) return MI355_SAGE_EINVAL;
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
+    if (!q_strides || !k_strides || !v_strides || !o_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
+        return MI355_SAGE_EINVAL;
+    if (causal) { SAGE_LOG("causal attention is not supported"); return MI355_SAGE_EUNSUPPORTED; }
+    if (!dims_ok(D)) { SAGE_LOG("head dim %d is not supported (64 or 128)", D); return MI355_SAGE_EUNSUPPORTED; }
+    int rc;
+    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off)) ||
+        (rc = check_view("V", V, v_strides, v_off)) || (rc = check_view("O", O, o_strides, o_off)) ||
+        (rc = check_view("dO", dO, do_strides, do_off)) || (rc = check_view("dQ", dQ, dq_strides, dq_off)) ||
+        (rc = check_view("dK", dK, dk_strides, dk_off)) || (rc = check_view("dV", dV, dv_strides, dv_off)))
+        return rc;
+    // the tile copies address a head's rows with 32-bit byte offsets
+    auto span_ok = [&](const char* name, int N, const int64_t* s) {
+        if (s[2] < 0 || (uint64_t)(N - 1) * (uint64_t)s[2] * 2 + (uint64_t)D * 2 > 0xFFFFFFFFull) {
+            SAGE_LOG("%s: a head's rows span more than 4 GiB (or the row stride is negative)", name);
+            return false;
+        }
+        return true;
+    };
+    if (!span_ok("Q", N_q, q_strides) || !span_ok("dO", N_q, do_strides) || !span_ok("K", N_kv, k_strides) ||
+        !span_ok("V", N_kv, v_strides))
+        return MI355_SAGE_EUNSUPPORTED;
+
+    const BwdCarve c = bwd_carve(B, H, N_q, N_kv, D);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (workspace == nullptr) {
+        if ((rc = internal_workspace(c.total, st, &workspace))) return rc;
+    } else if (workspace_bytes < c.total || (reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1))) {
+        SAGE_LOG("backward workspace: %zu bytes at a 256-byte boundary needed, %zu given", c.total, workspace_bytes);
+        return MI355_SAGE_EWORKSPACE;
+    }
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    BwdArgs a{};
+    a.q = make_view(Q, q_strides, q_off);
+    a.k = make_view(K, k_strides, k_off);
+    a.v = make_view(V, v_strides, v_off);
+    a.o = make_view(O, o_strides, o_off);
+    a.dout = make_view(dO, do_strides, do_off);
+    a.stats = static_cast<const float*>(Stats) + stats_off;
+    a.dq = static_cast<uint16_t*>(dQ) + dq_off; a.dq_sb = dq_strides[0]; a.dq_sh = dq_strides[1]; a.dq_sn = dq_strides[2];
+    a.dk = static_cast<uint16_t*>(dK) + dk_off; a.dk_sb = dk_strides[0]; a.dk_sh = dk_strides[1]; a.dk_sn = dk_strides[2];
+    a.dv = static_cast<uint16_t*>(dV) + dv_off; a.dv_sb = dv_strides[0]; a.dv_sh = dv_strides[1]; a.dv_sn = dv_strides[2];
+    a.B = B; a.H = H; a.Nq = N_q; a.Nkv = N_kv; a.D = D;
+    a.valid_q = real_N_q > 0 && real_N_q < N_q ? real_N_q : N_q;          // cudnn_sdpa_bwd.cpp:362-363
+    a.valid_kv = real_N_kv > 0 && real_N_kv < N_kv ? real_N_kv : N_kv;
+    a.scale = scale;
+    a.kT = reinterpret_cast<uint16_t*>(ws + c.kT);
+    a.qT = reinterpret_cast<uint16_t*>(ws + c.qT);
+    a.doT = reinterpret_cast<uint16_t*>(ws + c.doT);
+    a.lse2 = reinterpret_cast<float*>(ws + c.lse2);
+    a.delta = reinterpret_cast<float*>(ws + c.delta);
+    a.nq_pad = pad_to(N_q, 64);
+    a.nkv_pad = pad_to(N_kv, 64);
+    SAGE_HIP(launch_bwd(a, st));
+    return 0;
+}
+
 }  // extern "C"

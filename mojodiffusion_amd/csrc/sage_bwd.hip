@@ -1,0 +1,407 @@
+// sage_bwd.hip — backward of scaled-dot-product attention in bf16 for gfx950.
+//
+// Flash-style: no N_q x N_kv matrix is ever stored.  From Q, K, V, O, dO (bf16) and the forward's
+// log-sum-exp Stats (fp32) the probabilities are recomputed tile by tile,
+//     P = exp(scale * Q K^T - Stats[row]),   Delta[row] = sum_d dO * O,
+//     dV = P^T dO,   dS = P * (dO V^T - Delta),   dQ = scale * dS K,   dK = scale * dS^T Q,
+// with v_mfma_f32_32x32x16_bf16, fp32 accumulation, P and dS rounded to bf16 as matrix operands.
+//
+// Three launches:
+//   1. bwd_prep_kernel     Delta and Stats * log2(e) per query row (padding rows: +inf, so their
+//                          probabilities vanish), and transposed copies K^T, Q^T, dO^T in tiles of
+//                          64 rows whose rows sit in the slot order of the matrix instruction's
+//                          operand layout (v_slot_f16).
+//   2. bwd_pass_kernel<0>  owner = 128 query rows per workgroup, loop over key tiles   -> dQ
+//   3. bwd_pass_kernel<1>  owner = 128 keys per workgroup, loop over query tiles       -> dK, dV
+// In both passes a wave owns 32 rows ("x"), keeps their two bf16 row blocks resident as B operands
+// and walks the other side ("y") in tiles of 64 rows staged in LDS by register-bypassing copies,
+// double buffered, one barrier per tile.  A 32x32 block of scores T[y,x] lands in the accumulator
+// layout with the owner row as the lane's column, which is exactly the B-operand layout of the
+// products that contract over y — so P and dS go from registers straight into the next matrix
+// instruction, and the only transposed operands (rows = head channel, k = y) are the ones read
+// from the transposed copies of launch 1.
+#include "sage_internal.h"
+
+namespace sage {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---- LDS layouts -------------------------------------------------------------------------
+// Transposed tile [D rows][64 slots] bf16: 128-byte rows, 8 chunks of 16 bytes per row; chunk
+// position XORed with bits of the pair-of-rows index (same layout as the forward's V^T tile).
+__device__ __forceinline__ int tr_off(int L) { return (((L >> 3) << 3) | ((L & 7) ^ ((L >> 4) & 7))) << 4; }
+// Natural tile [64 rows][D] bf16: CPR chunks per row.  16 consecutive rows reading one logical
+// chunk must land in 16 different 16-byte bank groups.
+template <int CPR> __device__ __forceinline__ int nat_pos(int row, int c) {
+    if constexpr (CPR == 16) return c ^ (row & 15);
+    else return c ^ ((row >> 1) & 7);
+}
+template <int CPR> __device__ __forceinline__ int nat_off(int row, int c) { return (row * CPR + nat_pos<CPR>(row, c)) << 4; }
+
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+// 16 (4) bytes per lane from global memory straight into LDS: lane l lands at base + 16*l (4*l).
+__device__ __forceinline__ void dma16(const void* gbase_uniform, uint32_t goff, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_base_uniform), "v"(goff), "s"(gbase_uniform)
+                 : "memory");
+}
+__device__ __forceinline__ void dma4(const void* gbase_uniform, uint32_t goff, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :
+                 : "s"(lds_base_uniform), "v"(goff), "s"(gbase_uniform)
+                 : "memory");
+}
+__device__ __forceinline__ void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    const v2f f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, v2bf));       // round to nearest even
+}
+
+// inverse of v_slot_f16: which row of a 64-row tile sits at slot s
+__device__ __forceinline__ int row_of_slot(int s) {
+    const int g = s >> 4, r = s & 15;
+    const int quad = (((r >> 2) & 1) << 1) | (r >> 3);
+    return (g << 4) | (quad << 2) | (r & 3);
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// Launch 1.  Roles of one grid, per (b,h): K^T tiles | Q^T tiles | dO^T tiles | row statistics.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
+    constexpr int CPR = D / 8;
+    constexpr int LROW = D + 8;                     // LDS row stride in elements (keeps 16-byte alignment, spreads banks)
+    __shared__ __attribute__((aligned(16))) uint16_t tile[64 * LROW];
+    const int ntk = (int)(a.nkv_pad / 64), ntq = (int)(a.nq_pad / 64);
+    const int per_bh = ntk + 3 * ntq;
+    const int bh = blockIdx.x / per_bh;
+    int r = blockIdx.x % per_bh;
+    const int b = bh / a.H, h = bh % a.H;
+    const int tid = threadIdx.x;
+
+    if (r >= ntk + 2 * ntq) {
+        // row statistics of 64 query rows: 4 threads per row
+        const int row = (r - ntk - 2 * ntq) * 64 + (tid >> 2);
+        const int part = tid & 3;
+        float sum = 0.0f;
+        if (row < a.valid_q) {
+            const uint16_t* po = a.o.p + b * a.o.sb + h * a.o.sh + (int64_t)row * a.o.sn + part * (D / 4);
+            const uint16_t* pg = a.dout.p + b * a.dout.sb + h * a.dout.sh + (int64_t)row * a.dout.sn + part * (D / 4);
+#pragma unroll
+            for (int c = 0; c < D / 32; c++) {
+                const u32x4 wo = *reinterpret_cast<const u32x4*>(po + c * 8);
+                const u32x4 wg = *reinterpret_cast<const u32x4*>(pg + c * 8);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    sum = fmaf(__uint_as_float(wo[e] << 16), __uint_as_float(wg[e] << 16), sum);
+                    sum = fmaf(__uint_as_float(wo[e] & 0xFFFF0000u), __uint_as_float(wg[e] & 0xFFFF0000u), sum);
+                }
+            }
+        }
+        sum += __shfl_xor(sum, 1);
+        sum += __shfl_xor(sum, 2);
+        if (part == 0) {
+            const int64_t idx = (int64_t)bh * a.nq_pad + row;
+            const bool valid = row < a.valid_q;
+            a.delta[idx] = valid ? sum : 0.0f;
+            a.lse2[idx] = valid ? a.stats[(int64_t)bh * a.Nq + row] * kLog2e : INFINITY;
+        }
+        return;
+    }
+
+    // transposed copy of one 64-row tile
+    View src;
+    uint16_t* dst;
+    int valid, t;
+    int64_t ntiles;
+    if (r < ntk) { src = a.k; dst = a.kT; valid = a.valid_kv; t = r; ntiles = ntk; }
+    else if (r < ntk + ntq) { src = a.q; dst = a.qT; valid = a.valid_q; t = r - ntk; ntiles = ntq; }
+    else { src = a.dout; dst = a.doT; valid = a.valid_q; t = r - ntk - ntq; ntiles = ntq; }
+    const uint16_t* sp = src.p + b * src.sb + h * src.sh;
+#pragma unroll
+    for (int i = 0; i < 64 * CPR / 256; i++) {
+        const int c = i * 256 + tid;
+        const int row = c / CPR, col = (c % CPR) * 8;
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (t * 64 + row < valid) w = *reinterpret_cast<const u32x4*>(sp + (int64_t)(t * 64 + row) * src.sn + col);
+        *reinterpret_cast<u32x4*>(&tile[row * LROW + col]) = w;
+    }
+    __syncthreads();
+    uint16_t* out = dst + ((int64_t)bh * ntiles + t) * (int64_t)(D * 64);
+#pragma unroll
+    for (int i = 0; i < D * 8 / 256; i++) {
+        const int c = i * 256 + tid;
+        const int d = c >> 3, s0 = (c & 7) * 8;
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t lo = tile[row_of_slot(s0 + 2 * e) * LROW + d];
+            const uint32_t hi = tile[row_of_slot(s0 + 2 * e + 1) * LROW + d];
+            w[e] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(out + d * 64 + s0) = u32x4{w[0], w[1], w[2], w[3]};
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Launches 2 and 3.
+// ---------------------------------------------------------------------------------------------
+template <int D, int PASS>
+__global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
+    constexpr int CPR = D / 8;                      // 16-byte chunks per natural row
+    constexpr int TILE_BYTES = 64 * D * 2;          // natural and transposed tiles have the same size
+    constexpr int RUNS = TILE_BYTES / 1024;         // 1 KiB copies per tile
+    constexpr int RPW = RUNS / 4;                   // per wave
+    constexpr int KS = D / 16;                      // matrix-instruction steps over the head dim
+    constexpr int DB = D / 32;                      // 32-channel output blocks
+    constexpr int NTR = PASS == 0 ? 1 : 2;          // transposed operands per tile
+    static_assert(RUNS % 4 == 0, "tile copies must divide over four waves");
+
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_nat[2][2][TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_tr[2][NTR][TILE_BYTES];
+    __shared__ __attribute__((aligned(256))) float lds_row[2][2][64];
+
+    const int Nx = PASS == 0 ? a.Nq : a.Nkv;
+    const int valid_x = PASS == 0 ? a.valid_q : a.valid_kv;
+    const int Ny = PASS == 0 ? a.Nkv : a.Nq;
+    const int valid_y = PASS == 0 ? a.valid_kv : a.valid_q;
+    const int x_tiles = (Nx + 127) / 128;
+    const int xt = blockIdx.x % x_tiles;
+    const int bh = blockIdx.x / x_tiles;
+    const int b = bh / a.H, h = bh % a.H;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const int x = xt * 128 + wave * 32 + l32;
+    const int xc = min(x, Nx - 1);
+
+    // owner side: two resident row blocks (B operands: column = owner row, k = head channel)
+    const View& xv1 = PASS == 0 ? a.q : a.k;
+    const View& xv2 = PASS == 0 ? a.dout : a.v;
+    v4i b1[KS], b2[KS];
+    {
+        const uint16_t* p1 = xv1.p + b * xv1.sb + h * xv1.sh + (int64_t)xc * xv1.sn + half * 8;
+        const uint16_t* p2 = xv2.p + b * xv2.sb + h * xv2.sh + (int64_t)xc * xv2.sn + half * 8;
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            b1[s] = *reinterpret_cast<const v4i*>(p1 + s * 16);
+            b2[s] = *reinterpret_cast<const v4i*>(p2 + s * 16);
+        }
+    }
+    float lse_x = 0.0f, delta_x = 0.0f;
+    if constexpr (PASS == 0) {
+        const int64_t idx = (int64_t)bh * a.nq_pad + min((int64_t)x, a.nq_pad - 1);
+        lse_x = a.lse2[idx];
+        delta_x = a.delta[idx];
+    }
+    // the plain loads above must not be in flight when the copy counter is used below
+    dma_wait_all();
+
+    // y side
+    const View& yv1 = PASS == 0 ? a.k : a.q;
+    const View& yv2 = PASS == 0 ? a.v : a.dout;
+    const uint8_t* y1 = reinterpret_cast<const uint8_t*>(yv1.p + b * yv1.sb + h * yv1.sh);
+    const uint8_t* y2 = reinterpret_cast<const uint8_t*>(yv2.p + b * yv2.sb + h * yv2.sh);
+    const int64_t ny_pad = PASS == 0 ? a.nkv_pad : a.nq_pad;
+    const uint8_t* t1 = reinterpret_cast<const uint8_t*>(PASS == 0 ? a.kT : a.qT) + (int64_t)bh * ny_pad * D * 2;
+    const uint8_t* t2 = reinterpret_cast<const uint8_t*>(a.doT) + (int64_t)bh * ny_pad * D * 2;
+    const uint8_t* rows_l = reinterpret_cast<const uint8_t*>(a.lse2 + (int64_t)bh * a.nq_pad);
+    const uint8_t* rows_d = reinterpret_cast<const uint8_t*>(a.delta + (int64_t)bh * a.nq_pad);
+    // owners that are all padding have nothing to compute: they only store zeros
+    const int ntiles = xt * 128 < valid_x ? (valid_y + 63) / 64 : 0;
+
+    // per-lane pieces of the copy addresses: run i of this wave covers physical chunks
+    // (i*4 + wave)*64 + lane of a tile
+    int nat_row[RPW], nat_col[RPW];
+    uint32_t tr_src[RPW];
+#pragma unroll
+    for (int i = 0; i < RPW; i++) {
+        const int P = (i * 4 + wave) * 64 + lane;
+        const int row = P / CPR, pos = P % CPR;
+        nat_row[i] = row;
+        nat_col[i] = nat_pos<CPR>(row, pos) * 16;          // the XOR is its own inverse
+        tr_src[i] = (uint32_t)tr_off(P);
+    }
+    const uint32_t nat_base = lds_addr(&lds_nat[0][0][0]), tr_base = lds_addr(&lds_tr[0][0][0]);
+    const uint32_t row_base = lds_addr(&lds_row[0][0][0]);
+    const uint32_t ys1 = (uint32_t)(yv1.sn * 2), ys2 = (uint32_t)(yv2.sn * 2);
+    auto copy_tile = [&](int t, int stage) {
+#pragma unroll
+        for (int i = 0; i < RPW; i++) {
+            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], Ny - 1);
+            const uint32_t dst = (uint32_t)((i * 4 + wave) * 1024);
+            dma16(y1, row * ys1 + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 0) * TILE_BYTES + dst));
+            dma16(y2, row * ys2 + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 1) * TILE_BYTES + dst));
+            dma16(t1 + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * NTR + 0) * TILE_BYTES + dst));
+            if constexpr (PASS == 1)
+                dma16(t2 + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * NTR + 1) * TILE_BYTES + dst));
+        }
+        if constexpr (PASS == 1) {
+            if (wave == 0) dma4(rows_l + (int64_t)t * 256, lane * 4, __builtin_amdgcn_readfirstlane(row_base + (stage * 2 + 0) * 256));
+            if (wave == 1) dma4(rows_d + (int64_t)t * 256, lane * 4, __builtin_amdgcn_readfirstlane(row_base + (stage * 2 + 1) * 256));
+        }
+    };
+
+    // fragment offsets inside a tile
+    int nat_frag[2][KS];                 // [32-row block][k-step]
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int s = 0; s < KS; s++) nat_frag[blk][s] = nat_off<CPR>(blk * 32 + l32, s * 2 + half);
+    int tr_frag[4];                      // [k-step over the 64 slots]; 32-channel blocks are +32*128 bytes
+#pragma unroll
+    for (int j = 0; j < 4; j++) tr_frag[j] = tr_off(l32 * 8 + j * 2 + half);
+
+    v16f acc1[DB], acc2[PASS == 1 ? DB : 1];
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            acc1[d][i] = 0.0f;
+            if constexpr (PASS == 1) acc2[d][i] = 0.0f;
+        }
+    const float c = a.scale * kLog2e;
+
+    if (ntiles > 0) copy_tile(0, 0);
+    for (int t = 0; t < ntiles; t++) {
+        const int stage = t & 1;
+        dma_wait_all();
+        __syncthreads();                 // tile t is visible; every wave is done with the other stage
+        if (t + 1 < ntiles) copy_tile(t + 1, stage ^ 1);
+        const uint8_t* n1 = &lds_nat[stage][0][0];
+        const uint8_t* n2 = &lds_nat[stage][1][0];
+        const uint8_t* r1 = &lds_tr[stage][0][0];
+        const uint8_t* r2 = &lds_tr[stage][NTR - 1][0];
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {
+            v16f tacc, gacc;
+#pragma unroll
+            for (int i = 0; i < 16; i++) tacc[i] = 0.0f, gacc[i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const v4i f1 = *reinterpret_cast<const v4i*>(n1 + nat_frag[blk][s]);
+                tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f1), __builtin_bit_cast(v8bf, b1[s]), tacc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const v4i f2 = *reinterpret_cast<const v4i*>(n2 + nat_frag[blk][s]);
+                gacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f2), __builtin_bit_cast(v8bf, b2[s]), gacc, 0, 0, 0);
+            }
+            // element i of a lane: y row (i>>2)*8 + half*4 + (i&3) of the block, column = owner row
+            uint32_t pp[8], sp[8];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float lse[4], dl[4];
+                if constexpr (PASS == 0) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) lse[e] = lse_x, dl[e] = delta_x;
+                } else {
+                    const v4f vl = *reinterpret_cast<const v4f*>(&lds_row[stage][0][blk * 32 + g * 8 + half * 4]);
+                    const v4f vd = *reinterpret_cast<const v4f*>(&lds_row[stage][1][blk * 32 + g * 8 + half * 4]);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) lse[e] = vl[e], dl[e] = vd[e];
+                }
+                float p[4], ds[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float arg = fmaf(tacc[g * 4 + e], c, -lse[e]);
+                    if constexpr (PASS == 0) {
+                        // keys past the valid length (only possible in the last tile)
+                        if (t * 64 + blk * 32 + g * 8 + half * 4 + e >= valid_y) arg = -INFINITY;
+                    }
+                    p[e] = __builtin_amdgcn_exp2f(arg);
+                    ds[e] = p[e] * (gacc[g * 4 + e] - dl[e]);
+                }
+                sp[g * 2] = pack_bf16(ds[0], ds[1]);
+                sp[g * 2 + 1] = pack_bf16(ds[2], ds[3]);
+                if constexpr (PASS == 1) {
+                    pp[g * 2] = pack_bf16(p[0], p[1]);
+                    pp[g * 2 + 1] = pack_bf16(p[2], p[3]);
+                }
+            }
+#pragma unroll
+            for (int j2 = 0; j2 < 2; j2++) {
+                const int j = blk * 2 + j2;
+                const v4i sb = {(int)sp[j2 * 4], (int)sp[j2 * 4 + 1], (int)sp[j2 * 4 + 2], (int)sp[j2 * 4 + 3]};
+#pragma unroll
+                for (int d = 0; d < DB; d++) {
+                    const v4i fa = *reinterpret_cast<const v4i*>(r1 + tr_frag[j] + d * 32 * 128);
+                    acc1[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, sb), acc1[d], 0, 0, 0);
+                }
+                if constexpr (PASS == 1) {
+                    const v4i pb = {(int)pp[j2 * 4], (int)pp[j2 * 4 + 1], (int)pp[j2 * 4 + 2], (int)pp[j2 * 4 + 3]};
+#pragma unroll
+                    for (int d = 0; d < DB; d++) {
+                        const v4i fa = *reinterpret_cast<const v4i*>(r2 + tr_frag[j] + d * 32 * 128);
+                        acc2[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, pb), acc2[d], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- epilogue: rows of valid owners get their gradient, padding rows zeros -----------------
+    if (x < Nx) {
+        const bool live = x < valid_x;
+        uint16_t* o1 = (PASS == 0 ? a.dq : a.dk) + b * (PASS == 0 ? a.dq_sb : a.dk_sb) + h * (PASS == 0 ? a.dq_sh : a.dk_sh) +
+                       (int64_t)x * (PASS == 0 ? a.dq_sn : a.dk_sn);
+        uint16_t* o2 = PASS == 1 ? a.dv + b * a.dv_sb + h * a.dv_sh + (int64_t)x * a.dv_sn : nullptr;
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int ch = d * 32 + g * 8 + half * 4;
+                u32x2 w = {0u, 0u};
+                if (live) {
+                    w.x = pack_bf16(acc1[d][g * 4] * a.scale, acc1[d][g * 4 + 1] * a.scale);
+                    w.y = pack_bf16(acc1[d][g * 4 + 2] * a.scale, acc1[d][g * 4 + 3] * a.scale);
+                }
+                *reinterpret_cast<u32x2*>(o1 + ch) = w;
+                if constexpr (PASS == 1) {
+                    u32x2 u = {0u, 0u};
+                    if (live) {
+                        u.x = pack_bf16(acc2[d][g * 4], acc2[d][g * 4 + 1]);
+                        u.y = pack_bf16(acc2[d][g * 4 + 2], acc2[d][g * 4 + 3]);
+                    }
+                    *reinterpret_cast<u32x2*>(o2 + ch) = u;
+                }
+            }
+    }
+}
+
+template <int D>
+static hipError_t launch_bwd_d(const BwdArgs& a, hipStream_t st) {
+    const int64_t bh = (int64_t)a.B * a.H;
+    const int64_t prep = bh * (a.nkv_pad / 64 + 3 * (a.nq_pad / 64));
+    const int64_t gq = bh * ((a.Nq + 127) / 128), gk = bh * ((a.Nkv + 127) / 128);
+    if (prep > 0x7FFFFFFF || gq > 0x7FFFFFFF || gk > 0x7FFFFFFF) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((bwd_prep_kernel<D>), dim3((unsigned)prep), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((bwd_pass_kernel<D, 0>), dim3((unsigned)gq), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((bwd_pass_kernel<D, 1>), dim3((unsigned)gk), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_bwd(const BwdArgs& a, hipStream_t st) {
+    if (a.D == 128) return launch_bwd_d<128>(a, st);
+    if (a.D == 64) return launch_bwd_d<64>(a, st);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace sage

@@ -105,6 +105,23 @@ struct AttnArgs {
 };
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st);
 
+// ---- backward (sage_bwd.hip) -------------------------------------------------
+// bf16 flash backward: Q, K, V, O, dO and the forward's log-sum-exp in, dQ, dK, dV out.
+struct BwdArgs {
+    View q, k, v, o, dout;
+    const float* stats;                          // [B,H,Nq] contiguous, natural log
+    uint16_t *dq, *dk, *dv;
+    int64_t dq_sb, dq_sh, dq_sn, dk_sb, dk_sh, dk_sn, dv_sb, dv_sh, dv_sn;
+    int B, H, Nq, Nkv, D;
+    int valid_q, valid_kv;                       // rows / keys past these are padding
+    float scale;
+    // workspace
+    uint16_t *kT, *qT, *doT;                     // [B,H,n_pad/64,D,64] bf16, rows in v_slot_f16 order, zero past valid
+    float *lse2, *delta;                         // [B,H,nq_pad]: Stats*log2(e) (+inf past valid), rowsum(dO*O)
+    int64_t nq_pad, nkv_pad;                     // multiples of 64
+};
+hipError_t launch_bwd(const BwdArgs& a, hipStream_t st);
+
 // Key k of a 64-key tile is stored at this slot of the V tile (host + device).
 __host__ __device__ inline int v_slot_f16(int k) {
     // 16-key groups; inside a group the quads of 4 keys are ordered 0,2,1,3 so that

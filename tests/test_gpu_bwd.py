@@ -1,0 +1,207 @@
+"""GPU parity of the bf16 backward (mi355_sage_sdpa_bwd_bf16) through the C ABI.
+
+The checker is the CPU oracle's flash form in double precision, fed the same bf16 inputs, the same
+bf16 O and the same fp32 log-sum-exp.  What the kernels add on top of exact arithmetic: P and dS are
+rounded to bf16 (relative 2^-9 per element, independent from element to element, so they average
+out over the contraction) and the results are rounded to bf16 (relative 2^-9 of each element).  Bars:
+max-abs error <= 1e-2 of the largest reference magnitude of that gradient, cosine >= 0.9999; against
+the reference's own gates (cos >= 0.999 flash-vs-math, serenitymojo/ops/tests/sdpa_flash_parity.mojo:177;
+cos >= 0.99 for its bf16 run against torch, ops/parity/sdpa_bwd_parity.mojo:181) these are tighter."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from mojodiffusion_amd import _lib, attention_sage
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _bf16_round(x):
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch.bfloat16)
+
+
+def _cos(a, b):
+    a, b = a.reshape(-1).astype(np.float64), b.reshape(-1).astype(np.float64)
+    return float(a @ b / (np.linalg.norm(a) * np.linalg.norm(b) + 1e-300))
+
+
+def _check(name, got, want, abs_frac=1e-2, cos_bar=0.9999):
+    got = got.float().cpu().numpy()
+    scale = np.abs(want).max()
+    if scale == 0:          # e.g. a single key: the softmax is constant and no gradient reaches q or k
+        assert np.abs(got).max() <= 1e-3, name
+        return
+    err = np.abs(got - want).max()
+    assert err <= abs_frac * scale, "%s: max-abs %.3e > %.1e * %.3e" % (name, err, abs_frac, scale)
+    assert _cos(got, want) >= cos_bar, "%s: cosine %.6f" % (name, _cos(got, want))
+
+
+def _run_case(oracle, B, Sq, Skv, H, D, scale, seed, real_q=0, real_kv=0, spread=1.0):
+    rng = np.random.default_rng(seed)
+    q, k, v, g = (_bf16_round(rng.standard_normal(s) * spread) for s in
+                  ((B, Sq, H, D), (B, Skv, H, D), (B, Skv, H, D), (B, Sq, H, D)))
+    qf, kf, vf, gf = (t.float().numpy() for t in (q, k, v, g))
+    nk = real_kv if 0 < real_kv < Skv else Skv
+    o32, stats = oracle.sdpa_f32(qf, kf, vf, scale, mask_lo=nk, mask_hi=Skv, want_stats=True)
+    o = _bf16_round(o32)
+    want = oracle.sdpa_bwd_f32(qf, kf, vf, gf, scale, o=o.float().numpy(), stats=stats, real_nq=real_q, real_nkv=real_kv)
+    L = _lib.lib()
+    dev = [t.cuda() for t in (q, k, v, o, g)]
+    st = torch.from_numpy(stats).cuda()
+    outs = [torch.full_like(dev[0], 7.0), torch.full_like(dev[1], 7.0), torch.full_like(dev[2], 7.0)]
+    ws = torch.empty(L.mi355_sage_bwd_workspace_bytes(B, H, Sq, Skv, D), dtype=torch.uint8, device="cuda")
+    qs, ks = _lib.strides_bhnd(Sq, H, D), _lib.strides_bhnd(Skv, H, D)
+    rc = L.mi355_sage_sdpa_bwd_bf16(*(t.data_ptr() for t in dev), st.data_ptr(), *(t.data_ptr() for t in outs),
+                                    B, H, Sq, Skv, D, scale, qs, ks, ks, qs, qs, qs, ks, ks,
+                                    0, 0, 0, 0, 0, 0, 0, 0, 0, 0, real_q, real_kv,
+                                    torch.cuda.current_stream().cuda_stream, ws.data_ptr(), ws.numel())
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    return outs, want
+
+
+@pytest.mark.parametrize("shape", [
+    (1, 128, 128, 2, 128), (2, 200, 200, 3, 128), (1, 64, 77, 5, 64), (1, 96, 16, 4, 128), (1, 333, 257, 2, 64),
+    (1, 8, 8, 4, 128), (1, 1, 300, 2, 128), (1, 300, 1, 2, 64),
+])
+def test_bwd_matches_the_oracle(oracle, shape):
+    B, Sq, Skv, H, D = shape
+    outs, want = _run_case(oracle, B, Sq, Skv, H, D, float(1.0 / np.sqrt(D)), seed=100 + Sq)
+    for name, got, ref in zip(("dQ", "dK", "dV"), outs, want):
+        _check("%s %s" % (name, shape), got, ref)
+
+
+def test_bwd_peaked_attention(oracle):
+    """Inputs three times wider: rows dominated by a few keys, scores up to ~+-40."""
+    outs, want = _run_case(oracle, 1, 256, 256, 2, 128, float(1.0 / np.sqrt(128)), seed=7, spread=3.0)
+    for name, got, ref in zip(("dQ", "dK", "dV"), outs, want):
+        _check(name, got, ref)
+
+
+def test_bwd_valid_lengths(oracle):
+    """real_N_q / real_N_kv (cudnn_sdpa_bwd.cpp:344): padding takes no part and gets zero rows."""
+    B, Sq, Skv, H, D = 1, 256, 256, 2, 128
+    rq, rk = 201, 167
+    outs, want = _run_case(oracle, B, Sq, Skv, H, D, 0.09, seed=9, real_q=rq, real_kv=rk)
+    for name, got, ref in zip(("dQ", "dK", "dV"), outs, want):
+        _check(name, got, ref)
+    assert not outs[0][:, rq:].float().abs().max().item()
+    assert not outs[1][:, rk:].float().abs().max().item() and not outs[2][:, rk:].float().abs().max().item()
+
+
+def test_bwd_golden_shapes(oracle):
+    """The shapes and closed-form inputs of ops/parity/sdpa_bwd_parity.mojo:44-65 with its golden
+    gradients (ops/parity/sdpa_bwd_ref.txt).  The kernel sees the inputs rounded to bf16, which by
+    itself moves the gradients by a few 1e-3 relative; the bar is the cosine gate of that test's
+    bf16 run (:181, 0.99) tightened to 0.999."""
+    ref = np.load(os.path.join(GOLD, "sdpa_bwd_ref.npz"))
+    for tag, (B, S, H, D) in (("dh128", (1, 8, 32, 128)), ("dh64", (1, 8, 8, 64))):
+        i = np.arange(B * S * H * D, dtype=np.int64)
+        shp = (B, S, H, D)
+        q = _bf16_round(((((i * 7) % 13) - 6.0) * 0.05).reshape(shp))
+        k = _bf16_round(((((i * 5) % 11) - 5.0) * 0.05).reshape(shp))
+        v = _bf16_round(((((i * 3) % 9) - 4.0) * 0.05).reshape(shp))
+        g = _bf16_round(((((i * 2) % 7) - 3.0) * 0.05).reshape(shp))
+        scale = float(1.0 / np.sqrt(D))
+        o32, stats = oracle.sdpa_f32(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale, want_stats=True)
+        fwd = attention_sage.SdpaFlashFwd(None, _bf16_round(o32).cuda(), q.cuda(), k.cuda(), v.cuda(),
+                                          torch.from_numpy(stats).cuda().reshape(B, H, S, 1))
+        grads = attention_sage.sdpa_flash_backward(fwd, g.cuda(), scale)
+        torch.cuda.synchronize()
+        for name, got in (("dq", grads.d_q), ("dk", grads.d_k), ("dv", grads.d_v)):
+            want = ref[tag + "_" + name].reshape(shp)
+            assert _cos(got.float().cpu().numpy(), want) >= 0.999, (tag, name)
+
+
+def test_bwd_bhsd_memory_and_offsets(oracle):
+    """Every tensor in BHSD memory at a non-zero element offset, Stats at an offset too."""
+    B, S, H, D = 2, 160, 3, 64
+    scale = 0.125
+    rng = np.random.default_rng(21)
+    q, k, v, g = (_bf16_round(rng.standard_normal((B, S, H, D))) for _ in range(4))
+    qf, kf, vf, gf = (t.float().numpy() for t in (q, k, v, g))
+    o32, stats = oracle.sdpa_f32(qf, kf, vf, scale, want_stats=True)
+    o = _bf16_round(o32)
+    want = oracle.sdpa_bwd_f32(qf, kf, vf, gf, scale, o=o.float().numpy(), stats=stats)
+    off = 64
+    def bhsd(t):
+        buf = torch.zeros(off + B * H * S * D, dtype=torch.bfloat16, device="cuda")
+        buf[off:].view(B, H, S, D).copy_(t.cuda().permute(0, 2, 1, 3))
+        return buf
+    bufs = [bhsd(t) for t in (q, k, v, o, g)]
+    outs = [torch.full((off + B * H * S * D,), 7.0, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+    st = torch.zeros(5 + B * H * S, dtype=torch.float32, device="cuda")
+    st[5:] = torch.from_numpy(stats).cuda().reshape(-1)
+    strides = (_lib.ctypes.c_int64 * 4)(H * S * D, S * D, D, 1)
+    L = _lib.lib()
+    rc = L.mi355_sage_sdpa_bwd_bf16(*(t.data_ptr() for t in bufs), st.data_ptr(), *(t.data_ptr() for t in outs),
+                                    B, H, S, S, D, scale, *([strides] * 8), off, off, off, off, off, 5, off, off, off,
+                                    0, 0, 0, torch.cuda.current_stream().cuda_stream, None, 0)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    for name, got, ref in zip(("dQ", "dK", "dV"), outs, want):
+        assert (got[:off].float() == 7.0).all()          # nothing written in front of the offset
+        _check(name, got[off:].view(B, H, S, D).permute(0, 2, 1, 3), ref)
+
+
+def test_bwd_after_the_quantized_forward():
+    """Trainer shape (ops/tests/sdpa_flash_parity.mojo: zimage [1,1248,30,128]): forward by the
+    quantized kernel (its O and Stats), backward by the bf16 kernels, against torch's fp32 autograd
+    on the same bf16 inputs.  Gate of that test: cosine >= 0.999 per gradient."""
+    B, S, H, D = 1, 1248, 30, 128
+    scale = float(1.0 / np.sqrt(D))
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v, g = (torch.randn((B, S, H, D), device="cuda", generator=gen).to(torch.bfloat16) for _ in range(4))
+    fwd = attention_sage.sdpa_flash_train_fwd(q, k, v, scale)
+    grads = attention_sage.sdpa_flash_backward(fwd, g, scale)
+    Q, K, V = (t.float().permute(0, 2, 1, 3).detach().requires_grad_(True) for t in (q, k, v))
+    p = torch.softmax(scale * Q @ K.transpose(-1, -2), dim=-1)
+    (p @ V).backward(g.float().permute(0, 2, 1, 3))
+    for name, got, ref in (("dQ", grads.d_q, Q.grad), ("dK", grads.d_k, K.grad), ("dV", grads.d_v, V.grad)):
+        a = got.float().permute(0, 2, 1, 3).reshape(-1).double()
+        b = ref.reshape(-1).double()
+        cos = float(a @ b / (a.norm() * b.norm()))
+        assert cos >= 0.999, (name, cos)
+    # F32 boundary (attention_flash.mojo:478-535) on an aligned length
+    S2 = 1280
+    q2, k2, v2 = (torch.randn((B, S2, H, D), device="cuda", generator=gen) for _ in range(3))
+    att, f2 = attention_sage.sdpa_flash_train_fwd_f32(q2, k2, v2, scale)
+    g2 = attention_sage.sdpa_flash_backward_f32(f2.q_pad, f2.k_pad, f2.v_pad, f2.o_pad, f2.stats, torch.ones_like(att), scale)
+    assert g2.d_q.dtype == torch.float32 and g2.d_v.shape == v2.shape
+    # probabilities of a row sum to one: with dO = 1 every dV row sums (over keys) to S2 per channel
+    colsum = g2.d_v.sum(dim=1)
+    assert torch.allclose(colsum, torch.full_like(colsum, float(S2)), rtol=2e-2)
+
+
+def test_bwd_argument_errors():
+    L = _lib.lib()
+    B, S, H, D = 1, 64, 1, 64
+    t = [torch.zeros((B, S, H, D), dtype=torch.bfloat16, device="cuda") for _ in range(8)]
+    st = torch.zeros((B, H, S), dtype=torch.float32, device="cuda")
+    s4 = _lib.strides_bhnd(S, H, D)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(ptrs=None, causal=0, d=D, ws=(None, 0), strides=None):
+        p = [x.data_ptr() for x in t] if ptrs is None else ptrs
+        ss = [s4] * 8 if strides is None else strides
+        return L.mi355_sage_sdpa_bwd_bf16(p[0], p[1], p[2], p[3], p[4], st.data_ptr(), p[5], p[6], p[7],
+                                          B, H, S, S, d, 0.125, *ss, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+                                          causal, 0, 0, stream, ws[0], ws[1])
+    assert call() == 0
+    ptrs = [x.data_ptr() for x in t]
+    assert call(ptrs=ptrs[:5] + [None] + ptrs[6:]) == -1               # dQ missing
+    assert call(strides=[s4] * 7 + [None]) == -1
+    assert call(causal=1) == -2
+    assert call(d=96) == -2
+    small = torch.empty(256, dtype=torch.uint8, device="cuda")
+    assert call(ws=(small.data_ptr(), small.numel())) == -3
+    assert L.mi355_sage_bwd_workspace_bytes(B, H, S, S, 96) == 0
+    with pytest.raises(attention_sage.Error, match="d_out must be BF16"):
+        attention_sage.sdpa_flash_backward_raw(t[0], t[1], t[2], t[3], st, t[4].float(), 0.125)
+    with pytest.raises(attention_sage.Error, match="S must be 128-aligned"):
+        attention_sage.sdpa_flash_backward_f32(t[0], t[1], t[2], t[3], st, t[4].float(), 0.125)
+    torch.cuda.synchronize()
