@@ -1,0 +1,330 @@
+// attn_loop_structure.hip — what the attention kernel's main loop costs in shader clocks, piece by
+// piece.  Measurement tool, not part of the library.
+//
+// Every kernel here runs the loop's instruction mix on synthetic data (per wave and 64-key tile:
+// 8 INT8 + 16 FP16 matrix instructions, 32 fma + 32 exp + 16 cvt_pk + 16 dot2, the loop's real
+// dependencies between them) for 72 tiles and reports shader clocks per tile PER WAVE — the two
+// waves that share a SIMD do not progress at the same rate, and a workgroup barrier makes the
+// faster one wait.  Variants:
+//
+//   loop<8 waves>  features added one at a time: LDS fragment reads, tile copies
+//                  (global_load_lds), the workgroup barrier of every tile
+//   loop<4 waves>  the same loop as 128-row workgroups, one or two per CU; and with 64 rows per
+//                  wave (every LDS fragment feeds two matrix instructions, one wave per SIMD)
+//   pingpong       waves 0-3 and 4-7 alternate between a matrix phase (24 matrix instructions back
+//                  to back) and a vector phase (the exponentials), half a tile apart, a barrier
+//                  between phases
+//
+// usage: attn_loop_structure
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <type_traits>
+#include <vector>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+
+#define CHECK(x)                                                                       \
+    do {                                                                               \
+        hipError_t e_ = (x);                                                           \
+        if (e_ != hipSuccess) {                                                        \
+            std::fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_));               \
+            return 1;                                                                  \
+        }                                                                              \
+    } while (0)
+
+__device__ __forceinline__ int swz(int L) { return (((L >> 3) << 3) | ((L & 7) ^ ((L >> 4) & 7))) << 4; }
+__device__ __forceinline__ void dma16(const void* g, uint32_t goff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(goff), "s"(g) : "memory");
+}
+template <int N> __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+constexpr int FRAG = 1, COPY = 2, BARRIER = 4;
+constexpr int TILES = 72, HEADS = 24;
+
+struct Stamp { unsigned long long clocks, at_barrier, t_begin, t_end; };
+
+__device__ __forceinline__ void init_operands(v4i (&qf)[4], v4i (&kf)[2][4], v4i (&vf)[16]) {
+    unsigned seed = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+    for (int r = 0; r < 4; r++)
+        for (int e = 0; e < 4; e++) {
+            seed = seed * 1664525u + 1013904223u;
+            qf[r][e] = (int)((seed >> 3) & 0x3B3F3B3Fu);
+        }
+    for (int a = 0; a < 2; a++)
+        for (int r = 0; r < 4; r++) kf[a][r] = qf[(r + a) & 3] ^ v4i{a, r, 1, 2};
+    for (int u = 0; u < 16; u++) vf[u] = qf[u & 3] ^ v4i{u, 1, u, 3};
+}
+
+// The loop as the attention kernel runs it: scores of tile t, then the exponentials of tile t
+// interleaved with P.V of tile t-1, copies and barrier at the midpoint.
+template <int NW, int LEAD, int FEAT, int RB = 1>
+__global__ __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) void loop_kernel(int tiles, const uint8_t* kg_all, const uint8_t* vg_all, float* out, Stamp* stamps) {
+    constexpr int NSK = LEAD + 1, NSV = LEAD + 2;
+    constexpr int KCH = 8 / NW, VCH = 16 / NW;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NSK][8192];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][16384];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const uint8_t* kg = kg_all + (size_t)(blockIdx.x % HEADS) * tiles * 8192;
+    const uint8_t* vg = vg_all + (size_t)(blockIdx.x % HEADS) * tiles * 16384;
+    for (int i = tid; i < NSK * 8192 / 4; i += NW * 64) ((unsigned*)lds_k)[i] = (i * 2654435761u >> 3) & 0x3B3F3B3Fu;
+    for (int i = tid; i < NSV * 16384 / 4; i += NW * 64) ((unsigned*)lds_v)[i] = (i * 2654435761u >> 3) & 0x3BFF3BFFu;
+    __syncthreads();
+    int koff[4], voff[4];
+    for (int s = 0; s < 4; s++) koff[s] = swz(l32 * 8 + s * 2 + half), voff[s] = swz(l32 * 8 + s * 2 + half);
+    int ksrc[KCH], vsrc[VCH];
+    uint32_t kdst[KCH], vdst[VCH];
+    for (int i = 0; i < KCH; i++) { ksrc[i] = swz((i * NW + wave) * 64 + lane); kdst[i] = lds_addr(&lds_k[0][0]) + (i * NW + wave) * 1024; }
+    for (int i = 0; i < VCH; i++) { vsrc[i] = swz((i * NW + wave) * 64 + lane); vdst[i] = lds_addr(&lds_v[0][0]) + (i * NW + wave) * 1024; }
+
+    v4i qf[4], kf[2][4], vf[16];
+    init_operands(qf, kf, vf);
+    v4i qf2[RB][4];
+    for (int r = 0; r < RB; r++)
+        for (int st = 0; st < 4; st++) qf2[r][st] = qf[st] ^ v4i{r, 0, r, 0};
+    v16f o[RB][4] = {};
+    float l[RB] = {}, f = 1e-9f, c = -0.25f;
+    unsigned p[RB][2][16] = {};
+    v16i s[RB][2] = {};
+    unsigned long long at_barrier = 0;
+    auto mid = [&](int t) {
+        if constexpr (FEAT & COPY) dma_wait<(LEAD - 1) * (KCH + VCH)>();
+        if constexpr (FEAT & BARRIER) {
+            const unsigned long long b0 = __builtin_readcyclecounter();
+            __builtin_amdgcn_s_barrier();
+            at_barrier += __builtin_readcyclecounter() - b0;
+        }
+        if constexpr (FEAT & COPY) {
+            const int tk = min(t + LEAD + 1, tiles - 1), tv = min(t + LEAD, tiles - 1);
+#pragma unroll
+            for (int i = 0; i < KCH; i++) dma16(kg + (size_t)tk * 8192, ksrc[i], __builtin_amdgcn_readfirstlane(kdst[i] + ((t + LEAD + 1) % NSK) * 8192));
+#pragma unroll
+            for (int i = 0; i < VCH; i++) dma16(vg + (size_t)tv * 16384, vsrc[i], __builtin_amdgcn_readfirstlane(vdst[i] + ((t + LEAD) % NSV) * 16384));
+        }
+    };
+    auto body = [&](int t, auto xtag) {
+        constexpr int X = decltype(xtag)::value;
+        const int slot_kn = (t + 1) % NSK, slot_v = (t + NSV - 1) % NSV;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int r = 0; r < RB; r++) s[r][kb] = v16i{};
+#pragma unroll
+            for (int st = 0; st < 4; st++)
+#pragma unroll
+                for (int r = 0; r < RB; r++) s[r][kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf2[r][st], s[r][kb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            if ((FEAT & FRAG) && u + 2 < 16) vf[u + 2] = *reinterpret_cast<const v4i*>(&lds_v[slot_v][voff[(u + 2) >> 2] + ((u + 2) & 3) * 32 * 128]);
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                {
+                    const v4i pw = {(int)p[r][X ^ 1][(u >> 2) * 4], (int)p[r][X ^ 1][(u >> 2) * 4 + 1], (int)p[r][X ^ 1][(u >> 2) * 4 + 2], (int)p[r][X ^ 1][(u >> 2) * 4 + 3]};
+                    o[r][u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vf[u]), __builtin_bit_cast(v8h, pw), o[r][u & 3], 0, 0, 0);
+                }
+                const int kb = u >> 3, i = (u & 7) * 2;
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[r][kb][i]), f, c));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[r][kb][i + 1]), f, c));
+                const v2h pr = {(_Float16)p0, (_Float16)p1};
+                const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+                l[r] = __builtin_amdgcn_fdot2(pr, ones, l[r], false);
+                p[r][X][u] = __builtin_bit_cast(unsigned, pr);
+            }
+            if (u == 7) {
+                mid(t);
+                if constexpr (FEAT & FRAG)
+#pragma unroll
+                    for (int st = 0; st < 4; st++) kf[0][st] = *reinterpret_cast<const v4i*>(&lds_k[slot_kn][koff[st]]);
+            }
+        }
+        if constexpr (FEAT & FRAG) {
+            vf[0] = *reinterpret_cast<const v4i*>(&lds_v[t % NSV][voff[0]]);
+            vf[1] = *reinterpret_cast<const v4i*>(&lds_v[t % NSV][voff[0] + 32 * 128]);
+#pragma unroll
+            for (int st = 0; st < 4; st++) kf[1][st] = *reinterpret_cast<const v4i*>(&lds_k[slot_kn][koff[st] + 32 * 128]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+    const unsigned long long t0 = __builtin_readcyclecounter();
+    for (int t = 0; t < tiles; t += 2) {
+        body(t, std::integral_constant<int, 0>{});
+        body(t + 1, std::integral_constant<int, 1>{});
+    }
+    const unsigned long long t1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = __builtin_amdgcn_s_memrealtime();
+    dma_wait<0>();
+    float chk = 0.0f;
+    for (int r = 0; r < RB; r++) chk += o[r][0][0] + o[r][1][0] + o[r][2][0] + o[r][3][0] + l[r];
+    if (chk == 1.2345f) out[threadIdx.x] = chk;
+    if (lane == 0) stamps[blockIdx.x * 8 + wave] = Stamp{t1 - t0, at_barrier, r0, r1};
+}
+
+// Ping-pong: while waves 0-3 are in their matrix phase, waves 4-7 (the other wave of each SIMD) are in
+// their vector phase, and the other way round; a workgroup barrier ends every phase.
+__global__ __launch_bounds__(512, 2) void pingpong_kernel(int tiles, const uint8_t* kg_all, const uint8_t* vg_all, float* out, Stamp* stamps) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_k[4][8192];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_v[5][16384];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const int grp = wave >> 2;
+    const uint8_t* kg = kg_all + (size_t)(blockIdx.x % HEADS) * tiles * 8192;
+    const uint8_t* vg = vg_all + (size_t)(blockIdx.x % HEADS) * tiles * 16384;
+    for (int i = tid; i < 4 * 8192 / 4; i += 512) ((unsigned*)lds_k)[i] = (i * 2654435761u >> 3) & 0x3B3F3B3Fu;
+    for (int i = tid; i < 5 * 16384 / 4; i += 512) ((unsigned*)lds_v)[i] = (i * 2654435761u >> 3) & 0x3BFF3BFFu;
+    __syncthreads();
+    int koff[4], voff[4];
+    for (int s = 0; s < 4; s++) koff[s] = swz(l32 * 8 + s * 2 + half), voff[s] = swz(l32 * 8 + s * 2 + half);
+    const int ksrc = swz(wave * 64 + lane), vsrc0 = swz(wave * 64 + lane), vsrc1 = swz((8 + wave) * 64 + lane);
+    const uint32_t kdst = lds_addr(&lds_k[0][0]) + wave * 1024, vdst0 = lds_addr(&lds_v[0][0]) + wave * 1024, vdst1 = vdst0 + 8192;
+    v4i qf[4], kf[2][4], vf[16];
+    init_operands(qf, kf, vf);
+    v16f o[4] = {};
+    float l = 0.0f, f = 1e-9f, c = -0.25f;
+    unsigned p[16] = {};
+    v16i s[2] = {};
+    unsigned long long at_barrier = 0;
+    auto barrier = [&]() {
+        const unsigned long long b0 = __builtin_readcyclecounter();
+        __builtin_amdgcn_s_barrier();
+        at_barrier += __builtin_readcyclecounter() - b0;
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto matrix_phase = [&](int t) {
+        const int slot_v = (t + 4) % 5;                 // V(t-1)
+        const int tt = min(t + 3, tiles - 1);
+        dma16(kg + (size_t)tt * 8192, ksrc, __builtin_amdgcn_readfirstlane(kdst + ((t + 3) & 3) * 8192));
+        dma16(vg + (size_t)tt * 16384, vsrc0, __builtin_amdgcn_readfirstlane(vdst0 + ((t + 3) % 5) * 16384));
+        dma16(vg + (size_t)tt * 16384, vsrc1, __builtin_amdgcn_readfirstlane(vdst1 + ((t + 3) % 5) * 16384));
+#pragma unroll
+        for (int st = 0; st < 4; st++) kf[1][st] = *reinterpret_cast<const v4i*>(&lds_k[t & 3][koff[st] + 32 * 128]);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            s[kb] = v16i{};
+#pragma unroll
+            for (int st = 0; st < 4; st++) {
+                s[kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], s[kb], 0, 0, 0);
+                const int u = kb * 4 + st + 2;
+                vf[u] = *reinterpret_cast<const v4i*>(&lds_v[slot_v][voff[u >> 2] + (u & 3) * 32 * 128]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            if (u + 10 < 16) vf[u + 10] = *reinterpret_cast<const v4i*>(&lds_v[slot_v][voff[(u + 10) >> 2] + ((u + 10) & 3) * 32 * 128]);
+            const v4i pw = {(int)p[(u >> 2) * 4], (int)p[(u >> 2) * 4 + 1], (int)p[(u >> 2) * 4 + 2], (int)p[(u >> 2) * 4 + 3]};
+            o[u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vf[u]), __builtin_bit_cast(v8h, pw), o[u & 3], 0, 0, 0);
+        }
+    };
+    auto vector_phase = [&](int t) {
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int kb = u >> 3, i = (u & 7) * 2;
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f, c));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f, c));
+            const v2h pr = {(_Float16)p0, (_Float16)p1};
+            const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+            l = __builtin_amdgcn_fdot2(pr, ones, l, false);
+            p[u] = __builtin_bit_cast(unsigned, pr);
+        }
+#pragma unroll
+        for (int st = 0; st < 4; st++) kf[0][st] = *reinterpret_cast<const v4i*>(&lds_k[(t + 1) & 3][koff[st]]);
+        vf[0] = *reinterpret_cast<const v4i*>(&lds_v[t % 5][voff[0]]);
+        vf[1] = *reinterpret_cast<const v4i*>(&lds_v[t % 5][voff[0] + 32 * 128]);
+        dma_wait<3>();
+    };
+    const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+    const unsigned long long t0 = __builtin_readcyclecounter();
+    if (grp == 1) barrier();
+    for (int t = 0; t < tiles; t++) {
+        matrix_phase(t);
+        barrier();
+        vector_phase(t);
+        barrier();
+    }
+    if (grp == 0) barrier();
+    const unsigned long long t1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = __builtin_amdgcn_s_memrealtime();
+    dma_wait<0>();
+    if (o[0][0] + o[1][0] + o[2][0] + o[3][0] + l == 1.2345f) out[threadIdx.x] = l;
+    if (lane == 0) stamps[blockIdx.x * 8 + wave] = Stamp{t1 - t0, at_barrier, r0, r1};
+}
+
+static float* d_out;
+static Stamp* d_stamps;
+static uint8_t *d_k, *d_v;
+
+static int report(const char* what, int nw, int wgs, int rb = 1) {
+    std::vector<Stamp> h((size_t)wgs * 8);
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipMemcpy(h.data(), d_stamps, h.size() * sizeof(Stamp), hipMemcpyDeviceToHost));
+    // waves w and w + 4 of a workgroup share a SIMD; with 4-wave workgroups the two that share a CU do
+    double lo[2] = {0, 0}, bar[2] = {0, 0}, life = 0, cyc = 0;
+    int cnt[2] = {0, 0};
+    unsigned long long rmin = ~0ull, rmax = 0;
+    std::vector<double> per_wg(wgs);
+    for (int g = 0; g < wgs; g++) {
+        double m = 0;
+        for (int w = 0; w < nw; w++) m = std::max(m, (double)h[(size_t)g * 8 + w].clocks);
+        per_wg[g] = m;
+    }
+    std::vector<double> sorted = per_wg;
+    std::sort(sorted.begin(), sorted.end());
+    const double median = sorted[sorted.size() / 2];
+    for (int g = 0; g < wgs; g++)
+        for (int w = 0; w < nw; w++) {
+            const Stamp& e = h[(size_t)g * 8 + w];
+            const int cls = nw == 8 ? (w >= 4) : (per_wg[g] > median);
+            lo[cls] += (double)e.clocks; bar[cls] += (double)e.at_barrier; cnt[cls]++;
+            cyc += (double)e.clocks; life += (double)(e.t_end - e.t_begin);
+            rmin = std::min(rmin, e.t_begin); rmax = std::max(rmax, e.t_end);
+        }
+    const double rows_tiles = (double)wgs * nw * 32 * rb * TILES;
+    std::printf("%-62s %4d x %d waves: clocks per tile %5.0f | %5.0f (of which at the barrier %4.0f | %4.0f), clock %4.0f MHz, "
+                "%6.4f rows*tiles per clock and CU\n", what, wgs, nw,
+                cnt[0] ? lo[0] / cnt[0] / TILES : 0.0, cnt[1] ? lo[1] / cnt[1] / TILES : 0.0,
+                cnt[0] ? bar[0] / cnt[0] / TILES : 0.0, cnt[1] ? bar[1] / cnt[1] / TILES : 0.0, cyc / life * 100.0,
+                rows_tiles / ((double)(rmax - rmin) / 100.0 * (cyc / life * 100.0)) / std::min(wgs, 256));
+    std::fflush(stdout);
+    return 0;
+}
+
+template <int NW, int LEAD, int FEAT, int RB = 1> static int run_loop(const char* what, int wgs) {
+    for (int rep = 0; rep < 4; rep++)
+        hipLaunchKernelGGL((loop_kernel<NW, LEAD, FEAT, RB>), dim3(wgs), dim3(NW * 64), 0, 0, TILES, d_k, d_v, d_out, d_stamps);
+    return report(what, NW, wgs, RB);
+}
+
+int main() {
+    CHECK(hipMalloc(&d_out, 4096));
+    CHECK(hipMalloc(&d_stamps, 1024 * 8 * sizeof(Stamp)));
+    CHECK(hipMalloc(&d_k, (size_t)HEADS * TILES * 8192));
+    CHECK(hipMalloc(&d_v, (size_t)HEADS * TILES * 16384));
+    std::vector<uint32_t> hk((size_t)HEADS * TILES * 8192 / 4), hv((size_t)HEADS * TILES * 16384 / 4);
+    uint32_t s = 1;
+    for (auto& x : hk) { s = s * 1664525u + 1013904223u; x = (s >> 3) & 0x3B3F3B3Fu; }
+    for (auto& x : hv) { s = s * 1664525u + 1013904223u; x = (s >> 3) & 0x3BFF3BFFu; }
+    CHECK(hipMemcpy(d_k, hk.data(), hk.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(d_v, hv.data(), hv.size() * 4, hipMemcpyHostToDevice));
+    std::printf("clocks per tile: waves 0-3 | waves 4-7 of a workgroup (they share SIMDs pairwise); for 4-wave workgroups: faster | slower half\n");
+    if (run_loop<8, 2, 0>("instruction mix only", 256)) return 1;
+    if (run_loop<8, 2, FRAG>("+ LDS fragment reads", 256)) return 1;
+    if (run_loop<8, 2, FRAG | COPY>("+ tile copies", 256)) return 1;
+    if (run_loop<8, 2, FRAG | COPY | BARRIER>("+ workgroup barrier per tile (the kernel's loop)", 256)) return 1;
+    if (run_loop<4, 1, FRAG | COPY | BARRIER>("128-row workgroups, one per CU (one wave per SIMD)", 256)) return 1;
+    if (run_loop<4, 1, FRAG | COPY | BARRIER>("128-row workgroups, two per CU", 512)) return 1;
+    if (run_loop<4, 2, FRAG | COPY | BARRIER, 2>("64 rows per wave, 4 waves (one per SIMD), every fragment used twice", 256)) return 1;
+    if (run_loop<4, 2, FRAG | COPY, 2>("   the same without the barrier", 256)) return 1;
+    for (int rep = 0; rep < 4; rep++) hipLaunchKernelGGL(pingpong_kernel, dim3(256), dim3(512), 0, 0, TILES, d_k, d_v, d_out, d_stamps);
+    if (report("ping-pong: matrix phase | vector phase, barrier between", 8, 256)) return 1;
+    return 0;
+}
