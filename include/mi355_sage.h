@@ -43,6 +43,8 @@ extern "C" {
 
 /* Quantization recipe flags (k_flags). */
 #define MI355_SAGE_K_SMOOTH  1   /* subtract the per-channel mean of K over the keys          */
+#define MI355_SAGE_ROPE_INTERLEAVED 0   /* pairs (x[2i], x[2i+1]): serenitymojo/ops/rope.mojo:7-9 (FLUX, Klein, Z-Image) */
+#define MI355_SAGE_ROPE_HALFSPLIT   1   /* pairs (x[i], x[i+D/2]): serenitymojo/ops/rope.mojo:10-13 (Anima, Hunyuan, LTX-2 ...) */
 #define MI355_SAGE_K_BALANCE 2   /* per channel d: K / s_d, Q * s_d with s_d = sqrt(max|K - mean|)
                                     over the keys: scores are unchanged, and a channel whose
                                     range is r times the others' costs each side sqrt(r), not
@@ -133,7 +135,7 @@ int mi355_sage_sdpa_bf16_norm_rope(
     void* stream,
     int variant, int blkq, int blkk, int k_flags,
     const void* q_gain, const void* k_gain, float eps,
-    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows, int rope_layout,
     void* workspace, size_t workspace_bytes);
 
 /* Replaces flame_cudnn_sdpa_bf16_train_fwd (cudnn_sdpa.cpp:470-484), the symbol
@@ -211,7 +213,7 @@ int mi355_sage_sdpa_bf16_norm_rope_train_fwd(
     void* stream,
     int variant,
     const void* q_gain, const void* k_gain, float eps,
-    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows, int rope_layout,
     void* workspace, size_t workspace_bytes);
 
 /* Bytes of workspace the one-shot calls need for this problem (0 on bad
@@ -269,14 +271,17 @@ int mi355_sage_quant_qk_bf16(
  * (serenitymojo/sampling/klein_sampler.mojo:305-307), batch b starting at row
  * b*rope_batch_rows (0 = one table for all batches); both NULL = norm only.  Q rows and K rows
  * use the same table (self-attention positions), so with tables N_q must equal N_kv (-2
- * otherwise).  Gains and tables must be 16-byte aligned. */
+ * otherwise).  rope_layout: MI355_SAGE_ROPE_INTERLEAVED, or MI355_SAGE_ROPE_HALFSPLIT for the
+ * pairing (i, i + D/2) of rope_halfsplit (serenitymojo/ops/rope.mojo:147-165; per-head norm +
+ * half-split rotation as in serenitymojo/models/anima/block.mojo:360-366); ignored without tables.
+ * Gains and tables must be 16-byte aligned. */
 int mi355_sage_quant_qk_norm_rope_bf16(
     const void* Q, const void* K,
     int B, int H, int N_q, int N_kv, int D, float scale,
     const int64_t* q_strides, const int64_t* k_strides,
     int64_t q_offset_elems, int64_t k_offset_elems,
     const void* q_gain, const void* k_gain, float eps,
-    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+    const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows, int rope_layout,
     int blkq, int blkk, int k_flags,
     void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
     void* scratch, size_t scratch_bytes, void* stream);

@@ -37,14 +37,14 @@ SIGNATURES = {
     "mi355_sage_quant_qk_bf16": (_int, [_vp, _vp] + [_int] * 5 + [ctypes.c_float, _i64p, _i64p, _i64, _i64]
                                  + [_int] * 5 + [_vp] * 8 + [ctypes.c_size_t, _vp]),
     "mi355_sage_quant_qk_norm_rope_bf16": (_int, [_vp, _vp] + [_int] * 5 + [ctypes.c_float, _i64p, _i64p, _i64, _i64]
-                                           + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64]
+                                           + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64, _int]
                                            + [_int] * 3 + [_vp] * 8 + [ctypes.c_size_t, _vp]),
     "mi355_sage_sdpa_bf16_norm_rope": (_int, [_vp] * 4 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [_i64] * 4
                                        + [_int, _vp, _int, _int, _int, _int]
-                                       + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64] + [_vp, ctypes.c_size_t]),
+                                       + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64, _int] + [_vp, ctypes.c_size_t]),
     "mi355_sage_sdpa_bf16_norm_rope_train_fwd": (_int, [_vp] * 5 + [_int] * 5 + [ctypes.c_float] + [_i64p] * 4 + [_i64] * 5
                                                  + [_int, _int, _int, _vp, _int]
-                                                 + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64] + [_vp, ctypes.c_size_t]),
+                                                 + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64, _int] + [_vp, ctypes.c_size_t]),
     "mi355_sage_quant_v_f16": (_int, [_vp] + [_int] * 4 + [_i64p, _i64, _int, _int, _vp, _vp]),
     "mi355_sage_quant_v_fp8": (_int, [_vp] + [_int] * 4 + [_i64p, _i64, _int, _int, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "mi355_sage_attn_fwd": (_int, [_vp, _vp, _int, _vp, _vp, _int, _vp, _vp, _int] + [_int] * 8
@@ -54,6 +54,8 @@ SIGNATURES = {
 
 K_SMOOTH = 1
 K_BALANCE = 2
+ROPE_INTERLEAVED = 0
+ROPE_HALFSPLIT = 1
 
 _lib = None
 

@@ -335,6 +335,12 @@ def sdpa_chunked(q, k, v, mask, scale, variant=PV_FP16):
     return _masked("sdpa_chunked", q, k, v, mask, scale, variant, True)
 
 
+def sdpa_tiled(q, k, v, mask, scale, variant=PV_FP16):
+    """attention.mojo:1721-1759: the reference's online-softmax variant of `sdpa` for large S
+    (same contract and result; never holds the [S,S] scores).  This kernel is that already."""
+    return _masked("sdpa_tiled", q, k, v, mask, scale, variant, True)
+
+
 def sdpa_cross_masked(q, k, v, mask, scale, variant=PV_FP16):
     """attention.mojo:1897-1936: rectangular attention with an additive bias [B,H,Sq,Skv]."""
     return _masked("sdpa_cross_masked", q, k, v, mask, scale, variant, False)
@@ -424,7 +430,7 @@ def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin):
 
 
 def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16,
-                             blkq=None, blkk=64, k_flags=_lib.K_SMOOTH | _lib.K_BALANCE):
+                             blkq=None, blkk=64, k_flags=_lib.K_SMOOTH | _lib.K_BALANCE, halfsplit=False):
     """The attention block of a DiT layer from the projections on, in one call:
 
         q = rope_interleaved(rms_norm(q_pre, q_norm, eps), cos, sin)
@@ -434,7 +440,9 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
     (serenitymojo/models/klein/single_block.mojo:977-982) with the norm and the rotation fused
     into the quantizers.  q_pre/k_pre/v: BF16 [B,S,H,Dh]; q_norm/k_norm: [Dh] (cast to BF16 like
     ops/norm.mojo:170-172 does when the gain's dtype differs); cos/sin: F32 [S*H, Dh/2]
-    (sampling/klein_sampler.mojo:305-307) or [B*S*H, Dh/2], or None for norm only."""
+    (sampling/klein_sampler.mojo:305-307) or [B*S*H, Dh/2], or None for norm only.
+    halfsplit: rope_halfsplit instead of rope_interleaved (ops/rope.mojo:10-13; the per-head norm +
+    half-split rotation of models/anima/block.mojo:360-366)."""
     name = "qk_norm_rope_sdpa_nomask"
     gq, gk, cos, sin, batch_rows = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin)
     B, S, H, Dh = q_pre.shape
@@ -450,13 +458,14 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
         st, st, st, st, 0, 0, 0, 0, 0, torch.cuda.current_stream(q_pre.device).cuda_stream,
         variant, blkq, blkk, int(k_flags), gq.data_ptr(), gk.data_ptr(), float(eps),
         cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
-        ws.data_ptr(), ws.numel())
+        _lib.ROPE_HALFSPLIT if halfsplit else _lib.ROPE_INTERLEAVED, ws.data_ptr(), ws.numel())
     if rc != 0:
         raise Error("%s: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (name, rc, B, S, H, Dh))
     return o
 
 
-def qk_norm_rope_sdpa_flash_train_fwd(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16):
+def qk_norm_rope_sdpa_flash_train_fwd(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16,
+                                      halfsplit=False):
     """The same block where the caller keeps the attention statistics for a backward pass:
     rms_norm / rope_interleaved followed by sdpa_flash_train_fwd
     (serenitymojo/ops/attention_flash.mojo:149-202).  Returns an SdpaFlashFwd whose stats are the
@@ -475,7 +484,7 @@ def qk_norm_rope_sdpa_flash_train_fwd(q_pre, k_pre, v, q_norm, k_norm, eps, cos,
         st, st, st, st, 0, 0, 0, 0, 0, 0, S, S, torch.cuda.current_stream(q_pre.device).cuda_stream,
         variant, gq.data_ptr(), gk.data_ptr(), float(eps),
         cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
-        ws.data_ptr(), ws.numel())
+        _lib.ROPE_HALFSPLIT if halfsplit else _lib.ROPE_INTERLEAVED, ws.data_ptr(), ws.numel())
     if rc != 0:
         raise Error("%s: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (name, rc, B, S, H, Dh))
     return SdpaFlashFwd(o, o, q_pre, k_pre, v, stats)

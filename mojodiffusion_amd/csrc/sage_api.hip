@@ -158,17 +158,18 @@ struct Pre {
 
 // q_gain / k_gain null together = nothing to do.  Tables are optional on top of the gains.
 int make_pre(const void* q_gain, const void* k_gain, float eps, const void* rope_cos, const void* rope_sin,
-             int64_t rope_batch_rows, Pre* out) {
+             int64_t rope_batch_rows, int rope_layout, Pre* out) {
     *out = Pre{};
     if (!q_gain && !k_gain && !rope_cos && !rope_sin) return 0;
     if (!q_gain || !k_gain) { SAGE_LOG("RMSNorm gains must be given for both Q and K"); return MI355_SAGE_EINVAL; }
     if ((rope_cos == nullptr) != (rope_sin == nullptr)) return MI355_SAGE_EINVAL;
     if (!(eps >= 0.0f) || rope_batch_rows < 0) return MI355_SAGE_EINVAL;
+    if (rope_layout != MI355_SAGE_ROPE_INTERLEAVED && rope_layout != MI355_SAGE_ROPE_HALFSPLIT) return MI355_SAGE_EINVAL;
     const uintptr_t bits = reinterpret_cast<uintptr_t>(q_gain) | reinterpret_cast<uintptr_t>(k_gain) |
                            reinterpret_cast<uintptr_t>(rope_cos) | reinterpret_cast<uintptr_t>(rope_sin);
     if (bits & 15) { SAGE_LOG("gains and RoPE tables must be 16-byte aligned"); return MI355_SAGE_EUNSUPPORTED; }
     out->q = PreOp{static_cast<const uint16_t*>(q_gain), eps, static_cast<const float*>(rope_cos),
-                   static_cast<const float*>(rope_sin), rope_batch_rows};
+                   static_cast<const float*>(rope_sin), rope_batch_rows, rope_layout == MI355_SAGE_ROPE_HALFSPLIT ? 1 : 0};
     out->k = out->q;
     out->k.gain = static_cast<const uint16_t*>(k_gain);
     return 0;
@@ -518,14 +519,14 @@ int mi355_sage_quant_qk_norm_rope_bf16(const void* Q, const void* K, int B, int 
                                        float scale, const int64_t* q_strides, const int64_t* k_strides,
                                        int64_t q_off, int64_t k_off,
                                        const void* q_gain, const void* k_gain, float eps,
-                                       const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+                                       const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows, int rope_layout,
                                        int blkq, int blkk, int k_flags,
                                        void* q8, void* qscale, void* k8, void* kscale,
                                        void* kmean, void* qmul, void* kmul,
                                        void* scratch, size_t scratch_bytes, void* stream) {
     Pre pre;
     int rc;
-    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
+    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, rope_layout, &pre))) return rc;
     if (!pre.q.gain) return MI355_SAGE_EINVAL;
     return quant_qk_entry(Q, K, B, H, N_q, N_kv, D, scale, q_strides, k_strides, q_off, k_off, pre, blkq, blkk,
                           k_flags, 0, 0, q8, qscale, k8, kscale, kmean, qmul, kmul, scratch, scratch_bytes, stream);
@@ -539,11 +540,11 @@ int mi355_sage_sdpa_bf16_norm_rope(const void* Q, const void* K, const void* V, 
                                    int causal, void* stream,
                                    int variant, int blkq, int blkk, int k_flags,
                                    const void* q_gain, const void* k_gain, float eps,
-                                   const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+                                   const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows, int rope_layout,
                                    void* workspace, size_t workspace_bytes) {
     Pre pre;
     int rc;
-    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
+    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, rope_layout, &pre))) return rc;
     if (!pre.q.gain) return MI355_SAGE_EINVAL;
     return sdpa_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, 0, causal, 0, stream, variant, blkq, blkk,
@@ -558,13 +559,13 @@ int mi355_sage_sdpa_bf16_norm_rope_train_fwd(const void* Q, const void* K, const
                                              int64_t stats_off, int causal, int real_N_q, int real_N_kv,
                                              void* stream, int variant,
                                              const void* q_gain, const void* k_gain, float eps,
-                                             const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows,
+                                             const void* rope_cos, const void* rope_sin, int64_t rope_batch_rows, int rope_layout,
                                              void* workspace, size_t workspace_bytes) {
     if (!Stats) return MI355_SAGE_EINVAL;
     (void)real_N_q;
     Pre pre;
     int rc;
-    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, &pre))) return rc;
+    if ((rc = make_pre(q_gain, k_gain, eps, rope_cos, rope_sin, rope_batch_rows, rope_layout, &pre))) return rc;
     if (!pre.q.gain) return MI355_SAGE_EINVAL;
     return sdpa_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
                      o_strides, q_off, k_off, v_off, o_off, stats_off, causal, real_N_kv, stream, variant,

@@ -32,6 +32,7 @@ struct PreOp {
     const float* cos;            // fp32 [rows, D/2], row = n*H + h (+ b*batch_rows); null = no rotation
     const float* sin;
     int64_t batch_rows;          // 0: all batches share the table
+    int halfsplit;               // 0: pairs (2i, 2i+1) (ops/rope.mojo:7-9); 1: pairs (i, i + D/2) (ops/rope.mojo:10-13)
 };
 
 // Keys lo <= s < hi take no part (statistics, scale blocks, scores); lo >= hi: no such range.

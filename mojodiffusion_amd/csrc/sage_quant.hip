@@ -63,6 +63,7 @@ __device__ __forceinline__ bool key_kept(int s, int N, const KeyMask& m) { retur
 //   8, which pair lanes of the row, then 4, 2, 1 inside the lane;
 //   inv = 1/sqrt(sum/D + eps); y = bf16((x*inv)*gain); rotation of (y[2i], y[2i+1]) by
 //   the table angle with both products rounded before the subtract / add; result bf16.
+//   (p.halfsplit: the pairs are (y[i], y[i + D/2]) instead.)
 template <int D>
 __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, int row, int col, bool valid, float* x) {
     constexpr int CPR = D / 8;
@@ -89,7 +90,32 @@ __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, i
         const float t = x[e] * inv;
         y[e] = round_to_bf16(t * g[e]);
     }
-    if (p.cos != nullptr) {
+    if (p.cos != nullptr && p.halfsplit) {
+        // pairs (i, i + D/2): the partner channel sits in the lane CPR/2 further on (or back) among
+        // the CPR lanes of this row; both lanes of a pair use table entries (col mod D/2) .. +7
+        float yp[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) yp[e] = __shfl_xor(y[e], CPR / 2, 64);
+        const bool upper = col >= D / 2;
+        float cv[8], sv[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) cv[e] = 1.0f, sv[e] = 0.0f;
+        if (valid) {
+            const int64_t trow = (int64_t)b * p.batch_rows + (int64_t)row * H + h;
+            const float* pc = p.cos + trow * (D / 2) + (col & (D / 2 - 1));
+            const float* ps = p.sin + trow * (D / 2) + (col & (D / 2 - 1));
+            const float4 c0 = *reinterpret_cast<const float4*>(pc), c1 = *reinterpret_cast<const float4*>(pc + 4);
+            const float4 s0 = *reinterpret_cast<const float4*>(ps), s1 = *reinterpret_cast<const float4*>(ps + 4);
+            cv[0] = c0.x; cv[1] = c0.y; cv[2] = c0.z; cv[3] = c0.w; cv[4] = c1.x; cv[5] = c1.y; cv[6] = c1.z; cv[7] = c1.w;
+            sv[0] = s0.x; sv[1] = s0.y; sv[2] = s0.z; sv[3] = s0.w; sv[4] = s1.x; sv[5] = s1.y; sv[6] = s1.z; sv[7] = s1.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            // lower half: x0*c - x1*s with x0 = own, x1 = partner; upper half: x1*c + x0*s with x1 = own
+            const float own = y[e] * cv[e], oth = yp[e] * sv[e];
+            x[e] = round_to_bf16(upper ? own + oth : own - oth);
+        }
+    } else if (p.cos != nullptr) {
         float4 c4 = {1.f, 1.f, 1.f, 1.f}, s4 = {0.f, 0.f, 0.f, 0.f};
         if (valid) {
             const int64_t trow = (int64_t)b * p.batch_rows + (int64_t)row * H + h;

@@ -425,6 +425,23 @@ int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const floa
     return 0;
 }
 
+/* serenitymojo/ops/rope.mojo:10-13, :147-165: pairs (x[i], x[i + D/2]); separate multiplies, then
+ * one subtract / add. */
+int sage_oracle_rope_halfsplit_f32(const float* x, const float* cs, const float* sn,
+                                   int64_t rows, int D, float* out) {
+    if (!x || !cs || !sn || !out || rows <= 0 || D <= 0 || (D & 1)) return -1;
+    int half = D / 2;
+    for (int64_t r = 0; r < rows; r++)
+        for (int i = 0; i < half; i++) {
+            float x0 = x[r * D + i], x1 = x[r * D + i + half];
+            float cv = cs[r * half + i], sv = sn[r * half + i];
+            float a = x0 * cv, b = x1 * sv, c = x1 * cv, d = x0 * sv;
+            out[r * D + i] = a - b;
+            out[r * D + i + half] = c + d;
+        }
+    return 0;
+}
+
 /* bf16 activations: RMSNorm with a bf16 gain, stored as bf16 (norm.mojo:81-114), then
  * interleaved RoPE with fp32 tables on that bf16 tensor, stored as bf16 (rope.mojo:104-122).
  * x is logical [B,H,N,D] through strides; tables are [rows_per_batch, D/2] with row n*H + h
@@ -434,6 +451,15 @@ int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const floa
 int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
                                const uint16_t* gain, float eps, const float* cs, const float* sn,
                                int64_t table_batch_rows, uint16_t* y) {
+    return sage_oracle_norm_rope_bf16_ex(x, B, H, N, D, st, gain, eps, cs, sn, table_batch_rows, 0, y);
+}
+
+/* rope_layout 0: interleaved pairs (rope.mojo:7-9); 1: half-split pairs (rope.mojo:10-13), the
+ * per-head RMSNorm + rope_halfsplit sequence of serenitymojo/models/anima/block.mojo:360-366. */
+int sage_oracle_norm_rope_bf16_ex(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
+                                  const uint16_t* gain, float eps, const float* cs, const float* sn,
+                                  int64_t table_batch_rows, int rope_layout, uint16_t* y) {
+    if (rope_layout != 0 && rope_layout != 1) return -1;
     if (!x || !st || !gain || !y || B <= 0 || H <= 0 || N <= 0 || D <= 0 || (D & 1) || D > 1024) return -1;
     if ((cs == NULL) != (sn == NULL)) return -1;
     int half = D / 2;
@@ -456,11 +482,12 @@ int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, co
         if (cs) {
             int64_t row = (int64_t)b * table_batch_rows + (int64_t)n * H + h;
             for (int i = 0; i < half; i++) {
-                float x0 = t[2 * i], x1 = t[2 * i + 1];
+                int i0 = rope_layout ? i : 2 * i, i1 = rope_layout ? i + half : 2 * i + 1;
+                float x0 = t[i0], x1 = t[i1];
                 float cv = cs[row * half + i], sv = sn[row * half + i];
                 float a = x0 * cv, bb = x1 * sv, c = x0 * sv, dd = x1 * cv;
-                dst[2 * i] = sage_oracle_f32_to_bf16(a - bb);
-                dst[2 * i + 1] = sage_oracle_f32_to_bf16(c + dd);
+                dst[i0] = sage_oracle_f32_to_bf16(a - bb);
+                dst[i1] = sage_oracle_f32_to_bf16(c + dd);
             }
         } else {
             for (int d = 0; d < D; d++) dst[d] = sage_oracle_f32_to_bf16(t[d]);

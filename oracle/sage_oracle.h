@@ -105,6 +105,10 @@ int sage_oracle_rms_norm_f32(const float* x, const float* g, int64_t rows, int c
 /* Interleaved RoPE in fp32: serenitymojo/ops/rope.mojo:7-9.  Pinned by ops_smoke2.mojo:95-120. */
 int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const float* sn,
                                      int64_t rows, int D, float* out);
+/* Half-split RoPE in fp32 (pairs x[i], x[i + D/2]): serenitymojo/ops/rope.mojo:10-13.  Pinned by
+ * the reference's vector ops_smoke2.mojo:113-132 (y_half_ref). */
+int sage_oracle_rope_halfsplit_f32(const float* x, const float* cs, const float* sn,
+                                   int64_t rows, int D, float* out);
 /* The bf16 pipeline rms_norm -> (bf16) -> rope_interleaved -> (bf16) of
  * serenitymojo/models/klein/single_block.mojo:977-981 on a strided [B,H,N,D] view; output
  * contiguous [B,N,H,D].  Tables [.., D/2] fp32 with row n*H + h (+ b*table_batch_rows);
@@ -112,6 +116,11 @@ int sage_oracle_rope_interleaved_f32(const float* x, const float* cs, const floa
 int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
                                const uint16_t* gain, float eps, const float* cs, const float* sn,
                                int64_t table_batch_rows, uint16_t* y);
+/* The same with the pairing chosen: rope_layout 0 interleaved, 1 half-split (the per-head
+ * rms_norm -> rope_halfsplit sequence of serenitymojo/models/anima/block.mojo:360-366). */
+int sage_oracle_norm_rope_bf16_ex(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
+                                  const uint16_t* gain, float eps, const float* cs, const float* sn,
+                                  int64_t table_batch_rows, int rope_layout, uint16_t* y);
 
 /* ---- quantizers --------------------------------------------------------- */
 /* Padded token count used by every quantized tensor: N rounded up to `mult`. */

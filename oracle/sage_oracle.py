@@ -111,6 +111,11 @@ def lib():
                                                ctypes.c_float, ctypes.c_void_p]
         L.sage_oracle_rope_interleaved_f32.restype = ctypes.c_int
         L.sage_oracle_rope_interleaved_f32.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        L.sage_oracle_rope_halfsplit_f32.restype = ctypes.c_int
+        L.sage_oracle_rope_halfsplit_f32.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+        L.sage_oracle_norm_rope_bf16_ex.restype = ctypes.c_int
+        L.sage_oracle_norm_rope_bf16_ex.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p, ctypes.c_float,
+                                                    ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
         L.sage_oracle_norm_rope_bf16.restype = ctypes.c_int
         L.sage_oracle_norm_rope_bf16.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 4 + [_i64p, ctypes.c_void_p, ctypes.c_float,
                                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
@@ -254,9 +259,23 @@ def rope_interleaved_f32(x, cos, sin):
     return out
 
 
-def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=0):
+def rope_halfsplit_f32(x, cos, sin):
+    """x [rows, D], cos/sin [rows, D/2], all fp32; pairs (x[i], x[i + D/2]) (serenitymojo/ops/rope.mojo:10-13)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    cos = np.ascontiguousarray(cos, dtype=np.float32)
+    sin = np.ascontiguousarray(sin, dtype=np.float32)
+    if cos.shape != (x.shape[0], x.shape[1] // 2) or sin.shape != cos.shape:
+        raise ValueError("rope_halfsplit_f32: cos/sin must be [rows, D/2] with one row per row of x")
+    out = np.empty_like(x)
+    _chk(lib().sage_oracle_rope_halfsplit_f32(_p(x), _p(cos), _p(sin), x.shape[0], x.shape[1], _p(out)),
+         "rope_halfsplit_f32")
+    return out
+
+
+def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=0, halfsplit=False):
     """x: uint16 [B,S,H,D] bf16 bits; gain: uint16 [D]; cos/sin: fp32 [rows, D/2] with row s*H + h
-    (plus b*table_batch_rows), or None for no rotation.  Returns uint16 [B,S,H,D]."""
+    (plus b*table_batch_rows), or None for no rotation; halfsplit: pairs (i, i + D/2) instead of
+    (2i, 2i+1).  Returns uint16 [B,S,H,D]."""
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     g = np.ascontiguousarray(gain_bf16, dtype=np.uint16)
     B, S, H, D = x.shape
@@ -269,9 +288,10 @@ def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=
             raise ValueError("norm_rope_bf16: cos/sin must be [>= %d, %d]" % (need, D // 2))
     if g.shape != (D,):
         raise ValueError("norm_rope_bf16: gain must be [%d]" % D)
-    _chk(lib().sage_oracle_norm_rope_bf16(_p(x), B, H, S, D, strides_bshd(S, H, D), _p(g), eps,
-                                          _p(cos) if cos is not None else None,
-                                          _p(sin) if sin is not None else None, table_batch_rows, _p(y)),
+    _chk(lib().sage_oracle_norm_rope_bf16_ex(_p(x), B, H, S, D, strides_bshd(S, H, D), _p(g), eps,
+                                             _p(cos) if cos is not None else None,
+                                             _p(sin) if sin is not None else None, table_batch_rows,
+                                             1 if halfsplit else 0, _p(y)),
          "norm_rope_bf16")
     return y
 

@@ -11,7 +11,7 @@ Sources (relative to the reference checkout):
       inputs are the closed forms of ops/parity/sdpa_bwd_parity.mojo:44-65
   serenitymojo/ops_smoke2.mojo:239-278              q/k/v/out literals, [1,4,2,8], scale 0.35355339
   serenitymojo/ops_smoke.mojo:78-96                 rms_norm x[3,6], g[6], eps 1e-6 -> y[3,6]
-  serenitymojo/ops_smoke2.mojo:92-120               rope x[3,8], cos/sin[3,4] -> interleaved y[3,8]
+  serenitymojo/ops_smoke2.mojo:92-120               rope x[3,8], cos/sin[3,4] -> interleaved y[3,8], half-split y[3,8]
 
 Run once where the reference is mounted:  python tests/golden/make_fixtures.py [/root/reference]
 """
@@ -79,6 +79,7 @@ def main():
     pre["rope_cos"] = literals(text, "cos_rope", 12)
     pre["rope_sin"] = literals(text, "sin_rope", 12)
     pre["rope_y_interleaved"] = literals(text, "y_int_ref", 24)
+    pre["rope_y_halfsplit"] = literals(text, "y_half_ref", 24)
     with open(os.path.join(HERE, "ops_smoke_rmsnorm_rope_kat.json"), "w") as f:
         json.dump(pre, f, indent=0)
     print("wrote fixtures to", HERE)

@@ -192,7 +192,7 @@ def f32_to_bf16_bits_rne(x):
     return (r >> 16).astype(np.uint16)
 
 
-def norm_rope_bf16(x_bits_bshd, gain_bits, eps, cos=None, sin=None, table_batch_rows=0):
+def norm_rope_bf16(x_bits_bshd, gain_bits, eps, cos=None, sin=None, table_batch_rows=0, halfsplit=False):
     B, S, H, D = x_bits_bshd.shape
     x = bf16_to_f32(x_bits_bshd)                                   # [B,S,H,D]
     assert D <= 256
@@ -213,9 +213,13 @@ def norm_rope_bf16(x_bits_bshd, gain_bits, eps, cos=None, sin=None, table_batch_
     rows = (np.arange(B)[:, None, None] * table_batch_rows + np.arange(S)[None, :, None] * H + np.arange(H)[None, None, :])
     c = np.asarray(cos, np.float32)[rows]                          # [B,S,H,half]
     s = np.asarray(sin, np.float32)[rows]
-    y0, y1 = y[..., 0::2], y[..., 1::2]
+    # pairs (2i, 2i+1), or (i, i + D/2) in the half-split form
+    y0, y1 = (y[..., :half], y[..., half:]) if halfsplit else (y[..., 0::2], y[..., 1::2])
     o0 = ((y0 * c).astype(np.float32) - (y1 * s).astype(np.float32)).astype(np.float32)
     o1 = ((y0 * s).astype(np.float32) + (y1 * c).astype(np.float32)).astype(np.float32)
     out = np.empty((B, S, H, D), np.float32)
-    out[..., 0::2], out[..., 1::2] = o0, o1
+    if halfsplit:
+        out[..., :half], out[..., half:] = o0, o1
+    else:
+        out[..., 0::2], out[..., 1::2] = o0, o1
     return f32_to_bf16_bits_rne(out)

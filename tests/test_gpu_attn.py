@@ -362,6 +362,9 @@ def test_additive_mask_entry_points(oracle, variant, Sq, Skv):
     assert cos >= COS, (cos, mx)
     if Sq == Skv:
         np.testing.assert_array_equal(H.to_bits(A.sdpa_chunked(qd, kd, vd, md, w.scale, variant)), H.to_bits(got))
+        np.testing.assert_array_equal(H.to_bits(A.sdpa_tiled(qd, kd, vd, md, w.scale, variant)), H.to_bits(got))
+        with pytest.raises(A.Error, match=r"sdpa_tiled: mask must be \[B,H,S,S\]"):
+            A.sdpa_tiled(qd, kd, vd, md[:, :1], w.scale, variant)
         zero = torch.zeros_like(md)
         # (the biased instantiation takes every tile's maximum on the biased scores, the plain one
         # is lazy about it: same function, last-bit differences)

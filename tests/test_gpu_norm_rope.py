@@ -22,7 +22,7 @@ def _gains(rng, D):
             f32_to_bf16_bits((0.7 + 0.3 * rng.standard_normal(D)).astype(np.float32)))
 
 
-def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows):
+def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows, halfsplit=False):
     import torch
     import gpu_harness as H
     L = _lib.lib()
@@ -42,7 +42,7 @@ def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_row
     rc = L.mi355_sage_quant_qk_norm_rope_bf16(
         qd.data_ptr(), kd.data_ptr(), B, Hh, S, S, D, scale, st, st, 0, 0,
         gqd.data_ptr(), gkd.data_ptr(), eps, cd.data_ptr() if cd is not None else None,
-        sd.data_ptr() if sd is not None else None, batch_rows, blkq, blkk, (1 if smooth else 0) | 2,
+        sd.data_ptr() if sd is not None else None, batch_rows, 1 if halfsplit else 0, blkq, blkk, (1 if smooth else 0) | 2,
         q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
         scr.data_ptr(), scr.numel(), H.stream())
     assert rc == 0, rc
@@ -51,11 +51,14 @@ def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_row
                 kmean=km.cpu().numpy(), qmul=qm.cpu().numpy(), kmul=kmu.cpu().numpy())
 
 
+@pytest.mark.parametrize("halfsplit", [False, True])
 @pytest.mark.parametrize("D,S,blkq,blkk,smooth,rope,per_batch", [
     (128, 300, 128, 64, True, True, False), (128, 1100, 128, 64, True, True, True),
     (64, 200, 64, 64, True, True, False), (128, 77, 32, 32, False, True, False),
     (128, 513, 128, 64, True, False, False), (64, 1, 32, 32, True, True, False)])
-def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_batch):
+def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_batch, halfsplit):
+    if halfsplit and not rope:
+        pytest.skip("the pairing only matters with tables")
     rng = np.random.default_rng(100 + S)
     B, Hh = 2, 3
     q = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32) * 2.0)
@@ -66,9 +69,9 @@ def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_
     cos, sin = _tables(rng, S * Hh * (B if per_batch else 1), D) if rope else (None, None)
     batch_rows = S * Hh if per_batch else 0
     eps, scale = 1e-6, 1.0 / np.sqrt(D)
-    got = _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows)
-    qn = oracle.norm_rope_bf16(q, gq, eps, cos, sin, batch_rows)
-    kn = oracle.norm_rope_bf16(k, gk, eps, cos, sin, batch_rows)
+    got = _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows, halfsplit)
+    qn = oracle.norm_rope_bf16(q, gq, eps, cos, sin, batch_rows, halfsplit=halfsplit)
+    kn = oracle.norm_rope_bf16(k, gk, eps, cos, sin, batch_rows, halfsplit=halfsplit)
     import gpu_harness as H
     want = H.oracle_quant_qk(oracle, qn, kn, scale, blkq, blkk, smooth, True)
     for name in ("kmean", "qmul", "kmul"):
@@ -80,8 +83,8 @@ def test_fused_quantizers_bit_exact(oracle, D, S, blkq, blkk, smooth, rope, per_
     np.testing.assert_array_equal(got["k8"], want["k8"])
 
 
-@pytest.mark.parametrize("variant,wid", [(0, 2), (1, 2), (0, 1)])
-def test_one_shot_equals_unfused_pipeline(oracle, variant, wid):
+@pytest.mark.parametrize("variant,wid,halfsplit", [(0, 2, False), (1, 2, False), (0, 1, False), (0, 2, True), (1, 1, True)])
+def test_one_shot_equals_unfused_pipeline(oracle, variant, wid, halfsplit):
     """mi355_sage_sdpa_bf16_norm_rope on the projections == the plain one-shot call on
     norm/rope'd tensors (the CPU checker's, which the test above proves equal to the fused
     kernels' view bit for bit): same quantized tensors, hence the same output bits."""
@@ -96,10 +99,10 @@ def test_one_shot_equals_unfused_pipeline(oracle, variant, wid):
     qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
     got = A.qk_norm_rope_sdpa_nomask(qd, kd, vd, H.dev_bf16(gq), H.dev_bf16(gk), 1e-6,
                                      torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), w.scale, variant,
-                                     blkq=w.blkq, blkk=w.blkk)
+                                     blkq=w.blkq, blkk=w.blkk, halfsplit=halfsplit)
     torch.cuda.synchronize()
-    qn = oracle.norm_rope_bf16(q, gq, 1e-6, cos, sin, 0)
-    kn = oracle.norm_rope_bf16(k, gk, 1e-6, cos, sin, 0)
+    qn = oracle.norm_rope_bf16(q, gq, 1e-6, cos, sin, 0, halfsplit=halfsplit)
+    kn = oracle.norm_rope_bf16(k, gk, 1e-6, cos, sin, 0, halfsplit=halfsplit)
     want = torch.empty_like(qd)
     st = _lib.strides_bhnd(w.S, w.H, w.D)
     qnd, knd = H.dev_bf16(qn), H.dev_bf16(kn)
@@ -111,8 +114,9 @@ def test_one_shot_equals_unfused_pipeline(oracle, variant, wid):
     np.testing.assert_array_equal(H.to_bits(got), H.to_bits(want))
     # and against an fp32 attention on the fp32 norm/rope
     cb, sb = np.tile(cos, (w.B, 1)), np.tile(sin, (w.B, 1))      # the table is shared by the batches
-    qf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(q).reshape(-1, w.D), bf16_bits_to_f32(gq), 1e-6), cb, sb)
-    kf = oracle.rope_interleaved_f32(oracle.rms_norm_f32(bf16_bits_to_f32(k).reshape(-1, w.D), bf16_bits_to_f32(gk), 1e-6), cb, sb)
+    rope = oracle.rope_halfsplit_f32 if halfsplit else oracle.rope_interleaved_f32
+    qf = rope(oracle.rms_norm_f32(bf16_bits_to_f32(q).reshape(-1, w.D), bf16_bits_to_f32(gq), 1e-6), cb, sb)
+    kf = rope(oracle.rms_norm_f32(bf16_bits_to_f32(k).reshape(-1, w.D), bf16_bits_to_f32(gk), 1e-6), cb, sb)
     ref = oracle.sdpa_f32(qf.reshape(q.shape), kf.reshape(k.shape), bf16_bits_to_f32(v), w.scale)
     cos_sim, mx = H.cos_maxabs(got.float().cpu().numpy(), ref)
     assert cos_sim >= 0.999, (cos_sim, mx)
@@ -134,23 +138,28 @@ def test_argument_errors():
     # gains missing -> -1; misaligned gain -> -2
     rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 64, 64, 128, 0.1,
                                           st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 1,
-                                          None, None, 1e-6, None, None, 0, None, 0)
+                                          None, None, 1e-6, None, None, 0, 0, None, 0)
     assert rc == -1
     rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 64, 64, 128, 0.1,
                                           st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 1,
-                                          g.data_ptr() + 2, g.data_ptr(), 1e-6, None, None, 0, None, 0)
+                                          g.data_ptr() + 2, g.data_ptr(), 1e-6, None, None, 0, 0, None, 0)
     assert rc == -2
     # the table has one row per position, shared by Q and K: N_q != N_kv is refused (-2), norm only is fine
     t = torch.zeros((64 * 2, 64), dtype=torch.float32, device="cuda")
     st32 = _lib.strides_bhnd(32, 2, 128)
     rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 32, 64, 128, 0.1,
                                           st32, st, st, st32, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
-                                          g.data_ptr(), g.data_ptr(), 1e-6, t.data_ptr(), t.data_ptr(), 0, None, 0)
+                                          g.data_ptr(), g.data_ptr(), 1e-6, t.data_ptr(), t.data_ptr(), 0, 0, None, 0)
     assert rc == -2
     rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 32, 64, 128, 0.1,
                                           st32, st, st, st32, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
-                                          g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, None, 0)
+                                          g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, 0, None, 0)
     assert rc == 0
+    # an unknown pairing is refused
+    rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 64, 64, 128, 0.1,
+                                          st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
+                                          g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, 7, None, 0)
+    assert rc == -1
     torch.cuda.synchronize()
 
 

@@ -34,6 +34,12 @@ def test_rope_reference_vector(oracle, kat):
     s = np.array(kat["rope_sin"], np.float32).reshape(3, 4)
     got = oracle.rope_interleaved_f32(x, c, s)
     np.testing.assert_allclose(got, np.array(kat["rope_y_interleaved"]).reshape(3, 8), rtol=0, atol=3e-7)
+    # the same inputs in the half-split pairing (x[i], x[i + D/2]): y_half_ref of the same test
+    got = oracle.rope_halfsplit_f32(x, c, s)
+    np.testing.assert_allclose(got, np.array(kat["rope_y_halfsplit"]).reshape(3, 8), rtol=0, atol=3e-7)
+    # the two pairings are one rotation seen through a permutation of the channels
+    perm = np.concatenate([np.arange(0, 8, 2), np.arange(1, 8, 2)])          # interleaved -> half-split order
+    np.testing.assert_array_equal(oracle.rope_interleaved_f32(x, c, s)[:, perm], oracle.rope_halfsplit_f32(x[:, perm], c, s))
 
 
 @pytest.mark.parametrize("D", [64, 128, 2560, 3072, 4096])
@@ -98,8 +104,9 @@ def test_properties(oracle):
     assert abs(d1 - d2) < 1e-4 * max(1.0, abs(d1))
 
 
+@pytest.mark.parametrize("halfsplit", [False, True])
 @pytest.mark.parametrize("D,with_rope,batch_rows", [(128, True, 0), (64, True, 0), (128, False, 0), (128, True, 3 * 37)])
-def test_bf16_pipeline_matches_numpy_restatement(oracle, D, with_rope, batch_rows):
+def test_bf16_pipeline_matches_numpy_restatement(oracle, D, with_rope, batch_rows, halfsplit):
     rng = np.random.default_rng(11 + D)
     B, S, H = 2, 37, 3
     x = f32_to_bf16_bits(rng.standard_normal((B, S, H, D)).astype(np.float32) * 3.0)
@@ -108,8 +115,8 @@ def test_bf16_pipeline_matches_numpy_restatement(oracle, D, with_rope, batch_row
     rows = S * H * (B if batch_rows else 1)
     th = rng.uniform(-3.14, 3.14, (rows, D // 2))
     cos, sin = (np.cos(th).astype(np.float32), np.sin(th).astype(np.float32)) if with_rope else (None, None)
-    got = oracle.norm_rope_bf16(x, gain, 1e-6, cos, sin, batch_rows)
-    want = R.norm_rope_bf16(x, gain, 1e-6, cos, sin, batch_rows)
+    got = oracle.norm_rope_bf16(x, gain, 1e-6, cos, sin, batch_rows, halfsplit=halfsplit)
+    want = R.norm_rope_bf16(x, gain, 1e-6, cos, sin, batch_rows, halfsplit=halfsplit)
     np.testing.assert_array_equal(got, want)
     assert not bf16_bits_to_f32(got[0, 3, 1]).any()                 # (signed zeros allowed)
     # and it is the composition of the two fp32 ops with a bf16 store in between, to bf16 precision
@@ -117,6 +124,6 @@ def test_bf16_pipeline_matches_numpy_restatement(oracle, D, with_rope, batch_row
     y = oracle.rms_norm_f32(xf, bf16_bits_to_f32(gain), 1e-6)
     if with_rope:
         idx = (np.arange(B)[:, None, None] * batch_rows + np.arange(S)[None, :, None] * H + np.arange(H)[None, None, :]).reshape(-1)
-        y = oracle.rope_interleaved_f32(y, cos[idx], sin[idx])
+        y = (oracle.rope_halfsplit_f32 if halfsplit else oracle.rope_interleaved_f32)(y, cos[idx], sin[idx])
     # (a rotated pair can cancel, so the bf16 steps of the inputs show as absolute error)
     np.testing.assert_allclose(bf16_bits_to_f32(got).reshape(-1, D), y, rtol=2.0 ** -6, atol=3e-2)
