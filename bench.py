@@ -41,15 +41,28 @@ PEAK_FP8_TOPS = 5000.0       # MI355X dense FP8 MFMA, published
 PEAK_HBM_GBS = 8000.0
 K_FLAGS = 3                  # K mean smoothing + per-channel Q/K balancing (the default recipe)
 
-KERNEL_SOURCES = ("mojodiffusion_amd/csrc/sage_attn.hip", "mojodiffusion_amd/csrc/sage_internal.h")
+KERNEL_SOURCE = "mojodiffusion_amd/csrc/sage_attn.hip"
+KERNEL_HEADER = "mojodiffusion_amd/csrc/sage_internal.h"
 
 
 def kernel_source_digest():
+    """Digest of what the attention kernel is compiled from: its source file and, of the shared
+    header, the tile constants and the argument struct it uses (the other kernels' structs in
+    that header do not change it)."""
     import hashlib
+    import re
     h = hashlib.sha256()
-    for rel in KERNEL_SOURCES:
-        with open(os.path.join(ROOT, rel), "rb") as f:
-            h.update(f.read())
+    with open(os.path.join(ROOT, KERNEL_SOURCE), "rb") as f:
+        h.update(f.read())
+    with open(os.path.join(ROOT, KERNEL_HEADER)) as f:
+        text = f.read()
+    for line in text.split("\n"):
+        if line.startswith("constexpr int k"):
+            h.update(line.encode())
+    for name in ("struct KeyMask", "struct AttnArgs", "inline int v_slot_f16", "inline int v_slot_fp8"):
+        m = re.search(re.escape(name) + r".*?\n}", text, re.S)
+        assert m is not None, name
+        h.update(m.group(0).encode())
     return h.hexdigest()[:16]
 
 
