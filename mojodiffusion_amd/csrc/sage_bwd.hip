@@ -11,8 +11,8 @@
 //                          probabilities vanish), and transposed copies K^T, Q^T, dO^T in tiles of
 //                          64 rows whose rows sit in the slot order of the matrix instruction's
 //                          operand layout (v_slot_f16).
-//   2. bwd_pass_kernel<0>  owner = 128 query rows per workgroup, loop over key tiles   -> dQ
-//   3. bwd_pass_kernel<1>  owner = 128 keys per workgroup, loop over query tiles       -> dK, dV
+//   2. bwd_pass_kernel<0>  owner = 256 query rows per workgroup (8 waves), loop over key tiles  -> dQ
+//   3. bwd_pass_kernel<1>  owner = 128 keys per workgroup (4 waves), loop over query tiles     -> dK, dV
 // In both passes a wave owns 32 rows ("x"), keeps their two bf16 row blocks resident as B operands
 // and walks the other side ("y") in tiles of 64 rows staged in LDS by register-bypassing copies,
 // double buffered, one barrier per tile.  A 32x32 block of scores T[y,x] lands in the accumulator
@@ -163,16 +163,17 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
 // ---------------------------------------------------------------------------------------------
 // Launches 2 and 3.
 // ---------------------------------------------------------------------------------------------
-template <int D, int PASS>
-__global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
+template <int D, int PASS, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdArgs a) {
+    constexpr int XROWS = NW * 32;                  // owner rows per workgroup
     constexpr int CPR = D / 8;                      // 16-byte chunks per natural row
     constexpr int TILE_BYTES = 64 * D * 2;          // natural and transposed tiles have the same size
     constexpr int RUNS = TILE_BYTES / 1024;         // 1 KiB copies per tile
-    constexpr int RPW = RUNS / 4;                   // per wave
+    constexpr int RPW = RUNS / NW;                  // per wave
     constexpr int KS = D / 16;                      // matrix-instruction steps over the head dim
     constexpr int DB = D / 32;                      // 32-channel output blocks
     constexpr int NTR = PASS == 0 ? 1 : 2;          // transposed operands per tile
-    static_assert(RUNS % 4 == 0, "tile copies must divide over four waves");
+    static_assert(RUNS % NW == 0, "tile copies must divide over the waves");
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds_nat[2][2][TILE_BYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_tr[2][NTR][TILE_BYTES];
@@ -182,14 +183,14 @@ __global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
     const int valid_x = PASS == 0 ? a.valid_q : a.valid_kv;
     const int Ny = PASS == 0 ? a.Nkv : a.Nq;
     const int valid_y = PASS == 0 ? a.valid_kv : a.valid_q;
-    const int x_tiles = (Nx + 127) / 128;
+    const int x_tiles = (Nx + XROWS - 1) / XROWS;
     const int xt = blockIdx.x % x_tiles;
     const int bh = blockIdx.x / x_tiles;
     const int b = bh / a.H, h = bh % a.H;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
-    const int x = xt * 128 + wave * 32 + l32;
+    const int x = xt * XROWS + wave * 32 + l32;
     const int xc = min(x, Nx - 1);
 
     // owner side: two resident row blocks (B operands: column = owner row, k = head channel)
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
     const uint8_t* rows_l = reinterpret_cast<const uint8_t*>(a.lse2 + (int64_t)bh * a.nq_pad);
     const uint8_t* rows_d = reinterpret_cast<const uint8_t*>(a.delta + (int64_t)bh * a.nq_pad);
     // owners that are all padding have nothing to compute: they only store zeros
-    const int ntiles = xt * 128 < valid_x ? (valid_y + 63) / 64 : 0;
+    const int ntiles = xt * XROWS < valid_x ? (valid_y + 63) / 64 : 0;
 
     // per-lane pieces of the copy addresses: run i of this wave covers physical chunks
     // (i*4 + wave)*64 + lane of a tile
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
     uint32_t tr_src[RPW];
 #pragma unroll
     for (int i = 0; i < RPW; i++) {
-        const int P = (i * 4 + wave) * 64 + lane;
+        const int P = (i * NW + wave) * 64 + lane;
         const int row = P / CPR, pos = P % CPR;
         nat_row[i] = row;
         nat_col[i] = nat_pos<CPR>(row, pos) * 16;          // the XOR is its own inverse
@@ -246,7 +247,7 @@ __global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
 #pragma unroll
         for (int i = 0; i < RPW; i++) {
             const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], Ny - 1);
-            const uint32_t dst = (uint32_t)((i * 4 + wave) * 1024);
+            const uint32_t dst = (uint32_t)((i * NW + wave) * 1024);
             dma16(y1, row * ys1 + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 0) * TILE_BYTES + dst));
             dma16(y2, row * ys2 + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 1) * TILE_BYTES + dst));
             dma16(t1 + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * NTR + 0) * TILE_BYTES + dst));
@@ -289,26 +290,27 @@ __global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
         const uint8_t* n2 = &lds_nat[stage][1][0];
         const uint8_t* r1 = &lds_tr[stage][0][0];
         const uint8_t* r2 = &lds_tr[stage][NTR - 1][0];
+        // Two 32-row blocks per tile, software-pipelined so that the vector work of one block is
+        // issued between the matrix instructions of the other:
+        //   scores(0) | scores(1) + exponentials(0) | products(0) + exponentials(1) | products(1)
+        v16f tacc[2], gacc[2];
+        uint32_t pp[2][8], sp[2][8];
+        float lse[4], dl[4];
 #pragma unroll
-        for (int blk = 0; blk < 2; blk++) {
-            v16f tacc, gacc;
+        for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) tacc[i] = 0.0f, gacc[i] = 0.0f;
-#pragma unroll
-            for (int s = 0; s < KS; s++) {
-                const v4i f1 = *reinterpret_cast<const v4i*>(n1 + nat_frag[blk][s]);
-                tacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f1), __builtin_bit_cast(v8bf, b1[s]), tacc, 0, 0, 0);
-            }
-#pragma unroll
-            for (int s = 0; s < KS; s++) {
-                const v4i f2 = *reinterpret_cast<const v4i*>(n2 + nat_frag[blk][s]);
-                gacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f2), __builtin_bit_cast(v8bf, b2[s]), gacc, 0, 0, 0);
-            }
-            // element i of a lane: y row (i>>2)*8 + half*4 + (i&3) of the block, column = owner row
-            uint32_t pp[8], sp[8];
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                float lse[4], dl[4];
+            for (int i = 0; i < 16; i++) tacc[blk][i] = 0.0f, gacc[blk][i] = 0.0f;
+        // one k-step of the two score products of a block: T += Y1 . X1^T, G += Y2 . X2^T
+        auto scores_step = [&](int blk, int ks) {
+            const v4i f1 = *reinterpret_cast<const v4i*>(n1 + nat_frag[blk][ks]);
+            const v4i f2 = *reinterpret_cast<const v4i*>(n2 + nat_frag[blk][ks]);
+            tacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f1), __builtin_bit_cast(v8bf, b1[ks]), tacc[blk], 0, 0, 0);
+            gacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f2), __builtin_bit_cast(v8bf, b2[ks]), gacc[blk], 0, 0, 0);
+        };
+        // elements i, i+1 of a block (i even): y rows (i>>2)*8 + half*4 + (i&3) (+1), column = owner row
+        auto softmax_pair = [&](int blk, int i) {
+            const int g = i >> 2;
+            if ((i & 3) == 0) {
                 if constexpr (PASS == 0) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) lse[e] = lse_x, dl[e] = delta_x;
@@ -318,43 +320,59 @@ __global__ __launch_bounds__(256) void bwd_pass_kernel(BwdArgs a) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) lse[e] = vl[e], dl[e] = vd[e];
                 }
-                float p[4], ds[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float arg = fmaf(tacc[g * 4 + e], c, -lse[e]);
-                    if constexpr (PASS == 0) {
-                        // keys past the valid length (only possible in the last tile)
-                        if (t * 64 + blk * 32 + g * 8 + half * 4 + e >= valid_y) arg = -INFINITY;
-                    }
-                    p[e] = __builtin_amdgcn_exp2f(arg);
-                    ds[e] = p[e] * (gacc[g * 4 + e] - dl[e]);
-                }
-                sp[g * 2] = pack_bf16(ds[0], ds[1]);
-                sp[g * 2 + 1] = pack_bf16(ds[2], ds[3]);
-                if constexpr (PASS == 1) {
-                    pp[g * 2] = pack_bf16(p[0], p[1]);
-                    pp[g * 2 + 1] = pack_bf16(p[2], p[3]);
-                }
             }
+            float pr[2], ds[2];
 #pragma unroll
-            for (int j2 = 0; j2 < 2; j2++) {
-                const int j = blk * 2 + j2;
-                const v4i sb = {(int)sp[j2 * 4], (int)sp[j2 * 4 + 1], (int)sp[j2 * 4 + 2], (int)sp[j2 * 4 + 3]};
-#pragma unroll
-                for (int d = 0; d < DB; d++) {
-                    const v4i fa = *reinterpret_cast<const v4i*>(r1 + tr_frag[j] + d * 32 * 128);
-                    acc1[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, sb), acc1[d], 0, 0, 0);
+            for (int e = 0; e < 2; e++) {
+                float arg = fmaf(tacc[blk][i + e], c, -lse[(i & 3) + e]);
+                if constexpr (PASS == 0) {
+                    // keys past the valid length (only possible in the last tile)
+                    if (t * 64 + blk * 32 + g * 8 + half * 4 + (i & 3) + e >= valid_y) arg = -INFINITY;
                 }
-                if constexpr (PASS == 1) {
-                    const v4i pb = {(int)pp[j2 * 4], (int)pp[j2 * 4 + 1], (int)pp[j2 * 4 + 2], (int)pp[j2 * 4 + 3]};
+                pr[e] = __builtin_amdgcn_exp2f(arg);
+                ds[e] = pr[e] * (gacc[blk][i + e] - dl[(i & 3) + e]);
+            }
+            sp[blk][i >> 1] = pack_bf16(ds[0], ds[1]);
+            if constexpr (PASS == 1) pp[blk][i >> 1] = pack_bf16(pr[0], pr[1]);
+        };
+        // matrix instruction m of a block's accumulation: dX1^T += Y1^T . dS  (and dX2^T += Y2^T . P)
+        constexpr int ACC_M = 2 * DB * NTR;
+        auto acc_step = [&](int blk, int m) {
+            const int which = m / (2 * DB), j2 = (m / DB) & 1, d = m % DB;
+            const int j = blk * 2 + j2;
+            if (which == 0) {
+                const v4i sb = {(int)sp[blk][j2 * 4], (int)sp[blk][j2 * 4 + 1], (int)sp[blk][j2 * 4 + 2], (int)sp[blk][j2 * 4 + 3]};
+                const v4i fa = *reinterpret_cast<const v4i*>(r1 + tr_frag[j] + d * 32 * 128);
+                acc1[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, sb), acc1[d], 0, 0, 0);
+            } else if constexpr (PASS == 1) {
+                const v4i pb = {(int)pp[blk][j2 * 4], (int)pp[blk][j2 * 4 + 1], (int)pp[blk][j2 * 4 + 2], (int)pp[blk][j2 * 4 + 3]};
+                const v4i fa = *reinterpret_cast<const v4i*>(r2 + tr_frag[j] + d * 32 * 128);
+                acc2[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, pb), acc2[d], 0, 0, 0);
+            }
+        };
 #pragma unroll
-                    for (int d = 0; d < DB; d++) {
-                        const v4i fa = *reinterpret_cast<const v4i*>(r2 + tr_frag[j] + d * 32 * 128);
-                        acc2[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, pb), acc2[d], 0, 0, 0);
-                    }
-                }
+        for (int ks = 0; ks < KS; ks++) scores_step(0, ks);
+        // scores of block 1 with the exponentials of block 0: 8 pairs over KS k-steps
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            scores_step(1, ks);
+#pragma unroll
+            for (int q = 0; q < 8 / KS; q++) softmax_pair(0, (ks * (8 / KS) + q) * 2);
+        }
+        // accumulation of block 0 with the exponentials of block 1: 8 pairs over ACC_M instructions
+        // (ACC_M is 4, 8 or 16; with 16 a pair goes with every second instruction)
+#pragma unroll
+        for (int m = 0; m < ACC_M; m++) {
+            acc_step(0, m);
+            if constexpr (ACC_M <= 8) {
+#pragma unroll
+                for (int q = 0; q < 8 / ACC_M; q++) softmax_pair(1, (m * (8 / ACC_M) + q) * 2);
+            } else {
+                if (m & 1) softmax_pair(1, (m >> 1) * 2);
             }
         }
+#pragma unroll
+        for (int m = 0; m < ACC_M; m++) acc_step(1, m);
     }
 
     // ---- epilogue: rows of valid owners get their gradient, padding rows zeros -----------------
@@ -390,11 +408,12 @@ template <int D>
 static hipError_t launch_bwd_d(const BwdArgs& a, hipStream_t st) {
     const int64_t bh = (int64_t)a.B * a.H;
     const int64_t prep = bh * (a.nkv_pad / 64 + 3 * (a.nq_pad / 64));
-    const int64_t gq = bh * ((a.Nq + 127) / 128), gk = bh * ((a.Nkv + 127) / 128);
+    constexpr int NWQ = 8, NWK = 4;                 // waves per workgroup of the dQ pass / the dK, dV pass
+    const int64_t gq = bh * ((a.Nq + NWQ * 32 - 1) / (NWQ * 32)), gk = bh * ((a.Nkv + NWK * 32 - 1) / (NWK * 32));
     if (prep > 0x7FFFFFFF || gq > 0x7FFFFFFF || gk > 0x7FFFFFFF) return hipErrorInvalidValue;
     hipLaunchKernelGGL((bwd_prep_kernel<D>), dim3((unsigned)prep), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((bwd_pass_kernel<D, 0>), dim3((unsigned)gq), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((bwd_pass_kernel<D, 1>), dim3((unsigned)gk), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((bwd_pass_kernel<D, 0, NWQ>), dim3((unsigned)gq), dim3(NWQ * 64), 0, st, a);
+    hipLaunchKernelGGL((bwd_pass_kernel<D, 1, NWK>), dim3((unsigned)gk), dim3(NWK * 64), 0, st, a);
     return hipGetLastError();
 }
 
