@@ -322,9 +322,11 @@ int mi355_sage_attn_fwd(
  * operands).  real_N_q / real_N_kv (0 or >= N: all) are the valid lengths; padding rows and keys
  * take no part and their gradient rows are written as zeros.  causal must be 0.
  * Workspace: mi355_sage_bwd_workspace_bytes(...) bytes, 256-byte aligned, or NULL for the
- * library's per-stream buffer (same rules as the forward).  Unlike the log-sum-exp handed to
- * cuDNN, Stats may come from the quantized forward: the probabilities are then normalised by the
- * quantized scores' sum, which differs from the bf16 one by the forward's own error. */
+ * library's per-stream buffer (same rules as the forward).  Unlike the pair handed to cuDNN, O and
+ * Stats may come from the quantized forward: the probabilities recomputed here are then not quite
+ * the ones O and Stats belong to, and a row of dS no longer sums to zero exactly.  dQ is therefore
+ * taken as scale * dS (K - c) with c close to the mean key — the same value for a consistent
+ * forward, and free of the keys' common offset times that row sum otherwise. */
 size_t mi355_sage_bwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D);
 int mi355_sage_sdpa_bwd_bf16(
     const void* Q, const void* K, const void* V, const void* O, const void* dO, const void* Stats,

@@ -10,7 +10,8 @@
 //   1. bwd_prep_kernel     Delta and Stats * log2(e) per query row (padding rows: +inf, so their
 //                          probabilities vanish), and transposed copies K^T, Q^T, dO^T in tiles of
 //                          64 rows whose rows sit in the slot order of the matrix instruction's
-//                          operand layout (v_slot_f16).
+//                          operand layout (v_slot_f16).  K^T holds the keys minus (nearly) their
+//                          mean: dQ = scale * dS (K - c) for any constant vector c.
 //   2. bwd_pass_kernel<0>  owner = 256 query rows per workgroup (8 waves), loop over key tiles  -> dQ
 //   3. bwd_pass_kernel<1>  owner = 128 keys per workgroup (4 waves), loop over query tiles     -> dK, dV
 // In both passes a wave owns 32 rows ("x"), keeps their two bf16 row blocks resident as B operands
@@ -89,6 +90,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
     constexpr int CPR = D / 8;
     constexpr int LROW = D + 8;                     // LDS row stride in elements (keeps 16-byte alignment, spreads banks)
     __shared__ __attribute__((aligned(16))) uint16_t tile[64 * LROW];
+    __shared__ float kcen[D];
     const int ntk = (int)(a.nkv_pad / 64), ntq = (int)(a.nq_pad / 64);
     const int per_bh = ntk + 3 * ntq;
     const int bh = blockIdx.x / per_bh;
@@ -131,16 +133,55 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
     uint16_t* dst;
     int valid, t;
     int64_t ntiles;
+    const bool centre = r < ntk;
     if (r < ntk) { src = a.k; dst = a.kT; valid = a.valid_kv; t = r; ntiles = ntk; }
     else if (r < ntk + ntq) { src = a.q; dst = a.qT; valid = a.valid_q; t = r - ntk; ntiles = ntq; }
     else { src = a.dout; dst = a.doT; valid = a.valid_q; t = r - ntk - ntq; ntiles = ntq; }
     const uint16_t* sp = src.p + b * src.sb + h * src.sh;
+    // K^T holds the keys minus a vector close to their mean (the mean of 64 keys spread evenly over
+    // the valid ones, the same in every workgroup of the head): rows of dS sum to zero, so dS K is
+    // unchanged by it in exact arithmetic, and when O and Stats come from a forward of other
+    // precision the small non-zero row sum is no longer multiplied by the keys' common offset.
+    if (centre) {
+        float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 64 * CPR / 256; i++) {
+            const int c = i * 256 + tid;
+            const int smp = c / CPR, col = (c % CPR) * 8;
+            const int64_t key = ((int64_t)smp * valid) >> 6;
+            const u32x4 w = *reinterpret_cast<const u32x4*>(sp + key * src.sn + col);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                part[2 * e] += __uint_as_float(w[e] << 16);
+                part[2 * e + 1] += __uint_as_float(w[e] & 0xFFFF0000u);
+            }
+        }
+        // thread tid holds samples {tid / CPR + k * (256 / CPR)} of chunk tid % CPR: reduce over tid / CPR
+        float* red = reinterpret_cast<float*>(tile);                 // [256 / CPR][D]
+#pragma unroll
+        for (int e = 0; e < 8; e++) red[(tid / CPR) * D + (tid % CPR) * 8 + e] = part[e];
+        __syncthreads();
+        float sum = 0.0f;
+        if (tid < D)
+            for (int g = 0; g < 256 / CPR; g++) sum += red[g * D + tid];
+        __syncthreads();
+        if (tid < D) kcen[tid] = sum * (1.0f / 64.0f);
+        __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < 64 * CPR / 256; i++) {
         const int c = i * 256 + tid;
         const int row = c / CPR, col = (c % CPR) * 8;
         u32x4 w = {0u, 0u, 0u, 0u};
-        if (t * 64 + row < valid) w = *reinterpret_cast<const u32x4*>(sp + (int64_t)(t * 64 + row) * src.sn + col);
+        if (t * 64 + row < valid) {
+            w = *reinterpret_cast<const u32x4*>(sp + (int64_t)(t * 64 + row) * src.sn + col);
+            if (centre) {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    w[e] = pack_bf16(__uint_as_float(w[e] << 16) - kcen[col + 2 * e],
+                                     __uint_as_float(w[e] & 0xFFFF0000u) - kcen[col + 2 * e + 1]);
+            }
+        }
         *reinterpret_cast<u32x4*>(&tile[row * LROW + col]) = w;
     }
     __syncthreads();

@@ -265,7 +265,11 @@ int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, 
  * with both given (the flash interface of ops/cshim/cudnn_sdpa_bwd.cpp:325-347) they are
  * attn = exp(score - stats[row]) with the caller's log-sum-exp, and rowsum(dA * attn) is taken as
  * rowsum(dO * O) — equal in exact arithmetic, and what a kernel that never holds a whole row has
- * to use.  Query rows >= real_nq and keys >= real_nkv are padding: they take no part and their
+ * to use.  In that form dQ = scale * dS (K - kbar) with kbar the mean of the valid keys: a row of
+ * dS sums to zero when O and stats belong to these probabilities, so any constant vector may be
+ * taken off the keys; when they come from a forward of other precision (the quantized one) the
+ * row sum is a small non-zero number and the uncentred product would multiply it by the keys'
+ * common offset.  Query rows >= real_nq and keys >= real_nkv are padding: they take no part and their
  * gradient rows are zero (cudnn_sdpa_bwd.cpp:344 real_N_q / real_N_kv). */
 int sage_oracle_sdpa_bwd_f32(const float* q, const float* k, const float* v, const float* o,
                              const float* dout, const float* stats,
@@ -282,13 +286,20 @@ int sage_oracle_sdpa_bwd_f32(const float* q, const float* k, const float* v, con
     const int nk = real_nkv > 0 && real_nkv < Nkv ? real_nkv : Nkv;
     double* P = (double*)malloc(sizeof(double) * (size_t)nq * (size_t)nk);
     double* dS = (double*)malloc(sizeof(double) * (size_t)nq * (size_t)nk);
-    if (!P || !dS) { free(P); free(dS); return -1; }
+    double* kbar = (double*)malloc(sizeof(double) * (size_t)D);
+    if (!P || !dS || !kbar) { free(P); free(dS); free(kbar); return -1; }
     for (int b = 0; b < B; b++)
         for (int h = 0; h < H; h++) {
             const float* qb = q + b * qs[0] + h * qs[1];
             const float* kb = k + b * ks[0] + h * ks[1];
             const float* vb = v + b * vs[0] + h * vs[1];
             const float* gb = dout + b * dos[0] + h * dos[1];
+            for (int d = 0; d < D; d++) {
+                double m = 0.0;
+                if (stats)
+                    for (int j = 0; j < nk; j++) m += (double)kb[j * ks[2] + d * ks[3]];
+                kbar[d] = m / (double)nk;
+            }
 #pragma omp parallel for schedule(dynamic, 8)
             for (int i = 0; i < nq; i++) {
                 const float* qr = qb + i * qs[2];
@@ -325,7 +336,7 @@ int sage_oracle_sdpa_bwd_f32(const float* q, const float* k, const float* v, con
                 float* dqr = dq + b * dqs[0] + h * dqs[1] + i * dqs[2];
                 for (int d = 0; d < D; d++) {
                     double a = 0.0;
-                    for (int j = 0; j < nk; j++) a += Sr[j] * (double)kb[j * ks[2] + d * ks[3]];
+                    for (int j = 0; j < nk; j++) a += Sr[j] * ((double)kb[j * ks[2] + d * ks[3]] - kbar[d]);
                     dqr[d * dqs[3]] = (float)(a * (double)scale);
                 }
             }
@@ -353,6 +364,7 @@ int sage_oracle_sdpa_bwd_f32(const float* q, const float* k, const float* v, con
         }
     free(P);
     free(dS);
+    free(kbar);
     return 0;
 }
 

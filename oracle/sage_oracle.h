@@ -85,7 +85,10 @@ int sage_oracle_sdpa_online_f32(const float* q, const float* k, const float* v, 
  * o == stats == NULL: probabilities recomputed from q, k (the torch.autograd reference of
  * ops/parity/sdpa_bwd_oracle.py:56-63).  Both given: the flash interface of
  * ops/cshim/cudnn_sdpa_bwd.cpp:325-347 — attn = exp(score - stats[row]) and the softmax-backward
- * row term is rowsum(dO * O).  stats contiguous [B,H,Nq] (natural log).  Rows >= real_nq and keys
+ * row term is rowsum(dO * O), and dQ is taken with the keys centred on their mean (a row of dS sums
+ * to zero for consistent O and stats, so this changes nothing then; it keeps a small inconsistency
+ * of a lower-precision forward from being multiplied by the keys' common offset).
+ * stats contiguous [B,H,Nq] (natural log).  Rows >= real_nq and keys
  * >= real_nkv (0: all) are padding; their gradients are zero.  Pinned by the reference's golden
  * gradients ops/parity/sdpa_bwd_ref.txt, torch.autograd in float64, central differences, and the
  * invariance of attention to a common shift of all keys (sum over keys of dK is zero). */

@@ -166,6 +166,24 @@ def test_bwd_after_the_quantized_forward():
         b = ref.reshape(-1).double()
         cos = float(a @ b / (a.norm() * b.norm()))
         assert cos >= 0.999, (name, cos)
+    # keys with a large common offset (workload 2's K ~ N(offset, 1), offset ~ N(0, 4^2) per channel):
+    # the rows of dS do not sum to zero exactly when O and Stats come from the quantized forward, and
+    # only the centred keys in dQ = scale * dS (K - c) keep that from being multiplied by the offset
+    from mojodiffusion_amd.workloads import WORKLOADS, make_inputs, bf16_bits_to_f32
+    w = WORKLOADS[2].scaled(B=1, H=3, S=700)
+    qb, kb, vb = make_inputs(w)
+    dev = lambda x: torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16)
+    qd, kd, vd = dev(qb), dev(kb), dev(vb)
+    gd = torch.randn(qd.shape, device="cuda", generator=gen).to(torch.bfloat16)
+    f = attention_sage.sdpa_flash_train_fwd(qd, kd, vd, w.scale)
+    gr = attention_sage.sdpa_flash_backward(f, gd, w.scale)
+    Q, K, V = (t.float().permute(0, 2, 1, 3).detach().requires_grad_(True) for t in (qd, kd, vd))
+    (torch.softmax(w.scale * Q @ K.transpose(-1, -2), dim=-1) @ V).backward(gd.float().permute(0, 2, 1, 3))
+    for name, got, ref in (("dQ", gr.d_q, Q.grad), ("dK", gr.d_k, K.grad), ("dV", gr.d_v, V.grad)):
+        a = got.float().permute(0, 2, 1, 3).reshape(-1).double()
+        b2 = ref.reshape(-1).double()
+        cos = float(a @ b2 / (a.norm() * b2.norm()))
+        assert cos >= 0.9995, ("offset keys", name, cos)
     # F32 boundary (attention_flash.mojo:478-535) on an aligned length
     S2 = 1280
     q2, k2, v2 = (torch.randn((B, S2, H, D), device="cuda", generator=gen) for _ in range(3))
@@ -175,6 +193,44 @@ def test_bwd_after_the_quantized_forward():
     # probabilities of a row sum to one: with dO = 1 every dV row sums (over keys) to S2 per channel
     colsum = g2.d_v.sum(dim=1)
     assert torch.allclose(colsum, torch.full_like(colsum, float(S2)), rtol=2e-2)
+
+
+def test_bwd_in_a_captured_graph(oracle):
+    """With a caller workspace the three launches allocate nothing and use no memset: captured into
+    a HIP graph and replayed with other work in between, every replay gives the eager bits."""
+    B, S, H, D = 1, 200, 2, 128
+    scale = 0.09
+    rng = np.random.default_rng(31)
+    q, k, v, g = (_bf16_round(rng.standard_normal((B, S, H, D))).cuda() for _ in range(4))
+    fwd = attention_sage.sdpa_flash_train_fwd(q, k, v, scale)
+    L = _lib.lib()
+    ws = torch.empty(L.mi355_sage_bwd_workspace_bytes(B, H, S, S, D), dtype=torch.uint8, device="cuda")
+    st = _lib.strides_bhnd(S, H, D)
+    outs = [torch.empty_like(q) for _ in range(3)]
+    stats = fwd.stats.contiguous()
+
+    def call(stream):
+        rc = L.mi355_sage_sdpa_bwd_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), fwd.o.data_ptr(), g.data_ptr(), stats.data_ptr(),
+                                        outs[0].data_ptr(), outs[1].data_ptr(), outs[2].data_ptr(), B, H, S, S, D, scale,
+                                        *([st] * 8), 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, stream, ws.data_ptr(), ws.numel())
+        assert rc == 0, rc
+    call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    eager = [o.clone() for o in outs]
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(side.cuda_stream)
+    for rep in range(3):
+        for o in outs:
+            o.fill_(float(rep))
+        ws.random_(0, 255)                               # the workspace holds nothing between calls
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, e in zip(outs, eager):
+            assert torch.equal(o.view(torch.int16), e.view(torch.int16)), rep
 
 
 def test_bwd_argument_errors():

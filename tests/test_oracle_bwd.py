@@ -146,3 +146,31 @@ def test_valid_lengths(oracle):
     got2 = oracle.sdpa_bwd_f32(q, k, v, g, scale, o=o, stats=stats, real_nq=nq, real_nkv=nk)
     for a, b in zip(got2, want):
         np.testing.assert_allclose(a, b, atol=3e-6, rtol=1e-5)
+
+
+def test_flash_form_after_the_quantized_forward(oracle):
+    """O and stats from the quantized forward are consistent with ITS probabilities, not with the
+    exact ones the backward recomputes: the rows of dS then sum to a small non-zero number.  With keys
+    that share a large offset (workload 2) the uncentred dS K would multiply that number by the offset
+    (cosine of dQ against the exact gradient 0.9987); centred keys keep every gradient at 0.9999."""
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    from mojodiffusion_amd.workloads import WORKLOADS, make_inputs, bf16_bits_to_f32
+    w = WORKLOADS[2].scaled(B=1, H=2, S=320)
+    q, k, v = make_inputs(w)
+    qf, kf, vf = (bf16_bits_to_f32(t) for t in (q, k, v))
+    g = np.random.default_rng(3).standard_normal(q.shape).astype(np.float32)
+    ob, _, stats = oracle.sdpa_bf16(q, k, v, w.scale, variant=0, blkq=128, blkk=64, want_stats=True)
+    exact = oracle.sdpa_bwd_f32(qf, kf, vf, g, w.scale)
+    got = oracle.sdpa_bwd_f32(qf, kf, vf, g, w.scale, o=bf16_bits_to_f32(ob), stats=stats)
+    for a, b in zip(got, exact):
+        a, b = a.astype(np.float64).reshape(-1), b.astype(np.float64).reshape(-1)
+        assert a @ b / np.sqrt((a @ a) * (b @ b)) >= 0.9999
+    # the uncentred product, written out here, is what loses it
+    s = w.scale * np.einsum("bihd,bjhd->bhij", qf.astype(np.float64), kf.astype(np.float64))
+    P = np.exp(s - stats[..., None].astype(np.float64))
+    dP = np.einsum("bihd,bjhd->bhij", g.astype(np.float64), vf.astype(np.float64))
+    delta = np.einsum("bihd,bihd->bhi", g.astype(np.float64), bf16_bits_to_f32(ob).astype(np.float64))
+    dq = w.scale * np.einsum("bhij,bjhd->bihd", P * (dP - delta[..., None]), kf.astype(np.float64)).reshape(-1)
+    e = exact[0].astype(np.float64).reshape(-1)
+    assert dq @ e / np.sqrt((dq @ dq) * (e @ e)) < 0.9995
