@@ -45,6 +45,11 @@ extern "C" {
 #define MI355_SAGE_K_SMOOTH  1   /* subtract the per-channel mean of K over the keys          */
 #define MI355_SAGE_ROPE_INTERLEAVED 0   /* pairs (x[2i], x[2i+1]): serenitymojo/ops/rope.mojo:7-9 (FLUX, Klein, Z-Image) */
 #define MI355_SAGE_ROPE_HALFSPLIT   1   /* pairs (x[i], x[i+D/2]): serenitymojo/ops/rope.mojo:10-13 (Anima, Hunyuan, LTX-2 ...) */
+/* two more bits of the same argument (rope_layout): */
+#define MI355_SAGE_ROPE_TABLES_BF16 2   /* rope_cos / rope_sin hold bf16 (rope.mojo:147-165 casts them to fp32) */
+#define MI355_SAGE_NORM_FULL_ROW    4   /* the RMSNorm runs over all H*D channels of a token, q_gain / k_gain have H*D
+                                           entries (channel h*D + d): rms_norm on [S, H*D] before the reshape to heads,
+                                           serenitymojo/models/ltx2/ltx2_block.mojo:419-432 */
 #define MI355_SAGE_K_BALANCE 2   /* per channel d: K / s_d, Q * s_d with s_d = sqrt(max|K - mean|)
                                     over the keys: scores are unchanged, and a channel whose
                                     range is r times the others' costs each side sqrt(r), not
@@ -273,8 +278,10 @@ int mi355_sage_quant_qk_bf16(
  * use the same table (self-attention positions), so with tables N_q must equal N_kv (-2
  * otherwise).  rope_layout: MI355_SAGE_ROPE_INTERLEAVED, or MI355_SAGE_ROPE_HALFSPLIT for the
  * pairing (i, i + D/2) of rope_halfsplit (serenitymojo/ops/rope.mojo:147-165; per-head norm +
- * half-split rotation as in serenitymojo/models/anima/block.mojo:360-366); ignored without tables.
- * Gains and tables must be 16-byte aligned. */
+ * half-split rotation as in serenitymojo/models/anima/block.mojo:360-366), optionally ORed with
+ * MI355_SAGE_ROPE_TABLES_BF16 and MI355_SAGE_NORM_FULL_ROW (LTX-2's sequence: RMSNorm over the whole
+ * inner dim, half-split rotation with bf16 tables; that statistic takes one more launch and, like
+ * the tables, needs N_q == N_kv).  Gains and tables must be 16-byte aligned. */
 int mi355_sage_quant_qk_norm_rope_bf16(
     const void* Q, const void* K,
     int B, int H, int N_q, int N_kv, int D, float scale,

@@ -56,6 +56,8 @@ K_SMOOTH = 1
 K_BALANCE = 2
 ROPE_INTERLEAVED = 0
 ROPE_HALFSPLIT = 1
+ROPE_TABLES_BF16 = 2
+NORM_FULL_ROW = 4
 
 _lib = None
 

@@ -404,21 +404,25 @@ def sdpa_nomask_slab(q, k, v, scale, slab, variant=PV_FP16):
     return o
 
 
-def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin):
+def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin, halfsplit=False, full_row=False):
     _check_shapes(name, q_pre, k_pre, v, True)
     _require_bf16(name, q_pre, k_pre, v)
     _require_cuda(name, q_pre, k_pre, v)
     B, S, H, Dh = q_pre.shape
-    if q_norm.numel() != Dh or k_norm.numel() != Dh:
-        raise Error("%s: weight must be [%d]" % (name, Dh))
+    cols = H * Dh if full_row else Dh
+    if q_norm.numel() != cols or k_norm.numel() != cols:
+        raise Error("%s: weight must be [%d]" % (name, cols))
+    flags = (_lib.ROPE_HALFSPLIT if halfsplit else 0) | (_lib.NORM_FULL_ROW if full_row else 0)
     gq = q_norm.to(device=q_pre.device, dtype=torch.bfloat16).contiguous()
     gk = k_norm.to(device=q_pre.device, dtype=torch.bfloat16).contiguous()
     batch_rows = 0
     if (cos is None) != (sin is None):
         raise Error("%s: cos and sin come together" % name)
     if cos is not None:
-        if cos.dtype != torch.float32 or sin.dtype != torch.float32:
-            raise Error("%s: cos/sin tables must be F32" % name)
+        if cos.dtype != sin.dtype or cos.dtype not in (torch.float32, torch.bfloat16):
+            raise Error("%s: cos/sin tables must be F32 (or both BF16)" % name)
+        if cos.dtype == torch.bfloat16:
+            flags |= _lib.ROPE_TABLES_BF16
         if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != Dh // 2:
             raise Error("%s: cos/sin must be [rows, D/2]" % name)
         if cos.shape[0] == B * S * H and B > 1:
@@ -426,11 +430,12 @@ def _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin):
         elif cos.shape[0] != S * H:
             raise Error("%s: cos/sin rows must be S*H (or B*S*H)" % name)
         cos, sin = cos.contiguous(), sin.contiguous()
-    return gq, gk, cos, sin, batch_rows
+    return gq, gk, cos, sin, batch_rows, flags
 
 
 def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16,
-                             blkq=None, blkk=64, k_flags=_lib.K_SMOOTH | _lib.K_BALANCE, halfsplit=False):
+                             blkq=None, blkk=64, k_flags=_lib.K_SMOOTH | _lib.K_BALANCE, halfsplit=False,
+                             full_row=False):
     """The attention block of a DiT layer from the projections on, in one call:
 
         q = rope_interleaved(rms_norm(q_pre, q_norm, eps), cos, sin)
@@ -442,9 +447,11 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
     ops/norm.mojo:170-172 does when the gain's dtype differs); cos/sin: F32 [S*H, Dh/2]
     (sampling/klein_sampler.mojo:305-307) or [B*S*H, Dh/2], or None for norm only.
     halfsplit: rope_halfsplit instead of rope_interleaved (ops/rope.mojo:10-13; the per-head norm +
-    half-split rotation of models/anima/block.mojo:360-366)."""
+    half-split rotation of models/anima/block.mojo:360-366).  full_row: the RMSNorm runs over the
+    whole inner dim, q_norm/k_norm are [H*Dh] (rms_norm on [S, H*Dh] before the reshape to heads,
+    models/ltx2/ltx2_block.mojo:419-432, whose tables are BF16 — also accepted)."""
     name = "qk_norm_rope_sdpa_nomask"
-    gq, gk, cos, sin, batch_rows = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin)
+    gq, gk, cos, sin, batch_rows, flags = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin, halfsplit, full_row)
     B, S, H, Dh = q_pre.shape
     L = _lib.lib()
     o = torch.empty_like(q_pre)
@@ -458,20 +465,20 @@ def qk_norm_rope_sdpa_nomask(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, sca
         st, st, st, st, 0, 0, 0, 0, 0, torch.cuda.current_stream(q_pre.device).cuda_stream,
         variant, blkq, blkk, int(k_flags), gq.data_ptr(), gk.data_ptr(), float(eps),
         cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
-        _lib.ROPE_HALFSPLIT if halfsplit else _lib.ROPE_INTERLEAVED, ws.data_ptr(), ws.numel())
+        flags, ws.data_ptr(), ws.numel())
     if rc != 0:
         raise Error("%s: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (name, rc, B, S, H, Dh))
     return o
 
 
 def qk_norm_rope_sdpa_flash_train_fwd(q_pre, k_pre, v, q_norm, k_norm, eps, cos, sin, scale, variant=PV_FP16,
-                                      halfsplit=False):
+                                      halfsplit=False, full_row=False):
     """The same block where the caller keeps the attention statistics for a backward pass:
     rms_norm / rope_interleaved followed by sdpa_flash_train_fwd
     (serenitymojo/ops/attention_flash.mojo:149-202).  Returns an SdpaFlashFwd whose stats are the
     log-sum-exp of the normalised, rotated Q and K."""
     name = "qk_norm_rope_sdpa_flash_train_fwd"
-    gq, gk, cos, sin, batch_rows = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin)
+    gq, gk, cos, sin, batch_rows, flags = _norm_rope_args(name, q_pre, k_pre, v, q_norm, k_norm, cos, sin, halfsplit, full_row)
     B, S, H, Dh = q_pre.shape
     L = _lib.lib()
     o = torch.empty_like(q_pre)
@@ -484,7 +491,7 @@ def qk_norm_rope_sdpa_flash_train_fwd(q_pre, k_pre, v, q_norm, k_norm, eps, cos,
         st, st, st, st, 0, 0, 0, 0, 0, 0, S, S, torch.cuda.current_stream(q_pre.device).cuda_stream,
         variant, gq.data_ptr(), gk.data_ptr(), float(eps),
         cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None, batch_rows,
-        _lib.ROPE_HALFSPLIT if halfsplit else _lib.ROPE_INTERLEAVED, ws.data_ptr(), ws.numel())
+        flags, ws.data_ptr(), ws.numel())
     if rc != 0:
         raise Error("%s: shim rc=%d (B=%d S=%d H=%d Dh=%d)" % (name, rc, B, S, H, Dh))
     return SdpaFlashFwd(o, o, q_pre, k_pre, v, stats)

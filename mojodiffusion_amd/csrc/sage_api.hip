@@ -70,7 +70,7 @@ int check_kv_len(int N_kv, int blkk) {
 
 // Workspace layout of the one-shot calls.
 struct Carve {
-    size_t q8, k8, vq, qscale, kscale, kmean, qmul, kmul, vscale, kpart_sum, kpart_mm, vpart, qshift, total;
+    size_t q8, k8, vq, qscale, kscale, kmean, qmul, kmul, vscale, kpart_sum, kpart_mm, vpart, qshift, rowinv_q, rowinv_k, total;
 };
 
 Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
@@ -93,13 +93,15 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.kpart_mm = take(bh * ng * D * 2 * sizeof(float));
     c.vpart = take(variant == MI355_SAGE_PV_FP16 ? 0 : bh * ng * D * sizeof(float));
     c.qshift = take(bh * nqp * sizeof(float));
+    c.rowinv_q = take((size_t)B * Nq * sizeof(float));        // whole-row RMSNorm statistic per token (optional pre-op)
+    c.rowinv_k = take((size_t)B * Nkv * sizeof(float));
     c.total = off;
     return c;
 }
 
 // Scratch of the stage quantizers: K group sums and minima / maxima, V group maxima.
 struct ScratchCarve {
-    size_t kpart_sum, kpart_mm, vpart, total;
+    size_t kpart_sum, kpart_mm, vpart, rowinv_q, rowinv_k, total;
 };
 ScratchCarve scratch_carve(int B, int H, int Nkv, int D) {
     const size_t n = (size_t)B * H * ((Nkv + kGroup - 1) / kGroup) * D;
@@ -107,7 +109,10 @@ ScratchCarve scratch_carve(int B, int H, int Nkv, int D) {
     c.kpart_sum = 0;
     c.kpart_mm = align_up(n * sizeof(double));
     c.vpart = c.kpart_mm + align_up(n * 2 * sizeof(float));
-    c.total = c.vpart + align_up(n * sizeof(float));
+    // whole-row RMSNorm statistics (that pre-op needs N_q == N_kv)
+    c.rowinv_q = c.vpart + align_up(n * sizeof(float));
+    c.rowinv_k = c.rowinv_q + align_up((size_t)B * Nkv * sizeof(float));
+    c.total = c.rowinv_k + align_up((size_t)B * Nkv * sizeof(float));
     return c;
 }
 
@@ -154,6 +159,7 @@ int internal_workspace(size_t need, hipStream_t stream, void** out) {
 // The optional ops in front of the quantizers (RMSNorm + interleaved RoPE of Q and of K).
 struct Pre {
     PreOp q{}, k{};
+    bool full_row = false;      // RMSNorm over all H*D channels of a token (gains of H*D entries)
 };
 
 // q_gain / k_gain null together = nothing to do.  Tables are optional on top of the gains.
@@ -164,12 +170,14 @@ int make_pre(const void* q_gain, const void* k_gain, float eps, const void* rope
     if (!q_gain || !k_gain) { SAGE_LOG("RMSNorm gains must be given for both Q and K"); return MI355_SAGE_EINVAL; }
     if ((rope_cos == nullptr) != (rope_sin == nullptr)) return MI355_SAGE_EINVAL;
     if (!(eps >= 0.0f) || rope_batch_rows < 0) return MI355_SAGE_EINVAL;
-    if (rope_layout != MI355_SAGE_ROPE_INTERLEAVED && rope_layout != MI355_SAGE_ROPE_HALFSPLIT) return MI355_SAGE_EINVAL;
+    if (rope_layout & ~(MI355_SAGE_ROPE_HALFSPLIT | MI355_SAGE_ROPE_TABLES_BF16 | MI355_SAGE_NORM_FULL_ROW)) return MI355_SAGE_EINVAL;
     const uintptr_t bits = reinterpret_cast<uintptr_t>(q_gain) | reinterpret_cast<uintptr_t>(k_gain) |
                            reinterpret_cast<uintptr_t>(rope_cos) | reinterpret_cast<uintptr_t>(rope_sin);
     if (bits & 15) { SAGE_LOG("gains and RoPE tables must be 16-byte aligned"); return MI355_SAGE_EUNSUPPORTED; }
     out->q = PreOp{static_cast<const uint16_t*>(q_gain), eps, static_cast<const float*>(rope_cos),
-                   static_cast<const float*>(rope_sin), rope_batch_rows, rope_layout == MI355_SAGE_ROPE_HALFSPLIT ? 1 : 0};
+                   static_cast<const float*>(rope_sin), rope_batch_rows, (rope_layout & MI355_SAGE_ROPE_HALFSPLIT) ? 1 : 0,
+                   (rope_layout & MI355_SAGE_ROPE_TABLES_BF16) ? 1 : 0, nullptr, 0};
+    out->full_row = (rope_layout & MI355_SAGE_NORM_FULL_ROW) != 0;
     out->k = out->q;
     out->k.gain = static_cast<const uint16_t*>(k_gain);
     return 0;
@@ -209,12 +217,19 @@ struct QuantOut {
     float *kmean, *qmul, *kmul;
     double* kpart_sum; float* kpart_mm;
     float* rowdot;
+    float *rowinv_q, *rowinv_k;       // whole-row RMSNorm statistics (only with that pre-op)
 };
 
 // K statistics + Q / K encoders (+ the V passes when vq is given): launches 1-3.
 int quantize(const View& q, const View& k, const View* v, int B, int H, int Nq, int Nkv, int D, float scale,
              int blkq, int blkk, int k_flags, const KeyMask& km, int kept, const QuantOut& o,
-             int variant, void* vq, float* vscale, float* vpart, const Pre& pre, hipStream_t st) {
+             int variant, void* vq, float* vscale, float* vpart, const Pre& pre_in, hipStream_t st) {
+    Pre pre = pre_in;
+    if (pre.full_row) {
+        SAGE_HIP(launch_row_inv(q, k, B, H, Nq, Nkv, D, pre.q.eps, o.rowinv_q, o.rowinv_k, st));
+        pre.q.row_inv = o.rowinv_q; pre.q.row_n = Nq;
+        pre.k.row_inv = o.rowinv_k; pre.k.row_n = Nkv;
+    }
     const float cmul = cmul_of(scale);
     const int64_t nqp = pad_to(Nq, kTileQ), nkp = pad_to(Nkv, kPadKV);
     const bool kstats = (k_flags & 3) != 0;
@@ -278,8 +293,8 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if ((rc = check_view("Q", Q, qs, q_off)) || (rc = check_view("K", K, ks, k_off)) ||
         (rc = check_view("V", V, vs, v_off)) || (rc = check_view("O", O, os, o_off)))
         return rc;
-    if (pre.q.gain != nullptr && pre.q.cos != nullptr && N_q != N_kv) {
-        SAGE_LOG("fused RoPE uses one table row per position of Q and K alike: N_q must equal N_kv");
+    if (pre.q.gain != nullptr && (pre.q.cos != nullptr || pre.full_row) && N_q != N_kv) {
+        SAGE_LOG("fused RoPE / whole-row RMSNorm are self-attention pre-ops: N_q must equal N_kv");
         return MI355_SAGE_EUNSUPPORTED;
     }
     if (mask.add != nullptr) {
@@ -322,6 +337,8 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     o.kmul = reinterpret_cast<float*>(ws + c.kmul);
     o.kpart_sum = reinterpret_cast<double*>(ws + c.kpart_sum);
     o.kpart_mm = reinterpret_cast<float*>(ws + c.kpart_mm);
+    o.rowinv_q = reinterpret_cast<float*>(ws + c.rowinv_q);
+    o.rowinv_k = reinterpret_cast<float*>(ws + c.rowinv_k);
     // Stats needs <q, kmean> per row: K smoothing lowers every score of a row by it
     float* qshift = (Stats && (k_flags & MI355_SAGE_K_SMOOTH)) ? reinterpret_cast<float*>(ws + c.qshift) : nullptr;
     o.rowdot = qshift;
@@ -487,7 +504,8 @@ static int quant_qk_entry(const void* Q, const void* K, int B, int H, int N_q, i
     if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk) || (k_flags & ~3)) return MI355_SAGE_EUNSUPPORTED;
     const ScratchCarve sc = scratch_carve(B, H, N_kv, D);
     if ((k_flags & 3) && scratch_bytes < sc.total) return MI355_SAGE_EWORKSPACE;
-    if (pre.q.gain != nullptr && pre.q.cos != nullptr && N_q != N_kv) return MI355_SAGE_EUNSUPPORTED;
+    if (pre.q.gain != nullptr && (pre.q.cos != nullptr || pre.full_row) && N_q != N_kv) return MI355_SAGE_EUNSUPPORTED;
+    if (pre.full_row && (!scratch || scratch_bytes < sc.total)) return MI355_SAGE_EWORKSPACE;
     int rc;
     if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off))) return rc;
     KeyMask km;
@@ -499,6 +517,8 @@ static int quant_qk_entry(const void* Q, const void* K, int B, int H, int N_q, i
     o.kmean = static_cast<float*>(kmean); o.qmul = static_cast<float*>(qmul); o.kmul = static_cast<float*>(kmul);
     o.kpart_sum = reinterpret_cast<double*>(static_cast<uint8_t*>(scratch) + sc.kpart_sum);
     o.kpart_mm = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + sc.kpart_mm);
+    o.rowinv_q = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + sc.rowinv_q);
+    o.rowinv_k = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + sc.rowinv_k);
     return quantize(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), nullptr, B, H, N_q, N_kv, D,
                     scale, blkq, blkk, k_flags, km, kept, o, 0, nullptr, nullptr, nullptr, pre,
                     static_cast<hipStream_t>(stream));

@@ -33,6 +33,9 @@ struct PreOp {
     const float* sin;
     int64_t batch_rows;          // 0: all batches share the table
     int halfsplit;               // 0: pairs (2i, 2i+1) (ops/rope.mojo:7-9); 1: pairs (i, i + D/2) (ops/rope.mojo:10-13)
+    int tables_bf16;             // the tables hold bf16 instead of fp32
+    const float* row_inv;        // [B, row_n]: 1/sqrt(mean over all H*D channels + eps) per token; null: the
+    int64_t row_n;               //   statistic is taken per head over D.  With it the gain has H*D entries.
 };
 
 // Keys lo <= s < hi take no part (statistics, scale blocks, scores); lo >= hi: no such range.
@@ -56,6 +59,12 @@ struct PrepArgs {
     int ngroups, nk_wg, nv_units;    // filled by the launcher
 };
 hipError_t launch_prep(const PrepArgs& a, int B, int D, hipStream_t st);
+
+// Launch 0 (only with a whole-row RMSNorm in front): 1/sqrt(mean(x^2) + eps) over all H*D channels
+// of every token of Q (rows [0, B*Nq)) and K (the rows after them), squares added in the order of
+// serenitymojo/ops/norm.mojo:56-72.
+hipError_t launch_row_inv(const View& q, const View& k, int B, int H, int Nq, int Nkv, int D, float eps,
+                          float* inv_q, float* inv_k, hipStream_t st);
 
 // Launch 2: per (b,h,channel) K mean and balancing factor, V scale.
 struct FinalArgs {

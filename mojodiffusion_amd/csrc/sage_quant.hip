@@ -80,8 +80,14 @@ __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, i
     sq[1] = sq[1] + sq[3];
     const float a = sq[0] + sq[1];
     const float mean = a / (float)D;
-    const float inv = 1.0f / sqrtf(mean + p.eps);
-    const u32x4 gw = *reinterpret_cast<const u32x4*>(p.gain + col);
+    float inv = 1.0f / sqrtf(mean + p.eps);
+    const uint16_t* gain = p.gain;
+    if (p.row_inv != nullptr) {
+        // the statistic of the whole token (all heads), computed by launch 0; gain of H*D entries
+        inv = valid ? p.row_inv[(int64_t)b * p.row_n + row] : 0.0f;
+        gain += h * D;
+    }
+    const u32x4 gw = *reinterpret_cast<const u32x4*>(gain + col);
     float g[8];
     unpack8(gw, g);
     float y[8];
@@ -102,12 +108,18 @@ __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, i
         for (int e = 0; e < 8; e++) cv[e] = 1.0f, sv[e] = 0.0f;
         if (valid) {
             const int64_t trow = (int64_t)b * p.batch_rows + (int64_t)row * H + h;
-            const float* pc = p.cos + trow * (D / 2) + (col & (D / 2 - 1));
-            const float* ps = p.sin + trow * (D / 2) + (col & (D / 2 - 1));
-            const float4 c0 = *reinterpret_cast<const float4*>(pc), c1 = *reinterpret_cast<const float4*>(pc + 4);
-            const float4 s0 = *reinterpret_cast<const float4*>(ps), s1 = *reinterpret_cast<const float4*>(ps + 4);
-            cv[0] = c0.x; cv[1] = c0.y; cv[2] = c0.z; cv[3] = c0.w; cv[4] = c1.x; cv[5] = c1.y; cv[6] = c1.z; cv[7] = c1.w;
-            sv[0] = s0.x; sv[1] = s0.y; sv[2] = s0.z; sv[3] = s0.w; sv[4] = s1.x; sv[5] = s1.y; sv[6] = s1.z; sv[7] = s1.w;
+            const int64_t ti = trow * (D / 2) + (col & (D / 2 - 1));
+            if (p.tables_bf16) {
+                unpack8(*reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.cos) + ti), cv);
+                unpack8(*reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.sin) + ti), sv);
+            } else {
+                const float* pc = p.cos + ti;
+                const float* ps = p.sin + ti;
+                const float4 c0 = *reinterpret_cast<const float4*>(pc), c1 = *reinterpret_cast<const float4*>(pc + 4);
+                const float4 s0 = *reinterpret_cast<const float4*>(ps), s1 = *reinterpret_cast<const float4*>(ps + 4);
+                cv[0] = c0.x; cv[1] = c0.y; cv[2] = c0.z; cv[3] = c0.w; cv[4] = c1.x; cv[5] = c1.y; cv[6] = c1.z; cv[7] = c1.w;
+                sv[0] = s0.x; sv[1] = s0.y; sv[2] = s0.z; sv[3] = s0.w; sv[4] = s1.x; sv[5] = s1.y; sv[6] = s1.z; sv[7] = s1.w;
+            }
         }
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -119,8 +131,15 @@ __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, i
         float4 c4 = {1.f, 1.f, 1.f, 1.f}, s4 = {0.f, 0.f, 0.f, 0.f};
         if (valid) {
             const int64_t trow = (int64_t)b * p.batch_rows + (int64_t)row * H + h;
-            c4 = *reinterpret_cast<const float4*>(p.cos + trow * (D / 2) + col / 2);
-            s4 = *reinterpret_cast<const float4*>(p.sin + trow * (D / 2) + col / 2);
+            if (p.tables_bf16) {
+                const u32x2 cw = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.cos) + trow * (D / 2) + col / 2);
+                const u32x2 sw = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p.sin) + trow * (D / 2) + col / 2);
+                c4 = float4{__uint_as_float(cw.x << 16), __uint_as_float(cw.x & 0xFFFF0000u), __uint_as_float(cw.y << 16), __uint_as_float(cw.y & 0xFFFF0000u)};
+                s4 = float4{__uint_as_float(sw.x << 16), __uint_as_float(sw.x & 0xFFFF0000u), __uint_as_float(sw.y << 16), __uint_as_float(sw.y & 0xFFFF0000u)};
+            } else {
+                c4 = *reinterpret_cast<const float4*>(p.cos + trow * (D / 2) + col / 2);
+                s4 = *reinterpret_cast<const float4*>(p.sin + trow * (D / 2) + col / 2);
+            }
         }
         const float cv[4] = {c4.x, c4.y, c4.z, c4.w}, sv[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
@@ -517,6 +536,50 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
         kstats_group_body<D, PRE>(g < a.ngroups ? g : -1, h, b, threadIdx.x % (16 * (D / 8)), a.k.p, a.k.sb, a.k.sh,
                                   a.k.sn, a.Nkv, a.H, a.ngroups, a.km, a.kpart_sum, a.kpart_mm, sm.kg[sub], a.pre_k);
     }
+}
+
+// ---------------------------------------------------------------------------
+// Launch 0: whole-row RMSNorm statistic.  One workgroup of 256 threads per token, exactly the
+// reference's reduction (serenitymojo/ops/norm.mojo:56-72): thread t adds the squares of
+// channels t, t+256, ... in turn (multiply and add rounded separately), then the 256 partial
+// sums fold in halves through LDS, far pairs first.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void row_inv_kernel(View q, View k, int H, int Nq, int Nkv, int D, int rows_q, float eps,
+                                                      float* __restrict__ inv_q, float* __restrict__ inv_k) {
+    __shared__ float part[256];
+    const int tid = threadIdx.x;
+    int r = blockIdx.x;
+    const bool is_k = r >= rows_q;
+    if (is_k) r -= rows_q;
+    const View& x = is_k ? k : q;
+    const int N = is_k ? Nkv : Nq;
+    const int b = r / N, n = r % N;
+    const uint16_t* row = x.p + b * x.sb + (int64_t)n * x.sn;
+    const int cols = H * D;
+    float local = 0.0f;
+    for (int c = tid; c < cols; c += 256) {
+        const float v = __uint_as_float((uint32_t)row[(int64_t)(c / D) * x.sh + (c % D)] << 16);
+        const float sq = v * v;
+        local = local + sq;
+    }
+    part[tid] = local;
+    __syncthreads();
+    for (int active = 128; active > 0; active >>= 1) {
+        if (tid < active) part[tid] = part[tid] + part[tid + active];
+        __syncthreads();
+    }
+    if (tid == 0) {
+        const float mean = part[0] / (float)cols;
+        (is_k ? inv_k : inv_q)[r] = 1.0f / sqrtf(mean + eps);
+    }
+}
+
+hipError_t launch_row_inv(const View& q, const View& k, int B, int H, int Nq, int Nkv, int D, float eps,
+                          float* inv_q, float* inv_k, hipStream_t st) {
+    const int64_t rows_q = (int64_t)B * Nq, rows = rows_q + (int64_t)B * Nkv;
+    if (rows > 0x7FFFFFFF) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(row_inv_kernel, dim3((unsigned)rows), dim3(256), 0, st, q, k, H, Nq, Nkv, D, (int)rows_q, eps, inv_q, inv_k);
+    return hipGetLastError();
 }
 
 hipError_t launch_prep(const PrepArgs& a_in, int B, int D, hipStream_t st) {

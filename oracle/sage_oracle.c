@@ -466,15 +466,36 @@ int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, co
     return sage_oracle_norm_rope_bf16_ex(x, B, H, N, D, st, gain, eps, cs, sn, table_batch_rows, 0, y);
 }
 
-/* rope_layout 0: interleaved pairs (rope.mojo:7-9); 1: half-split pairs (rope.mojo:10-13), the
- * per-head RMSNorm + rope_halfsplit sequence of serenitymojo/models/anima/block.mojo:360-366. */
+/* pre_flags: bit 0 — half-split pairs (rope.mojo:10-13) instead of interleaved ones (rope.mojo:7-9),
+ * the per-head RMSNorm + rope_halfsplit sequence of serenitymojo/models/anima/block.mojo:360-366;
+ * bit 1 — the tables are bf16 (the kernels cast them to fp32, rope.mojo:160-163);
+ * bit 2 — the RMSNorm runs over the whole row of H*D channels with a gain of H*D entries
+ * (channel h*D + d), the rms_norm on [S, H*D] before the reshape of
+ * serenitymojo/models/ltx2/ltx2_block.mojo:419-432. */
 int sage_oracle_norm_rope_bf16_ex(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
-                                  const uint16_t* gain, float eps, const float* cs, const float* sn,
-                                  int64_t table_batch_rows, int rope_layout, uint16_t* y) {
-    if (rope_layout != 0 && rope_layout != 1) return -1;
+                                  const uint16_t* gain, float eps, const void* cs, const void* sn,
+                                  int64_t table_batch_rows, int pre_flags, uint16_t* y) {
+    if (pre_flags & ~7) return -1;
     if (!x || !st || !gain || !y || B <= 0 || H <= 0 || N <= 0 || D <= 0 || (D & 1) || D > 1024) return -1;
     if ((cs == NULL) != (sn == NULL)) return -1;
+    const int halfsplit = pre_flags & 1, tab16 = pre_flags & 2, fullrow = pre_flags & 4;
     int half = D / 2;
+    /* whole-row statistic first (one value per token) */
+    float* row_inv = NULL;
+    if (fullrow) {
+        row_inv = (float*)malloc(sizeof(float) * (size_t)B * (size_t)N);
+        if (!row_inv) return -1;
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < (int64_t)B * N; r++) {
+            int n = (int)(r % N), b = (int)(r / N);
+            float* v = (float*)malloc(sizeof(float) * (size_t)H * (size_t)D);
+            for (int h = 0; h < H; h++)
+                for (int d = 0; d < D; d++)
+                    v[h * D + d] = sage_oracle_bf16_to_f32(x[b * st[0] + h * st[1] + (int64_t)n * st[2] + d * st[3]]);
+            row_inv[r] = rms_inv(v, H * D, eps);
+            free(v);
+        }
+    }
     int64_t work = (int64_t)B * N * H;
 #pragma omp parallel for schedule(static)
     for (int64_t w = 0; w < work; w++) {
@@ -484,19 +505,21 @@ int sage_oracle_norm_rope_bf16_ex(const uint16_t* x, int B, int H, int N, int D,
         float v[1024], t[1024];
         const uint16_t* src = x + b * st[0] + h * st[1] + (int64_t)n * st[2];
         for (int d = 0; d < D; d++) v[d] = sage_oracle_bf16_to_f32(src[d * st[3]]);
-        float inv = rms_inv(v, D, eps);
+        float inv = fullrow ? row_inv[(int64_t)b * N + n] : rms_inv(v, D, eps);
+        const uint16_t* gh = fullrow ? gain + (int64_t)h * D : gain;
         for (int d = 0; d < D; d++) {
             float a = v[d] * inv;
-            float gq = sage_oracle_bf16_to_f32(gain[d]);
+            float gq = sage_oracle_bf16_to_f32(gh[d]);
             t[d] = sage_oracle_bf16_to_f32(sage_oracle_f32_to_bf16(a * gq));
         }
         uint16_t* dst = y + (((int64_t)b * N + n) * H + h) * D;
         if (cs) {
             int64_t row = (int64_t)b * table_batch_rows + (int64_t)n * H + h;
             for (int i = 0; i < half; i++) {
-                int i0 = rope_layout ? i : 2 * i, i1 = rope_layout ? i + half : 2 * i + 1;
+                int i0 = halfsplit ? i : 2 * i, i1 = halfsplit ? i + half : 2 * i + 1;
                 float x0 = t[i0], x1 = t[i1];
-                float cv = cs[row * half + i], sv = sn[row * half + i];
+                float cv = tab16 ? sage_oracle_bf16_to_f32(((const uint16_t*)cs)[row * half + i]) : ((const float*)cs)[row * half + i];
+                float sv = tab16 ? sage_oracle_bf16_to_f32(((const uint16_t*)sn)[row * half + i]) : ((const float*)sn)[row * half + i];
                 float a = x0 * cv, bb = x1 * sv, c = x0 * sv, dd = x1 * cv;
                 dst[i0] = sage_oracle_f32_to_bf16(a - bb);
                 dst[i1] = sage_oracle_f32_to_bf16(c + dd);
@@ -505,6 +528,7 @@ int sage_oracle_norm_rope_bf16_ex(const uint16_t* x, int B, int H, int N, int D,
             for (int d = 0; d < D; d++) dst[d] = sage_oracle_f32_to_bf16(t[d]);
         }
     }
+    free(row_inv);
     return 0;
 }
 

@@ -119,11 +119,16 @@ int sage_oracle_rope_halfsplit_f32(const float* x, const float* cs, const float*
 int sage_oracle_norm_rope_bf16(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
                                const uint16_t* gain, float eps, const float* cs, const float* sn,
                                int64_t table_batch_rows, uint16_t* y);
-/* The same with the pairing chosen: rope_layout 0 interleaved, 1 half-split (the per-head
- * rms_norm -> rope_halfsplit sequence of serenitymojo/models/anima/block.mojo:360-366). */
+/* The same with options, pre_flags: bit 0 half-split pairing (rope.mojo:10-13; the per-head
+ * rms_norm -> rope_halfsplit sequence of serenitymojo/models/anima/block.mojo:360-366); bit 1 bf16
+ * tables (cs / sn point at uint16); bit 2 RMSNorm over the whole row of H*D channels with a gain
+ * of H*D entries (serenitymojo/models/ltx2/ltx2_block.mojo:419-432: rms_norm on [S, H*D], then
+ * the reshape to heads).  Wide rows accumulate `local += v*v` per thread (norm.mojo:62-65); whether
+ * the reference's compiler fuses that multiply-add is not visible in its text: parity unpinned
+ * for that bit, separately rounded here. */
 int sage_oracle_norm_rope_bf16_ex(const uint16_t* x, int B, int H, int N, int D, const int64_t* st,
-                                  const uint16_t* gain, float eps, const float* cs, const float* sn,
-                                  int64_t table_batch_rows, int rope_layout, uint16_t* y);
+                                  const uint16_t* gain, float eps, const void* cs, const void* sn,
+                                  int64_t table_batch_rows, int pre_flags, uint16_t* y);
 
 /* ---- quantizers --------------------------------------------------------- */
 /* Padded token count used by every quantized tensor: N rounded up to `mult`. */

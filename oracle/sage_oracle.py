@@ -272,26 +272,38 @@ def rope_halfsplit_f32(x, cos, sin):
     return out
 
 
-def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=0, halfsplit=False):
-    """x: uint16 [B,S,H,D] bf16 bits; gain: uint16 [D]; cos/sin: fp32 [rows, D/2] with row s*H + h
-    (plus b*table_batch_rows), or None for no rotation; halfsplit: pairs (i, i + D/2) instead of
-    (2i, 2i+1).  Returns uint16 [B,S,H,D]."""
+PRE_HALFSPLIT = 1
+PRE_TABLES_BF16 = 2
+PRE_NORM_FULL_ROW = 4
+
+
+def norm_rope_bf16(x_bf16, gain_bf16, eps, cos=None, sin=None, table_batch_rows=0, halfsplit=False, full_row=False):
+    """x: uint16 [B,S,H,D] bf16 bits; gain: uint16 [D] (or [H*D] with full_row: the RMSNorm then
+    runs over all H*D channels of a token); cos/sin: fp32, or uint16 bf16 bits, [rows, D/2] with row
+    s*H + h (plus b*table_batch_rows), or None for no rotation; halfsplit: pairs (i, i + D/2)
+    instead of (2i, 2i+1).  Returns uint16 [B,S,H,D]."""
     x = np.ascontiguousarray(x_bf16, dtype=np.uint16)
     g = np.ascontiguousarray(gain_bf16, dtype=np.uint16)
     B, S, H, D = x.shape
     y = np.empty_like(x)
+    flags = (PRE_HALFSPLIT if halfsplit else 0) | (PRE_NORM_FULL_ROW if full_row else 0)
     if cos is not None:
-        cos = np.ascontiguousarray(cos, dtype=np.float32)
-        sin = np.ascontiguousarray(sin, dtype=np.float32)
+        if np.asarray(cos).dtype == np.uint16:
+            flags |= PRE_TABLES_BF16
+            cos = np.ascontiguousarray(cos, dtype=np.uint16)
+            sin = np.ascontiguousarray(sin, dtype=np.uint16)
+        else:
+            cos = np.ascontiguousarray(cos, dtype=np.float32)
+            sin = np.ascontiguousarray(sin, dtype=np.float32)
         need = (B - 1) * table_batch_rows + S * H
         if cos.shape[0] < need or cos.shape[1] != D // 2 or sin.shape != cos.shape:
             raise ValueError("norm_rope_bf16: cos/sin must be [>= %d, %d]" % (need, D // 2))
-    if g.shape != (D,):
-        raise ValueError("norm_rope_bf16: gain must be [%d]" % D)
+    if g.shape != ((H * D,) if full_row else (D,)):
+        raise ValueError("norm_rope_bf16: gain must be [%d]" % (H * D if full_row else D))
     _chk(lib().sage_oracle_norm_rope_bf16_ex(_p(x), B, H, S, D, strides_bshd(S, H, D), _p(g), eps,
                                              _p(cos) if cos is not None else None,
                                              _p(sin) if sin is not None else None, table_batch_rows,
-                                             1 if halfsplit else 0, _p(y)),
+                                             flags, _p(y)),
          "norm_rope_bf16")
     return y
 

@@ -192,27 +192,42 @@ def f32_to_bf16_bits_rne(x):
     return (r >> 16).astype(np.uint16)
 
 
-def norm_rope_bf16(x_bits_bshd, gain_bits, eps, cos=None, sin=None, table_batch_rows=0, halfsplit=False):
-    B, S, H, D = x_bits_bshd.shape
-    x = bf16_to_f32(x_bits_bshd)                                   # [B,S,H,D]
-    assert D <= 256
-    part = np.zeros((B, S, H, 256), np.float32)
-    part[..., :D] = (np.float32(0.0) + (x * x).astype(np.float32)).astype(np.float32)
+def _sumsq_256(x):
+    """Sum of squares over the last axis the way a block of 256 threads does it
+    (serenitymojo/ops/norm.mojo:56-72): thread t adds x[t]^2, x[t+256]^2, ... in turn, then the
+    256 partial sums fold in halves, far pairs first."""
+    cols = x.shape[-1]
+    part = np.zeros(x.shape[:-1] + (256,), np.float32)
+    for c0 in range(0, cols, 256):
+        chunk = x[..., c0:c0 + 256]
+        part[..., :chunk.shape[-1]] = (part[..., :chunk.shape[-1]] + (chunk * chunk).astype(np.float32)).astype(np.float32)
     while part.shape[-1] > 1:
         half_n = part.shape[-1] // 2
         part = (part[..., :half_n] + part[..., half_n:]).astype(np.float32)
-    ss = part[..., 0]
-    mean = (ss / np.float32(D)).astype(np.float32)
+    return part[..., 0]
+
+
+def norm_rope_bf16(x_bits_bshd, gain_bits, eps, cos=None, sin=None, table_batch_rows=0, halfsplit=False, full_row=False):
+    B, S, H, D = x_bits_bshd.shape
+    x = bf16_to_f32(x_bits_bshd)                                   # [B,S,H,D]
+    if full_row:                                                   # one statistic per token over all H*D channels
+        ss = _sumsq_256(x.reshape(B, S, H * D))[..., None]
+        mean = (ss / np.float32(H * D)).astype(np.float32)
+        g = bf16_to_f32(gain_bits).reshape(H, D)
+    else:
+        ss = _sumsq_256(x)
+        mean = (ss / np.float32(D)).astype(np.float32)
+        g = bf16_to_f32(gain_bits)
     inv = (np.float32(1.0) / np.sqrt((mean + np.float32(eps)).astype(np.float32))).astype(np.float32)
-    g = bf16_to_f32(gain_bits)
     y = ((x * inv[..., None]).astype(np.float32) * g).astype(np.float32)
     y = bf16_to_f32(f32_to_bf16_bits_rne(y))
     if cos is None:
         return f32_to_bf16_bits_rne(y)
     half = D // 2
     rows = (np.arange(B)[:, None, None] * table_batch_rows + np.arange(S)[None, :, None] * H + np.arange(H)[None, None, :])
-    c = np.asarray(cos, np.float32)[rows]                          # [B,S,H,half]
-    s = np.asarray(sin, np.float32)[rows]
+    tab = (lambda t: bf16_to_f32(np.asarray(t))) if np.asarray(cos).dtype == np.uint16 else (lambda t: np.asarray(t, np.float32))
+    c = tab(cos)[rows]                                             # [B,S,H,half]
+    s = tab(sin)[rows]
     # pairs (2i, 2i+1), or (i, i + D/2) in the half-split form
     y0, y1 = (y[..., :half], y[..., half:]) if halfsplit else (y[..., 0::2], y[..., 1::2])
     o0 = ((y0 * c).astype(np.float32) - (y1 * s).astype(np.float32)).astype(np.float32)

@@ -22,15 +22,16 @@ def _gains(rng, D):
             f32_to_bf16_bits((0.7 + 0.3 * rng.standard_normal(D)).astype(np.float32)))
 
 
-def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows, halfsplit=False):
+def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_rows, halfsplit=False, full_row=False):
     import torch
     import gpu_harness as H
     L = _lib.lib()
     B, S, Hh, D = q.shape
     qd, kd = H.dev_bf16(q), H.dev_bf16(k)
     gqd, gkd = H.dev_bf16(gq), H.dev_bf16(gk)
-    cd = torch.from_numpy(cos).cuda() if cos is not None else None
-    sd = torch.from_numpy(sin).cuda() if sin is not None else None
+    tab16 = cos is not None and cos.dtype == np.uint16
+    cd = (H.dev_bf16(cos) if tab16 else torch.from_numpy(cos).cuda()) if cos is not None else None
+    sd = (H.dev_bf16(sin) if tab16 else torch.from_numpy(sin).cuda()) if sin is not None else None
     nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
     q8 = torch.full((B, Hh, nqp, D), 77, dtype=torch.int8, device="cuda")
     k8 = torch.full((B, Hh, nkp, D), 77, dtype=torch.int8, device="cuda")
@@ -42,7 +43,8 @@ def _gpu_quant(q, k, scale, blkq, blkk, smooth, gq, gk, eps, cos, sin, batch_row
     rc = L.mi355_sage_quant_qk_norm_rope_bf16(
         qd.data_ptr(), kd.data_ptr(), B, Hh, S, S, D, scale, st, st, 0, 0,
         gqd.data_ptr(), gkd.data_ptr(), eps, cd.data_ptr() if cd is not None else None,
-        sd.data_ptr() if sd is not None else None, batch_rows, 1 if halfsplit else 0, blkq, blkk, (1 if smooth else 0) | 2,
+        sd.data_ptr() if sd is not None else None, batch_rows,
+        (1 if halfsplit else 0) | (2 if tab16 else 0) | (4 if full_row else 0), blkq, blkk, (1 if smooth else 0) | 2,
         q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
         scr.data_ptr(), scr.numel(), H.stream())
     assert rc == 0, rc
@@ -155,10 +157,10 @@ def test_argument_errors():
                                           st32, st, st, st32, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
                                           g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, 0, None, 0)
     assert rc == 0
-    # an unknown pairing is refused
+    # an unknown option bit is refused
     rc = L.mi355_sage_sdpa_bf16_norm_rope(x.data_ptr(), x.data_ptr(), x.data_ptr(), o.data_ptr(), 1, 2, 64, 64, 128, 0.1,
                                           st, st, st, st, 0, 0, 0, 0, 0, H.stream(), 0, 128, 64, 3,
-                                          g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, 7, None, 0)
+                                          g.data_ptr(), g.data_ptr(), 1e-6, None, None, 0, 8, None, 0)
     assert rc == -1
     torch.cuda.synchronize()
 
@@ -187,3 +189,44 @@ def test_fused_train_fwd_stats(oracle):
     s = np.einsum("bihd,bjhd->bhij", qn, kn) * w.scale
     lse = np.log(np.exp(s - s.max(-1, keepdims=True)).sum(-1)) + s.max(-1)
     np.testing.assert_allclose(fwd.stats.cpu().numpy()[..., 0], lse, atol=3e-2)
+
+
+@pytest.mark.parametrize("Hh,D,S", [(32, 128, 70), (5, 64, 130)])
+def test_full_row_norm_halfsplit_bf16_tables_bit_exact(oracle, Hh, D, S):
+    """LTX-2's pre-attention sequence (models/ltx2/ltx2_block.mojo:419-432) fused into the quantizers:
+    RMSNorm over the whole inner dim H*D with a gain of H*D entries, half-split RoPE with bf16
+    tables.  INT8 codes, scales and K statistics against the checker run on the checker's own
+    norm/rope output, bit for bit; and the one-shot call against the plain call on that output."""
+    import torch
+    import gpu_harness as H
+    from mojodiffusion_amd import attention_sage as A
+    rng = np.random.default_rng(40 + Hh)
+    B = 2
+    q = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32) * 2.0)
+    k = f32_to_bf16_bits((rng.standard_normal((B, S, Hh, D)) + 1.5 * rng.standard_normal((B, 1, Hh, D))).astype(np.float32))
+    v = f32_to_bf16_bits(rng.standard_normal((B, S, Hh, D)).astype(np.float32))
+    q[1, 3] = 0                                                # an all-zero token
+    gq = f32_to_bf16_bits((1.0 + 0.3 * rng.standard_normal(Hh * D)).astype(np.float32))
+    gk = f32_to_bf16_bits((0.7 + 0.3 * rng.standard_normal(Hh * D)).astype(np.float32))
+    th = rng.uniform(-3.14, 3.14, (S * Hh, D // 2))
+    cos, sin = f32_to_bf16_bits(np.cos(th).astype(np.float32)), f32_to_bf16_bits(np.sin(th).astype(np.float32))
+    eps, scale = 1e-6, 1.0 / np.sqrt(D)
+    got = _gpu_quant(q, k, scale, 128, 64, True, gq, gk, eps, cos, sin, 0, halfsplit=True, full_row=True)
+    qn = oracle.norm_rope_bf16(q, gq, eps, cos, sin, 0, halfsplit=True, full_row=True)
+    kn = oracle.norm_rope_bf16(k, gk, eps, cos, sin, 0, halfsplit=True, full_row=True)
+    want = H.oracle_quant_qk(oracle, qn, kn, scale, 128, 64, True, True)
+    for name in ("kmean", "qmul", "kmul"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    nqb, nkb = want["qscale"].shape[2], want["kscale"].shape[2]
+    np.testing.assert_array_equal(got["qscale"][:, :, :nqb].view(np.uint32), want["qscale"].view(np.uint32))
+    np.testing.assert_array_equal(got["kscale"][:, :, :nkb].view(np.uint32), want["kscale"].view(np.uint32))
+    np.testing.assert_array_equal(got["q8"], want["q8"])
+    np.testing.assert_array_equal(got["k8"], want["k8"])
+    qd, kd, vd = H.dev_bf16(q), H.dev_bf16(k), H.dev_bf16(v)
+    fused = A.qk_norm_rope_sdpa_nomask(qd, kd, vd, H.dev_bf16(gq), H.dev_bf16(gk), eps, H.dev_bf16(cos), H.dev_bf16(sin),
+                                       scale, halfsplit=True, full_row=True)
+    plain = A.sdpa_nomask(H.dev_bf16(qn), H.dev_bf16(kn), vd, scale)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(H.to_bits(fused), H.to_bits(plain))
+    with pytest.raises(A.Error, match="weight must be"):
+        A.qk_norm_rope_sdpa_nomask(qd, kd, vd, H.dev_bf16(gq)[:D], H.dev_bf16(gk)[:D], eps, None, None, scale, full_row=True)

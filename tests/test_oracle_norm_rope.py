@@ -127,3 +127,30 @@ def test_bf16_pipeline_matches_numpy_restatement(oracle, D, with_rope, batch_row
         y = (oracle.rope_halfsplit_f32 if halfsplit else oracle.rope_interleaved_f32)(y, cos[idx], sin[idx])
     # (a rotated pair can cancel, so the bf16 steps of the inputs show as absolute error)
     np.testing.assert_allclose(bf16_bits_to_f32(got).reshape(-1, D), y, rtol=2.0 ** -6, atol=3e-2)
+
+
+@pytest.mark.parametrize("H,D", [(32, 128), (5, 64)])
+def test_full_row_norm_halfsplit_bf16_tables(oracle, H, D):
+    """The pre-attention sequence of serenitymojo/models/ltx2/ltx2_block.mojo:419-432: rms_norm over
+    the whole inner dim H*D (gain [H*D]), reshape to heads, rope_halfsplit with bf16 tables.  Against
+    the numpy restatement bit for bit, and against the composition of the checker's fp32 ops."""
+    rng = np.random.default_rng(5 + H)
+    B, S = 2, 9
+    x = f32_to_bf16_bits(rng.standard_normal((B, S, H, D)).astype(np.float32) * 2.0)
+    x[1, 4] = 0                                                  # an all-zero token
+    gain = f32_to_bf16_bits((1.0 + 0.2 * rng.standard_normal(H * D)).astype(np.float32))
+    th = rng.uniform(-3.14, 3.14, (S * H, D // 2))
+    cos, sin = f32_to_bf16_bits(np.cos(th).astype(np.float32)), f32_to_bf16_bits(np.sin(th).astype(np.float32))
+    got = oracle.norm_rope_bf16(x, gain, 1e-6, cos, sin, 0, halfsplit=True, full_row=True)
+    want = R.norm_rope_bf16(x, gain, 1e-6, cos, sin, 0, halfsplit=True, full_row=True)
+    np.testing.assert_array_equal(got, want)
+    assert not bf16_bits_to_f32(got[1, 4]).any()
+    y = oracle.rms_norm_f32(bf16_bits_to_f32(x).reshape(B * S, H * D), bf16_bits_to_f32(gain), 1e-6).reshape(B * S * H, D)
+    idx = np.tile(np.arange(S * H), B)
+    y = oracle.rope_halfsplit_f32(y, bf16_bits_to_f32(cos)[idx], bf16_bits_to_f32(sin)[idx])
+    np.testing.assert_allclose(bf16_bits_to_f32(got).reshape(-1, D), y, rtol=2.0 ** -6, atol=3e-2)
+    # the statistic really is the row's: scaling one head changes every head's output
+    x2 = x.copy()
+    x2[:, :, 0] = f32_to_bf16_bits(bf16_bits_to_f32(x[:, :, 0]) * 4.0)
+    got2 = oracle.norm_rope_bf16(x2, gain, 1e-6, cos, sin, 0, halfsplit=True, full_row=True)
+    assert (got2[0, 0, 1] != got[0, 0, 1]).any()
