@@ -214,6 +214,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
     constexpr int KS = D / 16;                      // matrix-instruction steps over the head dim
     constexpr int DB = D / 32;                      // 32-channel output blocks
     constexpr int NTR = PASS == 0 ? 1 : 2;          // transposed operands per tile
+    // The dK/dV pass needs more than 256 registers per lane.  Its gradient accumulators are only
+    // ever touched by matrix instructions inside the loop, so they are steered into the
+    // accumulation registers (an empty statement with an "a" constraint per tile); left to itself
+    // the compiler parks the SCORE accumulators there, which the vector ALU reads element by
+    // element, and pays a copy for every one.
+    constexpr bool ACC_IN_AGPR = PASS == 1 && NW == 4;
     static_assert(RUNS % NW == 0, "tile copies must divide over the waves");
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds_nat[2][2][TILE_BYTES];
@@ -253,7 +259,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
         lse_x = a.lse2[idx];
         delta_x = a.delta[idx];
     }
-    // the plain loads above must not be in flight when the copy counter is used below
+    // The plain loads above must have landed before the loop: the compiler waits for a load at the
+    // first use of its result, and such a wait inside the loop would also wait for the tile copies
+    // that are meant to stay in flight (they share the counter).  Using the values here puts the
+    // waits here.
+#pragma unroll
+    for (int s = 0; s < KS; s++) asm volatile("" : "+v"(b1[s]), "+v"(b2[s]));
+    asm volatile("" : "+v"(lse_x), "+v"(delta_x));
     dma_wait_all();
 
     // y side
@@ -327,6 +339,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
         dma_wait_all();
         __syncthreads();                 // tile t is visible; every wave is done with the other stage
         if (t + 1 < ntiles) copy_tile(t + 1, stage ^ 1);
+        if constexpr (ACC_IN_AGPR) {
+#pragma unroll
+            for (int d = 0; d < DB; d++) asm volatile("" : "+a"(acc1[d]), "+a"(acc2[d]));
+        }
         const uint8_t* n1 = &lds_nat[stage][0][0];
         const uint8_t* n2 = &lds_nat[stage][1][0];
         const uint8_t* r1 = &lds_tr[stage][0][0];
@@ -341,12 +357,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
         for (int blk = 0; blk < 2; blk++)
 #pragma unroll
             for (int i = 0; i < 16; i++) tacc[blk][i] = 0.0f, gacc[blk][i] = 0.0f;
-        // one k-step of the two score products of a block: T += Y1 . X1^T, G += Y2 . X2^T
+        // one k-step of the two score products of a block: T += Y1 . X1^T, G += Y2 . X2^T.  The
+        // fragments of step ks + 1 are requested before the products of step ks are issued.
+        v4i f1[2], f2[2];
+        auto scores_load = [&](int blk, int ks) {
+            f1[ks & 1] = *reinterpret_cast<const v4i*>(n1 + nat_frag[blk][ks]);
+            f2[ks & 1] = *reinterpret_cast<const v4i*>(n2 + nat_frag[blk][ks]);
+        };
         auto scores_step = [&](int blk, int ks) {
-            const v4i f1 = *reinterpret_cast<const v4i*>(n1 + nat_frag[blk][ks]);
-            const v4i f2 = *reinterpret_cast<const v4i*>(n2 + nat_frag[blk][ks]);
-            tacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f1), __builtin_bit_cast(v8bf, b1[ks]), tacc[blk], 0, 0, 0);
-            gacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f2), __builtin_bit_cast(v8bf, b2[ks]), gacc[blk], 0, 0, 0);
+            if (ks + 1 < KS) scores_load(blk, ks + 1);
+            tacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f1[ks & 1]), __builtin_bit_cast(v8bf, b1[ks]), tacc[blk], 0, 0, 0);
+            gacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f2[ks & 1]), __builtin_bit_cast(v8bf, b2[ks]), gacc[blk], 0, 0, 0);
+            // The vector ALU reads every element of the finished scores: keep them in ordinary
+            // registers.  (Only a register-class hint: the matrix instructions stay compiler-visible
+            // builtins, so the wait states between them and their readers are still inserted.)
+            if (ACC_IN_AGPR && ks == KS - 1) asm volatile("" : "+v"(tacc[blk]), "+v"(gacc[blk]));
         };
         // elements i, i+1 of a block (i even): y rows (i>>2)*8 + half*4 + (i&3) (+1), column = owner row
         auto softmax_pair = [&](int blk, int i) {
@@ -391,9 +416,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
                 acc2[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, pb), acc2[d], 0, 0, 0);
             }
         };
+        scores_load(0, 0);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) scores_step(0, ks);
         // scores of block 1 with the exponentials of block 0: 8 pairs over KS k-steps
+        scores_load(1, 0);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             scores_step(1, ks);
