@@ -113,6 +113,11 @@ def summarize_traffic(dirs):
     f_scale, w_scale = copy_kib / fetch_copy, copy_kib / write_copy
     total = int(round((fetch * f_scale + write * w_scale) * 1024.0))
     print("# HBM traffic of sage_attn_kernel per launch, rocprofv3 --pmc (one counter per run)")
+    print("# Commands (repository root on the MI355X box, after `cd /tmp && export TMPDIR=/tmp` and back), C = FETCH_SIZE, then WRITE_SIZE:")
+    print("#   rocprofv3 --pmc C --output-format csv -d gpurun_out/pmc_C_bench -o p -- python3 bench.py --skip-cpu-baseline --steps 3 --warmup 2")
+    print("#   rocprofv3 --pmc C --output-format csv -d gpurun_out/pmc_C_copy -o p -- python3 bench.py --copy-calibration")
+    print("#   python3 bench.py --summarize-traffic gpurun_out/pmc_FETCH_SIZE_bench gpurun_out/pmc_WRITE_SIZE_bench "
+          "gpurun_out/pmc_FETCH_SIZE_copy gpurun_out/pmc_WRITE_SIZE_copy")
     print("kernel_source_digest = %s" % kernel_source_digest())
     print("fetch_size_kib_per_dispatch = %.1f   # %d dispatches" % (fetch, n_f))
     print("write_size_kib_per_dispatch = %.1f   # %d dispatches" % (write, n_w))
@@ -184,8 +189,8 @@ def clock_probe(args, L, w, qd, kd, vd, o, st, stream):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--summarize-traffic", nargs=4, metavar="DIR",
@@ -244,6 +249,16 @@ def main():
         if rc != 0:
             raise RuntimeError("mi355_sage_sdpa_bf16_ex rc=%d" % rc)
 
+    # The chip takes some milliseconds of load to leave its idle clocks (a 50-step run right after
+    # start-up reads 12 % slower than a 1000-step one): run the same step, untimed, for 0.15 s
+    # before the warm-up proper, whatever --warmup says.
+    ramp_steps = 0
+    r0 = time.perf_counter()
+    while time.perf_counter() - r0 < 0.15:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        ramp_steps += 20
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -362,6 +377,7 @@ def main():
             "stage_ms": {"quant_qk": round(qk_avg, 5), "quant_v": round(v_avg, 5), "attn": round(at_avg, 5)},
             "one_shot_quant_ms": round(ms_per_step - at_avg, 5),
             "graph_replay_ms": None if graph_ms is None else round(graph_ms, 5),
+            "clock_ramp_steps": ramp_steps,      # untimed steps run before the warm-up, see above
             "quant_stage_hbm": {"algorithmic_bytes": quant_bytes, "GB/s": round(quant_gbs, 1),
                                 "frac_of_8TB/s": round(quant_gbs / PEAK_HBM_GBS, 4)},
             "device": torch.cuda.get_device_name(0),

@@ -317,6 +317,20 @@ int mi355_sage_attn_fwd(
     void* O, const int64_t* o_strides, int64_t o_offset_elems,
     const void* qshift, void* stats, void* stream);
 
+/* Scheduling of the attention kernel (no counterpart in the reference; for tests and tuning).
+ * One workgroup computes 256 query rows of one head against all keys; a shape whose row tiles
+ * leave the last round of the 256 compute units at most half full (more than 256 tiles, 16 % or
+ * more of the launch idle) is instead cut into equal shares of (row tile, key tile) steps for
+ * exactly 256 workgroups, which hand unnormalised partial results to each other inside the launch.  The choice depends on the
+ * shape only, so all entry points give the same bits for the same problem; outputs of the two
+ * schedules differ by rounding (the probabilities of a row are rounded against a different
+ * running maximum).  mode 0: by shape (default); -1: never split; n > 0 (multiple of 8, <= 1024):
+ * always split over n workgroups.  Process-wide; affects workspace sizes (the hand-over slots are
+ * part of mi355_sage_workspace_bytes), so set it before sizing workspaces.  mi355_sage_attn_fwd,
+ * which takes no workspace, keeps its slots in a library-owned per-stream buffer (allocated on
+ * the first such call of a stream, never while that stream is being captured). */
+int mi355_sage_set_attn_split(int mode);
+
 /* Backward.  Replaces flame_cudnn_sdpa_bwd_bf16 (serenitymojo/ops/cshim/cudnn_sdpa_bwd.cpp:325-347;
  * Mojo callers ops/attention_flash.mojo:345-433, :478-535, :538-607): identical parameter list up
  * to `stream`, then the workspace pair.  Q, K, V, O, dO bf16 and dQ, dK, dV bf16, each a logical

@@ -70,7 +70,7 @@ int check_kv_len(int N_kv, int blkk) {
 
 // Workspace layout of the one-shot calls.
 struct Carve {
-    size_t q8, k8, vq, qscale, kscale, kmean, qmul, kmul, vscale, kpart_sum, kpart_mm, vpart, qshift, rowinv_q, rowinv_k, total;
+    size_t q8, k8, vq, qscale, kscale, kmean, qmul, kmul, vscale, kpart_sum, kpart_mm, vpart, qshift, rowinv_q, rowinv_k, split, total;
 };
 
 Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
@@ -95,6 +95,8 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.qshift = take(bh * nqp * sizeof(float));
     c.rowinv_q = take((size_t)B * Nq * sizeof(float));        // whole-row RMSNorm statistic per token (optional pre-op)
     c.rowinv_k = take((size_t)B * Nkv * sizeof(float));
+    // hand-over slots of the attention kernel's split scheduling (shapes that use it only)
+    c.split = take(attn_split_bytes(attn_split_workgroups(B, H, Nq, Nkv), D));
     c.total = off;
     return c;
 }
@@ -123,11 +125,14 @@ ScratchCarve scratch_carve(int B, int H, int Nkv, int D) {
 // so the retired buffers of a stream add up to less than its current one.  Allocation is not
 // possible while the stream is being captured into a graph: such a call fails with
 // MI355_SAGE_EWORKSPACE unless the buffer is already large enough.
+struct StreamWs;
+std::vector<StreamWs>& sage_api_ws();
 std::mutex g_ws_mutex;
 struct StreamWs { int dev; hipStream_t stream; void* p; size_t bytes; };
-std::vector<StreamWs> g_ws;
+std::vector<StreamWs> g_ws;          // one-shot calls
+std::vector<StreamWs> g_split_ws;    // hand-over slots of mi355_sage_attn_fwd, which takes no workspace
 
-int internal_workspace(size_t need, hipStream_t stream, void** out) {
+int internal_workspace(size_t need, hipStream_t stream, void** out, std::vector<StreamWs>& g_ws = sage_api_ws()) {
     int dev = 0;
     SAGE_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_ws_mutex);
@@ -155,6 +160,7 @@ int internal_workspace(size_t need, hipStream_t stream, void** out) {
     *out = w->p;
     return 0;
 }
+std::vector<StreamWs>& sage_api_ws() { return g_ws; }
 
 // The optional ops in front of the quantizers (RMSNorm + interleaved RoPE of Q and of K).
 struct Pre {
@@ -365,6 +371,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         a.amask = static_cast<const uint16_t*>(mask.add) + mask.add_off;
         a.amb = mask.add_strides[0]; a.amh = mask.add_strides[1]; a.amn = mask.add_strides[2];
     }
+    a.split = ws + c.split;
     SAGE_HIP(launch_attn(a, st));
     return MI355_SAGE_OK;
 }
@@ -658,7 +665,17 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(N_kv, kPadKV);
     a.o = static_cast<uint16_t*>(O) + o_off; a.osb = o_strides[0]; a.osh = o_strides[1]; a.osn = o_strides[2];
     a.stats = static_cast<float*>(stats);
+    // Same scheduling, hence the same bits, as the one-shot calls: shapes that are split over a
+    // fixed number of workgroups need hand-over slots, kept per (device, stream) by the library.
+    const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid), D);
+    if (split_bytes > 0 && (rc = internal_workspace(split_bytes, static_cast<hipStream_t>(stream), &a.split, g_split_ws))) return rc;
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
+    return MI355_SAGE_OK;
+}
+
+int mi355_sage_set_attn_split(int mode) {
+    if (mode < -1 || mode > kSplitMaxWorkgroups || (mode > 0 && (mode & 7))) return MI355_SAGE_EINVAL;
+    attn_split_override(mode);
     return MI355_SAGE_OK;
 }
 

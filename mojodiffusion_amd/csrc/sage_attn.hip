@@ -29,6 +29,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include <atomic>
 #include <type_traits>
 
 namespace sage {
@@ -37,6 +38,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -120,7 +122,7 @@ template <int VARIANT> struct Lazy {
 // for every tile's maximum on the biased scores (no optimistic tiles) and lets its ordinary
 // global loads share the vector-memory counter with the tile copies, i.e. it waits for all of
 // them at the midpoint: it is bound by the N_q x N_kv bias it has to read, not by the copies.
-template <int D, int VARIANT, bool STATS, bool ADDMASK>
+template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT>
 __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
@@ -129,7 +131,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     int H, int Nq, int kv_valid, int mask_lo, int mask_hi, int64_t nq_pad, int64_t nkv_pad,
     uint16_t* __restrict__ o, int64_t osb, int64_t osh, int64_t osn,
     float* __restrict__ stats, int n_qtiles, int total_wg,
-    const uint16_t* __restrict__ amask, int64_t amb, int64_t amh, int64_t amn) {
+    const uint16_t* __restrict__ amask, int64_t amb, int64_t amh, int64_t amn,
+    int split_groups, float* split_part, int* split_flags) {
     constexpr int VB = (VARIANT == 0) ? 2 : 1;          // bytes per V element
     constexpr int KSTEPS = D / 32;                      // int8 MFMA steps over the head dim
     constexpr int DB = D / 32;                          // 32-channel output blocks
@@ -156,19 +159,33 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][V_BYTES];
     __shared__ float lds_ks[kMaxKScales];
 
-    // Workgroup -> (q tile, b*h).  Hardware hands consecutive workgroup ids to the 8
-    // XCDs round-robin; give each XCD a contiguous range of (head, q tile) work so the
-    // workgroups sharing one head's K/V also share one L2.
-    int wg = blockIdx.x;
-    {
-        const int per = (total_wg + 7) >> 3;
-        const int xcd = wg & 7, idx = wg >> 3;
-        const int full = total_wg - (per - 1) * 8;      // XCDs that own `per` items (1..8)
-        wg = (xcd < full) ? xcd * per + idx : full * per + (xcd - full) * (per - 1) + idx;
-    }
-    const int qt = wg % n_qtiles;
-    const int64_t bh = wg / n_qtiles;
-    const int b = (int)(bh / H), h = (int)(bh % H);
+    // Work items are (q tile, b*h) pairs, `total_wg` of them; an item takes `ntiles` steps (key
+    // tiles).  Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; each XCD gets a
+    // contiguous range of items, so the workgroups sharing one head's K/V also share one L2.
+    //
+    // split_groups == 0: one workgroup per item.  Otherwise the XCD's steps, laid end to end, are
+    // cut into split_groups equal spans, one per workgroup of that XCD, so that every compute unit
+    // gets the same number of steps whatever the item count.  A span covers the tail of one item,
+    // whole items, and the head of another.  The workgroup that holds an item's last key tile
+    // writes the item's output; the others leave their unnormalised accumulators, reference
+    // maxima and row sums in split_part and raise their flag.  A workgroup walks its span from
+    // the back, so what it leaves for others it leaves first, and the only workgroups it ever
+    // waits for are ones with a lower id in the same XCD — dispatched before it, and not waiting
+    // for anybody when they produce what it needs.
+    const int bid = blockIdx.x;
+    const int xcd = bid & 7, wg_j = bid >> 3;
+    const int items_per = (total_wg + 7) >> 3;
+    const int xcd_full = total_wg - (items_per - 1) * 8;        // XCDs that own `items_per` items (1..8)
+    const int n_items = xcd < xcd_full ? items_per : items_per - 1;
+    const int item0 = xcd < xcd_full ? xcd * items_per : xcd_full * items_per + (xcd - xcd_full) * (items_per - 1);
+    const int ntiles_item = (kv_valid + kTileKV - 1) / kTileKV;
+    // (the launcher has checked that steps x workgroups stays inside 32 bits)
+    const uint32_t xcd_steps = (uint32_t)n_items * (uint32_t)ntiles_item;
+    auto span_lo = [&](int j) -> int {
+        return SPLIT ? (int)(xcd_steps * (uint32_t)j / (uint32_t)split_groups) : min(j, n_items) * ntiles_item;
+    };
+    const int span_begin = span_lo(wg_j);
+    int span_end = span_lo(wg_j + 1);
 
 #ifdef SAGE_CLOCK_PROBE
     // Measurement build only (libmi355_sage_probe.so): shader cycles and constant-rate time of
@@ -179,7 +196,31 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
-    const int qrow = qt * kTileQ + wave * 32 + l32;     // this lane's query (padded index)
+
+    // ---- one segment = key tiles [t_off, t_off + ntiles) of one item, last segment of the span first
+    // (the instantiation without splitting is straight-line code: one segment, the whole item)
+    if (SPLIT && span_end <= span_begin) return;        // an empty span
+    do {
+    // (divisors through an empty statement: a few divisions per segment are cheaper than their
+    // reciprocals kept in registers across the main loop)
+    int ntiles_div = ntiles_item, qtiles_div = n_qtiles, heads_div = H;
+    if constexpr (SPLIT) asm volatile("" : "+s"(ntiles_div), "+s"(qtiles_div), "+s"(heads_div));
+    const int item_local = SPLIT ? (int)((uint32_t)(span_end - 1) / (uint32_t)ntiles_div) : wg_j;
+    const int item_base = item_local * ntiles_item;
+    const int t_off = SPLIT ? max(span_begin, item_base) - item_base : 0;
+    const int ntiles = SPLIT ? span_end - item_base - t_off : ntiles_item;
+    const bool seg_finishes = !SPLIT || t_off + ntiles == ntiles_item;   // holds the item's last key tile: writes the output
+    span_end = item_base + t_off;
+    const int wg = item0 + item_local;
+    const int qt = (int)((uint32_t)wg % (uint32_t)qtiles_div);
+    const int64_t bh = (uint32_t)wg / (uint32_t)qtiles_div;
+    const int b = (int)((uint32_t)bh / (uint32_t)heads_div), h = (int)((uint32_t)bh % (uint32_t)heads_div);
+    // (through an empty statement: the per-lane addresses derived from the row are formed in the
+    // segment that uses them instead of being carried in registers across the main loop)
+    int row_in_tile = wave * 32 + l32;
+    if constexpr (SPLIT) asm volatile("" : "+v"(row_in_tile));
+    const int qrow = qt * kTileQ + row_in_tile;         // this lane's query (padded index)
+    __syncthreads();                                    // every wave has left the previous segment's LDS
 
     // Q^T fragments: 16 bytes of the head dim per step, resident for the whole kernel.
     v4i qf[KSTEPS];
@@ -198,12 +239,12 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const float* ksc = kscale + bh * (nkv_pad / blkk);
     const int nks = (int)(nkv_pad / blkk);
     const int ush = blkk == 32 ? 0 : (blkk == 64 ? 1 : 2);      // log2(32-key blocks per scale block)
-    for (int i = tid; i < nks; i += 64 * NW) lds_ks[i] = ksc[i];
+    for (int i = row_in_tile + half * 256; i < nks; i += 64 * NW) lds_ks[i] = ksc[i];     // (indices 0..511, once each)
     auto kscale_of = [&](int u32blk) -> float { return lds_ks[u32blk >> ush]; };
 
-    const uint8_t* kg = reinterpret_cast<const uint8_t*>(k8) + bh * nkv_pad * D;
-    const uint8_t* vg = vq + bh * nkv_pad * D * VB;
-    const int ntiles = (kv_valid + kTileKV - 1) / kTileKV;
+    // tile indices below are relative to the segment's first tile
+    const uint8_t* kg = reinterpret_cast<const uint8_t*>(k8) + bh * nkv_pad * D + (int64_t)t_off * K_BYTES;
+    const uint8_t* vg = vq + bh * nkv_pad * D * VB + (int64_t)t_off * V_BYTES;
     const int last = ntiles - 1;
 
     // Tile-relative LDS byte offsets of this lane's MFMA A-operand fragments.  Rows
@@ -337,11 +378,11 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
 
         float f[2], c0[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) f[kb] = sq * kscale_of(t * 2 + kb);
+        for (int kb = 0; kb < 2; kb++) f[kb] = sq * kscale_of((t + t_off) * 2 + kb);
         // Tiles that hold masked keys (the ragged end, the masked range) are rare: a real branch.
         // A masked score becomes -inf (as an integer: below every real accumulator), which the
         // exponent path below turns into p = 0 without any further test.
-        const int key0 = t * kTileKV;
+        const int key0 = (t + t_off) * kTileKV;
         if (key0 + kTileKV > kv_valid || (key0 < mask_hi && key0 + kTileKV > mask_lo)) {
             asm volatile("" ::: "memory");
 #pragma unroll
@@ -526,6 +567,68 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     if (last & 1) drain(X1{});
     else drain(X0{});
 
+    // Hand-over between workgroups of ONE XCD goes through that XCD's L2, which every compute unit
+    // of the XCD reads and writes: the producer only has to wait until its stores have left the
+    // compute unit (the vector L1 writes through), the consumer reads past its own L1.  No L2
+    // write-back or invalidation — device-scope fences would throw the K/V tiles out of the L2 for
+    // everybody.  That both sides sit on the same XCD follows from the round-robin placement of
+    // workgroup ids; the flag carries the producer's XCD number so that the consumer can check.
+    constexpr int PART_FLOATS = (DB * 16 + 2) * 512;    // one workgroup's slot of split_part
+    const int my_xcd = SPLIT ? (int)__builtin_amdgcn_s_getreg(20 | (3 << 11)) : 0;     // XCC_ID, bits 3:0
+    if (SPLIT && !seg_finishes) {
+        // ---- this item ends in another workgroup's span: hand over the running state ----------
+        float* part = split_part + (int64_t)bid * PART_FLOATS;
+        // (taken through an empty statement so that the store addresses are formed here, not kept
+        // in registers from before the loop)
+        uint32_t lane_off = (uint32_t)tid;
+        asm volatile("" : "+v"(lane_off));
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) part[(d * 16 + i) * 512 + lane_off] = oacc[d][i];
+        part[DB * 16 * 512 + lane_off] = m_used;
+        part[DB * 16 * 512 + 512 + lane_off] = VARIANT == 0 ? l_run : lacc[0];
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) __hip_atomic_store(split_flags + bid, 1 + my_xcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        continue;
+    }
+    float poison = 0.0f;
+    if (SPLIT && t_off > 0) {
+        // ---- fold in what the workgroups before this one computed for the item's earlier tiles
+        int need = item_base + t_off;                   // steps [need, end of item) are accounted for
+        uint32_t lane_off = (uint32_t)tid;
+        asm volatile("" : "+v"(lane_off));
+        for (int jp = wg_j - 1; need > item_base && jp >= 0; jp--) {
+            const int ps0 = span_lo(jp), ps1 = span_lo(jp + 1);
+            if (ps1 <= ps0) continue;                   // an empty span
+            const int pb = jp * 8 + xcd;
+            // Bounded wait.  The producer runs this part first and waits for nobody, so the flag
+            // is normally up long before; if it never comes, or comes from another XCD, the rows
+            // are poisoned with NaN rather than left to hang or to read stale data.
+            int spins = 0, flag;
+            while ((flag = __hip_atomic_load(split_flags + pb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) == 0) {
+                if (++spins > (1 << 22)) break;
+                __builtin_amdgcn_s_sleep(16);
+            }
+            asm volatile("" ::: "memory");
+            if (flag != 1 + my_xcd) poison = __builtin_nanf("");
+            const float* part = split_part + (int64_t)pb * PART_FLOATS;
+            auto peer = [&](int idx) { return __hip_atomic_load(part + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+            const float m_p = peer(DB * 16 * 512 + lane_off), l_p = peer(DB * 16 * 512 + 512 + lane_off);
+            const float m_new = fmaxf(m_used, m_p);
+            const float ca = __builtin_amdgcn_exp2f(m_used - m_new), cb = __builtin_amdgcn_exp2f(m_p - m_new);
+            if constexpr (VARIANT == 0) l_run = l_run * ca + l_p * cb;
+            else lacc[0] = lacc[0] * ca + l_p * cb;
+#pragma unroll
+            for (int d = 0; d < DB; d++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) oacc[d][i] = oacc[d][i] * ca + peer((d * 16 + i) * 512 + lane_off) * cb;
+            m_used = m_new;
+            need = ps0;
+        }
+    }
+
     // ---- epilogue: normalise, bf16 round-to-nearest-even, caller's strides ---------
     float l_tot;
     if constexpr (VARIANT == 0) {
@@ -534,7 +637,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     } else {
         l_tot = lacc[0];
     }
-    const float inv = 1.0f / l_tot;      // l carries pscale, which cancels the pscale in P
+    const float inv = 1.0f / l_tot + poison;      // l carries pscale, which cancels the pscale in P
     if (qrow < Nq) {
         uint16_t* op = o + b * osb + h * osh + (int64_t)qrow * osn;
 #pragma unroll
@@ -561,6 +664,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             stats[bh * Nq + qrow] = (m_used + __builtin_amdgcn_logf(l_tot) - Lazy<VARIANT>::log2_pscale + shift) * 0.6931471805599453f;
         }
     }
+    } while (SPLIT && span_end > span_begin);       // segments
 #ifdef SAGE_CLOCK_PROBE
     if (STATS) {
         __syncthreads();
@@ -575,17 +679,36 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
 #endif
 }
 
+__global__ void split_clear_kernel(int* flags, int n) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) flags[i] = 0;
+}
+
 template <int D, int VARIANT>
 static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     const int n_qtiles = (int)(a.nq_pad / kTileQ);
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    dim3 grid((unsigned)total), block(512);
-#define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                                                                          \
-    hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
-                       a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,   \
-                       a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,        \
-                       (int)total, a.amask, a.amb, a.amh, a.amn)
+    const int split = attn_split_workgroups(a.B, a.H, a.Nq, a.kv_valid);
+    int* flags = nullptr;
+    float* part = nullptr;
+    if (split > 0) {
+        if (a.split == nullptr || (split & 7)) return hipErrorInvalidValue;
+        flags = static_cast<int*>(a.split);
+        part = reinterpret_cast<float*>(static_cast<uint8_t*>(a.split) + kSplitFlagBytes);
+        // (a kernel, not a memset: the call may be recorded into a graph)
+        hipLaunchKernelGGL(split_clear_kernel, dim3(1), dim3(256), 0, st, flags, split);
+    }
+    dim3 grid((unsigned)(split > 0 ? split : total)), block(512);
+#define SAGE_LAUNCH_ATTN2(STATS, ADDMASK, SPLIT)                                                                         \
+    hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK, SPLIT>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
+                       a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,          \
+                       a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,               \
+                       (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags)
+#define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                   \
+    do {                                                   \
+        if (split > 0) SAGE_LAUNCH_ATTN2(STATS, ADDMASK, true); \
+        else SAGE_LAUNCH_ATTN2(STATS, ADDMASK, false);     \
+    } while (0)
     if (a.amask != nullptr) {
         if (a.stats != nullptr) SAGE_LAUNCH_ATTN(true, true);
         else SAGE_LAUNCH_ATTN(false, true);
@@ -594,7 +717,49 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
         else SAGE_LAUNCH_ATTN(false, false);
     }
 #undef SAGE_LAUNCH_ATTN
+#undef SAGE_LAUNCH_ATTN2
     return hipGetLastError();
+}
+
+// ---- split scheduling: when, and over how many workgroups -------------------------------------
+// One workgroup per item runs in ceil(items / 256) rounds on the 256 compute units (a workgroup
+// fills one).  When the last round is at most half full and leaves 16 % or more of the launch's
+// compute-unit time idle, the steps are spread over exactly 256 workgroups instead.  Measured on
+// an MI355X (one-shot call, D = 128): 323 items -13 %, 576 items -11 %, 640 items -5 %, 320 items
+// of 32 steps -6 %; under 3 % either way at 400, 432 and 864 items (last round 56 %, 69 %, 38 %
+// full) and at 1584 items (seven rounds): a partly filled round runs at a higher clock — the chip
+// is power-limited under this kernel — and every hand-over costs a second prologue and 132 KB
+// each way.  Twice as many workgroups (two per compute unit, one after the other) were slower
+// everywhere but at 1584 items.  The decision depends on the shape only, so every entry point
+// produces the same bits for the same problem.
+static std::atomic<int> g_split_mode{0};       // 0: by shape; -1: never; n > 0: always, over n workgroups
+
+void attn_split_override(int mode) { g_split_mode.store(mode); }
+
+int attn_split_workgroups(int B, int H, int Nq, int kv_valid) {
+#ifdef SAGE_CLOCK_PROBE
+    return 0;                                  // the measurement build reports per-item clocks
+#else
+    const int64_t items = pad_to(Nq, kTileQ) / kTileQ * B * H;
+    const int64_t ntiles = (kv_valid + kTileKV - 1) / kTileKV;
+    const int mode = g_split_mode.load();
+    if (mode < 0) return 0;
+    if ((items / 8 + 1) * ntiles * kSplitMaxWorkgroups >= (int64_t)1 << 31) return 0;    // 32-bit step arithmetic in the kernel
+    if (mode > 0) return mode;
+    constexpr int64_t kUnits = 256;
+    if (items <= kUnits) return 0;
+    const int64_t rounds = (items + kUnits - 1) / kUnits;
+    const int64_t in_last = items - (rounds - 1) * kUnits;     // 1..256 workgroups in the last round
+    if (in_last * 2 > kUnits) return 0;                        // more than half full
+    if ((kUnits - in_last) * 100 < rounds * kUnits * 16) return 0;     // idle share under 16 %
+    if (items * ntiles < kUnits * 16) return 0;                // spans too short to be worth the hand-over
+    return (int)kUnits;
+#endif
+}
+
+size_t attn_split_bytes(int workgroups, int D) {
+    if (workgroups <= 0) return 0;
+    return kSplitFlagBytes + (size_t)workgroups * ((D / 32) * 16 + 2) * 512 * sizeof(float);
 }
 
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st) {
