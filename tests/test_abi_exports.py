@@ -39,6 +39,39 @@ def test_no_gpu_helpers():
     assert L.mi355_sage_workspace_bytes(0, 24, 4608, 4608, 128, 0) == 0
 
 
+def test_split_schedule_is_a_function_of_the_shape():
+    """Hand-over slots (256 workgroups x (D/32*16 + 2) x 512 floats + 4 KiB of flags) are part of the
+    workspace exactly for the shapes that split: more than 256 row tiles, last round of 256 at most
+    half full, 16 % or more of the launch idle, spans of 16 steps or more."""
+    L = _lib.lib()
+    slots = lambda D: 4096 + 256 * ((D // 32) * 16 + 2) * 512 * 4
+
+    def extra(B, H, S, D):
+        assert L.mi355_sage_set_attn_split(0) == 0
+        with_split = L.mi355_sage_workspace_bytes(B, H, S, S, D, 0)
+        assert L.mi355_sage_set_attn_split(-1) == 0
+        try:
+            return with_split - L.mi355_sage_workspace_bytes(B, H, S, S, D, 0)
+        finally:
+            L.mi355_sage_set_attn_split(0)
+    assert extra(1, 33, 2048, 64) == slots(64)          # 264 tiles: 1.03 rounds
+    assert extra(1, 19, 4352, 128) == slots(128)        # 323 tiles
+    assert extra(1, 32, 4608, 128) == slots(128)        # 576 tiles: 2.25 rounds
+    assert extra(1, 24, 4608, 128) == 0                 # 432 tiles: last round 69 % full
+    assert extra(2, 30, 4352, 128) == 0                 # 1020 tiles: 3.98 rounds
+    assert extra(1, 24, 16896, 128) == 0                # 1584 tiles: idle share 12 %
+    assert extra(1, 32, 1536, 128) == 0                 # 192 tiles: fewer than compute units
+    assert extra(1, 8, 1024, 64) == 0
+    # forced modes
+    assert L.mi355_sage_set_attn_split(64) == 0
+    try:
+        assert L.mi355_sage_workspace_bytes(1, 2, 512, 512, 64, 0) > 64 * 34 * 512 * 4
+    finally:
+        L.mi355_sage_set_attn_split(0)
+    for bad in (-2, 12, 1032):
+        assert L.mi355_sage_set_attn_split(bad) == -1
+
+
 def test_argument_validation_without_device():
     """Order and codes of serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393: null
     pointers, non-positive dims, null strides -> -1 before anything touches a GPU."""
