@@ -37,7 +37,8 @@ def _close_to_plain(got_bits, plain_bits):
 
 
 @pytest.mark.parametrize("wid,variant,S,groups", [(2, 0, 1100, 24), (2, 0, 1100, 64), (2, 0, 1100, 8), (2, 1, 1100, 24),
-                                                  (4, 1, 700, 64), (3, 0, 333, 1024), (1, 0, 1024, 40), (1, 1, 520, 16)])
+                                                  (4, 1, 700, 64), (3, 0, 333, 1024), (1, 0, 1024, 40), (1, 1, 520, 16),
+                                                  (2, 0, 50, 16), (1, 1, 64, 24), (2, 0, 2000, 8), (1, 0, 2000, 200)])
 def test_forced_split_against_checker_and_plain_schedule(oracle, split, wid, variant, S, groups):
     import gpu_harness as H
     from test_gpu_attn import _one_shot
