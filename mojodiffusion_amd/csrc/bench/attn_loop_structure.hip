@@ -47,7 +47,7 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
-constexpr int FRAG = 1, COPY = 2, BARRIER = 4;
+constexpr int FRAG = 1, COPY = 2, BARRIER = 4, EVERY2 = 8, EVERY4 = 16;     // EVERYn: the barrier only in every n-th tile
 constexpr int TILES = 72, HEADS = 24;
 
 struct Stamp { unsigned long long clocks, at_barrier, t_begin, t_end; };
@@ -98,7 +98,8 @@ __global__ __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) void loop_kernel(int tile
     unsigned long long at_barrier = 0;
     auto mid = [&](int t) {
         if constexpr (FEAT & COPY) dma_wait<(LEAD - 1) * (KCH + VCH)>();
-        if constexpr (FEAT & BARRIER) {
+        constexpr int EVERY = (FEAT & EVERY2) ? 2 : (FEAT & EVERY4) ? 4 : 1;
+        if ((FEAT & BARRIER) && t % EVERY == 0) {
             const unsigned long long b0 = __builtin_readcyclecounter();
             __builtin_amdgcn_s_barrier();
             at_barrier += __builtin_readcyclecounter() - b0;
@@ -320,6 +321,8 @@ int main() {
     if (run_loop<8, 2, FRAG>("+ LDS fragment reads", 256)) return 1;
     if (run_loop<8, 2, FRAG | COPY>("+ tile copies", 256)) return 1;
     if (run_loop<8, 2, FRAG | COPY | BARRIER>("+ workgroup barrier per tile (the kernel's loop)", 256)) return 1;
+    if (run_loop<8, 2, FRAG | COPY | BARRIER | EVERY2>("   barrier in every 2nd tile only (timing only: the rings are not that deep)", 256)) return 1;
+    if (run_loop<8, 2, FRAG | COPY | BARRIER | EVERY4>("   barrier in every 4th tile only", 256)) return 1;
     if (run_loop<4, 1, FRAG | COPY | BARRIER>("128-row workgroups, one per CU (one wave per SIMD)", 256)) return 1;
     if (run_loop<4, 1, FRAG | COPY | BARRIER>("128-row workgroups, two per CU", 512)) return 1;
     if (run_loop<4, 2, FRAG | COPY | BARRIER, 2>("64 rows per wave, 4 waves (one per SIMD), every fragment used twice", 256)) return 1;
