@@ -113,11 +113,12 @@ def summarize_traffic(dirs):
     f_scale, w_scale = copy_kib / fetch_copy, copy_kib / write_copy
     total = int(round((fetch * f_scale + write * w_scale) * 1024.0))
     print("# HBM traffic of sage_attn_kernel per launch, rocprofv3 --pmc (one counter per run)")
-    print("# Commands (repository root on the MI355X box, after `cd /tmp && export TMPDIR=/tmp` and back), C = FETCH_SIZE, then WRITE_SIZE:")
-    print("#   rocprofv3 --pmc C --output-format csv -d gpurun_out/pmc_C_bench -o p -- python3 bench.py --skip-cpu-baseline --steps 3 --warmup 2")
-    print("#   rocprofv3 --pmc C --output-format csv -d gpurun_out/pmc_C_copy -o p -- python3 bench.py --copy-calibration")
-    print("#   python3 bench.py --summarize-traffic gpurun_out/pmc_FETCH_SIZE_bench gpurun_out/pmc_WRITE_SIZE_bench "
-          "gpurun_out/pmc_FETCH_SIZE_copy gpurun_out/pmc_WRITE_SIZE_copy")
+    print("# Commands (repository root on the MI355X box, after `cd /tmp && export TMPDIR=/tmp` and back; OUT = any "
+          "scratch directory), C = FETCH_SIZE, then WRITE_SIZE:")
+    print("#   rocprofv3 --pmc C --output-format csv -d OUT/pmc_C_bench -o p -- python3 bench.py --skip-cpu-baseline --steps 3 --warmup 2")
+    print("#   rocprofv3 --pmc C --output-format csv -d OUT/pmc_C_copy -o p -- python3 bench.py --copy-calibration")
+    print("#   python3 bench.py --summarize-traffic OUT/pmc_FETCH_SIZE_bench OUT/pmc_WRITE_SIZE_bench "
+          "OUT/pmc_FETCH_SIZE_copy OUT/pmc_WRITE_SIZE_copy")
     print("kernel_source_digest = %s" % kernel_source_digest())
     print("fetch_size_kib_per_dispatch = %.1f   # %d dispatches" % (fetch, n_f))
     print("write_size_kib_per_dispatch = %.1f   # %d dispatches" % (write, n_w))
