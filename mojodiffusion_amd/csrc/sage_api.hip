@@ -125,19 +125,17 @@ ScratchCarve scratch_carve(int B, int H, int Nkv, int D) {
 // so the retired buffers of a stream add up to less than its current one.  Allocation is not
 // possible while the stream is being captured into a graph: such a call fails with
 // MI355_SAGE_EWORKSPACE unless the buffer is already large enough.
-struct StreamWs;
-std::vector<StreamWs>& sage_api_ws();
 std::mutex g_ws_mutex;
 struct StreamWs { int dev; hipStream_t stream; void* p; size_t bytes; };
 std::vector<StreamWs> g_ws;          // one-shot calls
 std::vector<StreamWs> g_split_ws;    // hand-over slots of mi355_sage_attn_fwd, which takes no workspace
 
-int internal_workspace(size_t need, hipStream_t stream, void** out, std::vector<StreamWs>& g_ws = sage_api_ws()) {
+int internal_workspace(std::vector<StreamWs>& registry, size_t need, hipStream_t stream, void** out) {
     int dev = 0;
     SAGE_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     StreamWs* w = nullptr;
-    for (auto& e : g_ws)
+    for (auto& e : registry)
         if (e.dev == dev && e.stream == stream) { w = &e; break; }
     if (w == nullptr || w->bytes < need) {
         hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -150,8 +148,8 @@ int internal_workspace(size_t need, hipStream_t stream, void** out, std::vector<
         void* p = nullptr;
         SAGE_HIP(hipMalloc(&p, bytes));
         if (w == nullptr) {
-            g_ws.push_back(StreamWs{dev, stream, p, bytes});
-            w = &g_ws.back();
+            registry.push_back(StreamWs{dev, stream, p, bytes});
+            w = &registry.back();
         } else {
             w->p = p;              // the old buffer stays allocated (see above)
             w->bytes = bytes;
@@ -160,7 +158,6 @@ int internal_workspace(size_t need, hipStream_t stream, void** out, std::vector<
     *out = w->p;
     return 0;
 }
-std::vector<StreamWs>& sage_api_ws() { return g_ws; }
 
 // The optional ops in front of the quantizers (RMSNorm + interleaved RoPE of Q and of K).
 struct Pre {
@@ -330,7 +327,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         if (reinterpret_cast<uintptr_t>(ws) & (kAlign - 1)) return MI355_SAGE_EUNSUPPORTED;
     } else {
         void* p = nullptr;
-        if ((rc = internal_workspace(c.total, st, &p))) return rc;
+        if ((rc = internal_workspace(g_ws, c.total, st, &p))) return rc;
         ws = static_cast<uint8_t*>(p);
     }
     QuantOut o{};
@@ -668,7 +665,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     // Same scheduling, hence the same bits, as the one-shot calls: shapes that are split over a
     // fixed number of workgroups need hand-over slots, kept per (device, stream) by the library.
     const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid), D);
-    if (split_bytes > 0 && (rc = internal_workspace(split_bytes, static_cast<hipStream_t>(stream), &a.split, g_split_ws))) return rc;
+    if (split_bytes > 0 && (rc = internal_workspace(g_split_ws, split_bytes, static_cast<hipStream_t>(stream), &a.split))) return rc;
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
 }
@@ -740,7 +737,7 @@ int mi355_sage_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const 
     const BwdCarve c = bwd_carve(B, H, N_q, N_kv, D);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (workspace == nullptr) {
-        if ((rc = internal_workspace(c.total, st, &workspace))) return rc;
+        if ((rc = internal_workspace(g_ws, c.total, st, &workspace))) return rc;
     } else if (workspace_bytes < c.total || (reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1))) {
         SAGE_LOG("backward workspace: %zu bytes at a 256-byte boundary needed, %zu given", c.total, workspace_bytes);
         return MI355_SAGE_EWORKSPACE;
