@@ -1,0 +1,115 @@
+"""The gates of the reference's probe for its memory-efficient SDPA
+(serenitymojo/ops/sdpa_tiled_probe.mojo), on the quantized path: the probe's own deterministic
+inputs (`_pseudo`, :41-44), shapes and bars (cos >= 0.999, :101, :144, :183), with the fp32 SDPA
+as the trusted side where the probe uses its math-mode kernels.
+
+  gate 1   sdpa_nomask_tiled and sdpa_tiled (random additive [B,H,S,S] mask) at S=1536, Dh=128, H=3
+  gate 1b  sdpa_cross_nomask (Sq=1536, Skv=1024) against the square call on zero-padded K/V with a
+           -1e30 mask on the padded keys
+  gate 1c  sdpa_cross_masked with a random [B,H,Sq,Skv] mask against the padded square call
+  bf16     the same masked / rectangular calls with BF16 storage at S=64, Dh=64, Skv=48: BF16 out
+  gate 2   S=8192 completes with a finite output of the right shape
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+COS = 0.999
+
+
+def _pseudo(n, salt):
+    """sdpa_tiled_probe.mojo:41-44: deterministic values in about [-1, 1]."""
+    i = np.arange(n, dtype=np.int64)
+    x = (i * 2654435761 + salt * 40503 + 12345) % 100003
+    return ((x.astype(np.float32) / np.float32(100003.0)) - np.float32(0.5)) * np.float32(2.0)
+
+
+def _cos_ratio(a, b):
+    a, b = a.double().reshape(-1), b.double().reshape(-1)
+    return float(a @ b / (a.norm() * b.norm() + 1e-30)), float(a.norm() / (b.norm() + 1e-30))
+
+
+def _referee(q, k, v, scale, mask=None):
+    """fp32 softmax(q k^T scale + mask) v on [B,S,H,Dh] tensors."""
+    import torch
+    qq, kk, vv = (t.float().permute(0, 2, 1, 3) for t in (q, k, v))
+    s = torch.matmul(qq, kk.transpose(-1, -2)) * scale
+    if mask is not None:
+        s = s + mask.float()
+    return torch.matmul(torch.softmax(s, dim=-1), vv).permute(0, 2, 1, 3)
+
+
+def _dev(x, shape, dtype):
+    import torch
+    return torch.from_numpy(x.reshape(shape)).cuda().to(dtype)
+
+
+@pytest.mark.parametrize("storage", ["f32", "bf16"])
+def test_probe_gates(storage):
+    import torch
+    from mojodiffusion_amd import attention_sage as A
+    big = storage == "f32"
+    dt = torch.float32 if big else torch.bfloat16
+    B, S, H, Dh, Skv = (1, 1536, 3, 128, 1024) if big else (1, 64, 2, 64, 48)
+    salts = (1, 2, 3, 7, 17, 19, 23) if big else (31, 32, 33, 34, 35, 36, 37)
+    amp_sq, amp_rect = (2.0, 1.5) if big else (1.25, 1.25)
+    scale = 1.0 / float(np.sqrt(Dh))
+    n = B * S * H * Dh
+    q, k, v = (_dev(_pseudo(n, s) * np.float32(0.5), (B, S, H, Dh), dt) for s in salts[:3])
+
+    # gate 1: no mask, and a random additive mask
+    got = A.sdpa_nomask_tiled(q, k, v, scale)
+    assert got.dtype == dt and got.shape == q.shape
+    cos, ratio = _cos_ratio(got, _referee(q, k, v, scale))
+    assert cos >= COS and abs(ratio - 1.0) < 2e-2, (cos, ratio)
+    mask = _dev(_pseudo(B * H * S * S, salts[3]) * np.float32(amp_sq), (B, H, S, S), dt)
+    got = A.sdpa_tiled(q, k, v, mask, scale)
+    assert got.dtype == dt
+    cos, ratio = _cos_ratio(got, _referee(q, k, v, scale, mask))
+    assert cos >= COS and abs(ratio - 1.0) < 2e-2, (cos, ratio)
+    np.testing.assert_array_equal(got.float().cpu().numpy(), A.sdpa(q, k, v, mask, scale).float().cpu().numpy())
+
+    # gate 1b: rectangular against the padded square call with the padded keys masked
+    ks, vs = (_dev(_pseudo(B * Skv * H * Dh, s) * np.float32(0.5), (B, Skv, H, Dh), dt) for s in salts[4:6])
+    k_pad, v_pad = torch.zeros_like(q), torch.zeros_like(q)
+    k_pad[:, :Skv], v_pad[:, :Skv] = ks, vs
+    cross_mask = torch.zeros((B, H, S, S), dtype=dt, device="cuda")
+    cross_mask[..., Skv:] = -1.0e30
+    rect = A.sdpa_cross_nomask(q, ks, vs, scale)
+    padded = A.sdpa(q, k_pad, v_pad, cross_mask, scale)
+    ref = _referee(q, ks, vs, scale)
+    for name, t in (("rect", rect), ("padded", padded)):
+        assert t.dtype == dt and torch.isfinite(t.float()).all(), name
+        cos, ratio = _cos_ratio(t, ref)
+        assert cos >= COS and abs(ratio - 1.0) < 2e-2, (name, cos, ratio)
+    cos, ratio = _cos_ratio(rect, padded)
+    assert cos >= COS, (cos, ratio)
+
+    # gate 1c: masked rectangular against the padded square call
+    rect_mask = _dev(_pseudo(B * H * S * Skv, salts[6]) * np.float32(amp_rect), (B, H, S, Skv), dt)
+    padded_mask = torch.full((B, H, S, S), -1.0e30, dtype=dt, device="cuda")
+    padded_mask[..., :Skv] = rect_mask
+    rect_m = A.sdpa_cross_masked(q, ks, vs, rect_mask, scale)
+    padded_m = A.sdpa(q, k_pad, v_pad, padded_mask, scale)
+    ref = _referee(q, ks, vs, scale, rect_mask)
+    assert rect_m.dtype == dt
+    for name, t in (("rect", rect_m), ("padded", padded_m)):
+        cos, ratio = _cos_ratio(t, ref)
+        assert cos >= COS and abs(ratio - 1.0) < 2e-2, (name, cos, ratio)
+    cos, ratio = _cos_ratio(rect_m, padded_m)
+    assert cos >= COS, (cos, ratio)
+
+
+def test_probe_gate_2_large_s_completes():
+    """S=8192, Dh=128: the math path's [S,S] score slab is what the tiled path exists to avoid."""
+    import torch
+    from mojodiffusion_amd import attention_sage as A
+    B, S, H, Dh = 1, 8192, 4, 128
+    n = B * S * H * Dh
+    q, k, v = (_dev(_pseudo(n, s) * np.float32(0.5), (B, S, H, Dh), torch.float32) for s in (41, 42, 43))
+    got = A.sdpa_nomask_tiled(q, k, v, 1.0 / float(np.sqrt(Dh)))
+    torch.cuda.synchronize()
+    assert got.shape == (B, S, H, Dh) and got.dtype == torch.float32 and torch.isfinite(got).all()
+    cos, ratio = _cos_ratio(got[:, :512], _referee(q[:, :512], k, v, 1.0 / float(np.sqrt(Dh))))
+    assert cos >= COS, (cos, ratio)
