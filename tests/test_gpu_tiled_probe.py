@@ -113,3 +113,32 @@ def test_probe_gate_2_large_s_completes():
     assert got.shape == (B, S, H, Dh) and got.dtype == torch.float32 and torch.isfinite(got).all()
     cos, ratio = _cos_ratio(got[:, :512], _referee(q[:, :512], k, v, 1.0 / float(np.sqrt(Dh))))
     assert cos >= COS, (cos, ratio)
+
+
+@pytest.mark.parametrize("Dh", [128, 64])
+def test_reviewer_cases_causal_mask_and_fully_masked_row(Dh):
+    """The cases of ops/parity/SKEPTIC_FINDINGS_TILED_SDPA_2026-06-03.md: a causal additive mask
+    (0 if j <= i else -1e30 — not symmetric, so a transposed mask read fails it), the same with row 0
+    masked everywhere (finite large-negative bias: every key ties, the row is the mean of V, no NaN),
+    at Dh = 128 and Dh = 64, S = 1536."""
+    import torch
+    from mojodiffusion_amd import attention_sage as A
+    B, S, H = 1, 1536, 3
+    scale = 1.0 / float(np.sqrt(Dh))
+    n = B * S * H * Dh
+    q, k, v = (_dev(_pseudo(n, s) * np.float32(0.5), (B, S, H, Dh), torch.float32) for s in (1, 2, 3))
+    i = torch.arange(S, device="cuda")
+    causal = torch.where(i[None, :] <= i[:, None], 0.0, -1.0e30).to(torch.float32).expand(B, H, S, S).contiguous()
+    got = A.sdpa_tiled(q, k, v, causal, scale)
+    assert torch.isfinite(got).all()
+    cos, ratio = _cos_ratio(got, _referee(q, k, v, scale, causal))
+    assert cos >= COS and abs(ratio - 1.0) < 2e-2, (cos, ratio)
+    # the first rows see one, two, three keys: sharp cases of the same check
+    np.testing.assert_allclose(got[:, 0].cpu().numpy(), v[:, 0].to(torch.bfloat16).float().cpu().numpy(), atol=4e-3)
+    masked_row = causal.clone()
+    masked_row[:, :, 0, :] = -1.0e30
+    got = A.sdpa_tiled(q, k, v, masked_row, scale)
+    assert torch.isfinite(got).all()
+    np.testing.assert_allclose(got[:, 0].cpu().numpy(), v.mean(dim=1).cpu().numpy(), atol=2e-3)
+    cos, ratio = _cos_ratio(got[:, 1:], _referee(q, k, v, scale, causal)[:, 1:])
+    assert cos >= COS, (cos, ratio)
