@@ -142,3 +142,34 @@ def test_reviewer_cases_causal_mask_and_fully_masked_row(Dh):
     np.testing.assert_allclose(got[:, 0].cpu().numpy(), v.mean(dim=1).cpu().numpy(), atol=2e-3)
     cos, ratio = _cos_ratio(got[:, 1:], _referee(q, k, v, scale, causal)[:, 1:])
     assert cos >= COS, (cos, ratio)
+
+
+@pytest.mark.parametrize("storage", ["f32", "bf16"])
+def test_qwen_keymask_parity_gate(storage):
+    """ops/parity/sdpa_qwen_keymask_parity.mojo: the in-kernel mask of the padded text keys
+    [real_txt_len, N_TXT) against the full [B,H,S,S] additive mask (-1e4 on those columns), on
+    that file's fills ((7i)%17, (5i)%19, (3i)%13), S=7, H=2, N_TXT=4, real_txt_len=2, in F32 and
+    BF16 storage, and the case without padding (real_txt_len == N_TXT) against a zero mask.  The
+    reference runs it at Dh=8; the kernels here start at Dh=64."""
+    import torch
+    from mojodiffusion_amd import attention_sage as A
+    dt = torch.float32 if storage == "f32" else torch.bfloat16
+    B, S, H, Dh, N_TXT = 1, 7, 2, 64, 4
+    scale = 1.0 / float(np.sqrt(Dh))
+    i = np.arange(B * S * H * Dh, dtype=np.int64)
+    q = _dev((((i * 7) % 17).astype(np.float32) - 8.0) * np.float32(0.07), (B, S, H, Dh), dt)
+    k = _dev((((i * 5) % 19).astype(np.float32) - 9.0) * np.float32(0.06), (B, S, H, Dh), dt)
+    v = _dev((((i * 3) % 13).astype(np.float32) - 6.0) * np.float32(0.05), (B, S, H, Dh), dt)
+    for real in (2, N_TXT):
+        full_mask = torch.zeros((B, H, S, S), dtype=dt, device="cuda")
+        full_mask[..., real:N_TXT] = -1.0e4
+        full = A.sdpa(q, k, v, full_mask, scale)
+        key = A.sdpa_qwen_keymask(q, k, v, N_TXT, real, scale)
+        assert key.dtype == dt and full.dtype == dt
+        ref = _referee(q, k, v, scale, full_mask)
+        for name, t in (("keymask", key), ("full mask", full)):
+            cos, ratio = _cos_ratio(t, ref)
+            assert cos >= COS and abs(ratio - 1.0) < 2e-2, (name, real, cos, ratio)
+        # serenitymojo/parity.mojo:41-106: cosine >= 0.999 and a max-abs bar between the two paths
+        cos, _ = _cos_ratio(key, full)
+        assert cos >= 0.9999 and (key.float() - full.float()).abs().max() <= 2e-2, (real, cos)
