@@ -1,7 +1,7 @@
 """A gate shaped like the reference's own acceptance test for a new attention backend
 (serenitymojo/ops/tests/sdpa_flash_parity.mojo): the trainer shapes, the same generator for the
-inputs, agreement with the incumbent, an fp32 referee on the same bf16-rounded values, and speed.
-The incumbent here is a bf16 attention with explicit matmuls and an fp32 softmax (what the
+inputs, agreement with the incumbent, an fp32 referee on the same bf16-rounded values, and speed —
+forward, and backward on the saved forward set.  The incumbent here is a bf16 attention with explicit matmuls and an fp32 softmax (what the
 reference's math-mode path computes, ops/attention.mojo:332-463); the referee is the same in fp32."""
 import time
 
@@ -94,4 +94,36 @@ def test_gate_like_the_reference_flash_gate(name, B, S, H, Dh):
     t_math = timeit(lambda: math_mode(q, k, v, torch.bfloat16))
     t_sage = timeit(lambda: A.sdpa_nomask(q, k, v, scale))
     print("GATE sdpa_sage %s speed: sage %.3f ms, math-mode %.3f ms" % (name, t_sage * 1e3, t_math * 1e3))
+    assert t_sage < t_math
+
+    # ---- backward, as the reference's gate has it (:160-181): d_out from seed 44; the flash
+    # backward on the saved forward set against the math-mode backward in bf16 (cos >= 0.999) and,
+    # against the fp32 gradients, not worse than 1.5x the bf16 incumbent.  (Measured ratios 0.80-0.96.)
+    d_o = G.dev_bf16(f32_to_bf16_bits(_pattern(n, 44, 1.0)).reshape(B, S, H, Dh))
+
+    def math_bwd(dt):
+        qq, kk, vv = (x.to(dt).clone().requires_grad_(True) for x in (q, k, v))
+        qh, kh, vh = (x.permute(0, 2, 1, 3) for x in (qq, kk, vv))
+        p = torch.softmax((qh @ kh.transpose(-1, -2)).float() * scale, dim=-1)
+        ((p.to(dt) @ vh).permute(0, 2, 1, 3)).backward(d_o.to(dt))
+        return qq.grad, kk.grad, vv.grad
+
+    def sage_fwd_bwd():
+        fwd = A.sdpa_flash_train_fwd(q, k, v, scale)
+        return A.sdpa_flash_backward(fwd, d_o, scale)
+
+    g_math, g_ref, g = math_bwd(torch.bfloat16), math_bwd(torch.float32), sage_fwd_bwd()
+    torch.cuda.synchronize()
+    for which, g_sage in (("d_q", g.d_q), ("d_k", g.d_k), ("d_v", g.d_v)):
+        i = ("d_q", "d_k", "d_v").index(which)
+        cos_m, _, _ = _agree(g_sage, g_math[i])
+        _, _, rms_sage = _agree(g_sage, g_ref[i])
+        _, _, rms_math = _agree(g_math[i], g_ref[i])
+        print("GATE sdpa_sage %s bwd %s sage-vs-math cos=%.6f | rms_vs_f32: sage=%.3e math=%.3e"
+              % (name, which, cos_m, rms_sage, rms_math))
+        assert cos_m >= 0.999, (which, cos_m)
+        assert rms_sage <= 1.5 * rms_math + 1e-7, (which, rms_sage, rms_math)
+    t_math = timeit(lambda: math_bwd(torch.bfloat16))
+    t_sage = timeit(sage_fwd_bwd)
+    print("GATE sdpa_sage %s speed fwd+bwd: sage %.3f ms, math-mode %.3f ms" % (name, t_sage * 1e3, t_math * 1e3))
     assert t_sage < t_math
