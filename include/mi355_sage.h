@@ -346,8 +346,8 @@ int mi355_sage_set_attn_split(int mode);
  * library's per-stream buffer (same rules as the forward).  Unlike the pair handed to cuDNN, O and
  * Stats may come from the quantized forward: the probabilities recomputed here are then not quite
  * the ones O and Stats belong to, and a row of dS no longer sums to zero exactly.  dQ is therefore
- * taken as scale * dS (K - c) with c close to the mean key — the same value for a consistent
- * forward, and free of the keys' common offset times that row sum otherwise. */
+ * taken as scale * (dS K - rowsum(dS) c) with c close to the mean key — the same value for a
+ * consistent forward, and free of the keys' common offset times that row sum otherwise. */
 size_t mi355_sage_bwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D);
 int mi355_sage_sdpa_bwd_bf16(
     const void* Q, const void* K, const void* V, const void* O, const void* dO, const void* Stats,

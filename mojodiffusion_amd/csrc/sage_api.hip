@@ -677,7 +677,7 @@ int mi355_sage_set_attn_split(int mode) {
 }
 
 // ---- backward ---------------------------------------------------------------------------------
-struct BwdCarve { size_t kT, qT, doT, lse2, delta, total; };
+struct BwdCarve { size_t kT, qT, doT, lse2, delta, kcen, total; };
 static BwdCarve bwd_carve(int B, int H, int Nq, int Nkv, int D) {
     const size_t bh = (size_t)B * H;
     const size_t nqp = (size_t)pad_to(Nq, 64), nkp = (size_t)pad_to(Nkv, 64);
@@ -689,6 +689,7 @@ static BwdCarve bwd_carve(int B, int H, int Nq, int Nkv, int D) {
     c.doT = take(bh * nqp * D * 2);
     c.lse2 = take(bh * nqp * sizeof(float));
     c.delta = take(bh * nqp * sizeof(float));
+    c.kcen = take(bh * D * sizeof(float));
     c.total = off;
     return c;
 }
@@ -762,6 +763,7 @@ int mi355_sage_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const 
     a.doT = reinterpret_cast<uint16_t*>(ws + c.doT);
     a.lse2 = reinterpret_cast<float*>(ws + c.lse2);
     a.delta = reinterpret_cast<float*>(ws + c.delta);
+    a.kcen = reinterpret_cast<float*>(ws + c.kcen);
     a.nq_pad = pad_to(N_q, 64);
     a.nkv_pad = pad_to(N_kv, 64);
     SAGE_HIP(launch_bwd(a, st));

@@ -10,9 +10,9 @@
 //   1. bwd_prep_kernel     Delta and Stats * log2(e) per query row (padding rows: +inf, so their
 //                          probabilities vanish), and transposed copies K^T, Q^T, dO^T in tiles of
 //                          64 rows whose rows sit in the slot order of the matrix instruction's
-//                          operand layout (v_slot_f16).  K^T holds the keys minus (nearly) their
-//                          mean: dQ = scale * dS (K - c) for any constant vector c.
-//   2. bwd_pass_kernel<0>  owner = 256 query rows per workgroup (8 waves), loop over key tiles  -> dQ
+//                          operand layout (v_slot_f16); and a vector c close to the mean key.
+//   2. bwd_pass_kernel<0>  owner = 256 query rows per workgroup (8 waves), loop over key tiles  -> dQ,
+//                          as scale * (dS K - rowsum(dS) c) = scale * dS (K - c)
 //   3. bwd_pass_kernel<1>  owner = 128 keys per workgroup (4 waves), loop over query tiles     -> dK, dV
 // In both passes a wave owns 32 rows ("x"), keeps their two bf16 row blocks resident as B operands
 // and walks the other side ("y") in tiles of 64 rows staged in LDS by register-bypassing copies,
@@ -28,6 +28,7 @@ namespace sage {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
@@ -90,7 +91,6 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
     constexpr int CPR = D / 8;
     constexpr int LROW = D + 8;                     // LDS row stride in elements (keeps 16-byte alignment, spreads banks)
     __shared__ __attribute__((aligned(16))) uint16_t tile[64 * LROW];
-    __shared__ float kcen[D];
     const int ntk = (int)(a.nkv_pad / 64), ntq = (int)(a.nq_pad / 64);
     const int per_bh = ntk + 3 * ntq;
     const int bh = blockIdx.x / per_bh;
@@ -133,16 +133,18 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
     uint16_t* dst;
     int valid, t;
     int64_t ntiles;
-    const bool centre = r < ntk;
+    const bool is_k = r < ntk;
     if (r < ntk) { src = a.k; dst = a.kT; valid = a.valid_kv; t = r; ntiles = ntk; }
     else if (r < ntk + ntq) { src = a.q; dst = a.qT; valid = a.valid_q; t = r - ntk; ntiles = ntq; }
     else { src = a.dout; dst = a.doT; valid = a.valid_q; t = r - ntk - ntq; ntiles = ntq; }
     const uint16_t* sp = src.p + b * src.sb + h * src.sh;
-    // K^T holds the keys minus a vector close to their mean (the mean of 64 keys spread evenly over
-    // the valid ones, the same in every workgroup of the head): rows of dS sum to zero, so dS K is
-    // unchanged by it in exact arithmetic, and when O and Stats come from a forward of other
-    // precision the small non-zero row sum is no longer multiplied by the keys' common offset.
-    if (centre) {
+    // Rows of dS sum to zero in exact arithmetic, so dS K = dS (K - c) for any vector c; when O and
+    // Stats come from a forward of other precision the row sum is small but not zero, and dS K
+    // would multiply it by the keys' common offset.  The dQ pass therefore also sums every row of
+    // dS (the rounded values the matrix instruction takes) and subtracts rowsum * c at the end,
+    // with c close to the mean key: the mean of 64 keys spread evenly over the valid ones, computed
+    // here once per head.  (Centring the K^T copy itself would round K - c to bf16 a second time.)
+    if (is_k && t == 0) {
         float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < 64 * CPR / 256; i++) {
@@ -161,11 +163,11 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; e++) red[(tid / CPR) * D + (tid % CPR) * 8 + e] = part[e];
         __syncthreads();
-        float sum = 0.0f;
-        if (tid < D)
+        if (tid < D) {
+            float sum = 0.0f;
             for (int g = 0; g < 256 / CPR; g++) sum += red[g * D + tid];
-        __syncthreads();
-        if (tid < D) kcen[tid] = sum * (1.0f / 64.0f);
+            a.kcen[(int64_t)bh * D + tid] = sum * (1.0f / 64.0f);
+        }
         __syncthreads();
     }
 #pragma unroll
@@ -173,15 +175,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
         const int c = i * 256 + tid;
         const int row = c / CPR, col = (c % CPR) * 8;
         u32x4 w = {0u, 0u, 0u, 0u};
-        if (t * 64 + row < valid) {
-            w = *reinterpret_cast<const u32x4*>(sp + (int64_t)(t * 64 + row) * src.sn + col);
-            if (centre) {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    w[e] = pack_bf16(__uint_as_float(w[e] << 16) - kcen[col + 2 * e],
-                                     __uint_as_float(w[e] & 0xFFFF0000u) - kcen[col + 2 * e + 1]);
-            }
-        }
+        if (t * 64 + row < valid) w = *reinterpret_cast<const u32x4*>(sp + (int64_t)(t * 64 + row) * src.sn + col);
         *reinterpret_cast<u32x4*>(&tile[row * LROW + col]) = w;
     }
     __syncthreads();
@@ -254,6 +248,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
         }
     }
     float lse_x = 0.0f, delta_x = 0.0f;
+    float ds_rowsum = 0.0f;                         // dQ pass: sum over the keys of this lane's dS values
     if constexpr (PASS == 0) {
         const int64_t idx = (int64_t)bh * a.nq_pad + min((int64_t)x, a.nq_pad - 1);
         lse_x = a.lse2[idx];
@@ -399,6 +394,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
                 ds[e] = pr[e] * (gacc[blk][i + e] - dl[(i & 3) + e]);
             }
             sp[blk][i >> 1] = pack_bf16(ds[0], ds[1]);
+            // dQ pass: this lane's share of the row sum of dS, over the rounded values
+            if constexpr (PASS == 0)
+                ds_rowsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, sp[blk][i >> 1]),
+                                                            __builtin_bit_cast(v2bf, 0x3F803F80u), ds_rowsum, false);
             if constexpr (PASS == 1) pp[blk][i >> 1] = pack_bf16(pr[0], pr[1]);
         };
         // matrix instruction m of a block's accumulation: dX1^T += Y1^T . dS  (and dX2^T += Y2^T . P)
@@ -449,6 +448,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
         uint16_t* o1 = (PASS == 0 ? a.dq : a.dk) + b * (PASS == 0 ? a.dq_sb : a.dk_sb) + h * (PASS == 0 ? a.dq_sh : a.dk_sh) +
                        (int64_t)x * (PASS == 0 ? a.dq_sn : a.dk_sn);
         uint16_t* o2 = PASS == 1 ? a.dv + b * a.dv_sb + h * a.dv_sh + (int64_t)x * a.dv_sn : nullptr;
+        // dQ = scale * (dS K - rowsum(dS) c): the two half-waves hold different keys of the same query
+        float rs = 0.0f;
+        if constexpr (PASS == 0) {
+            const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(ds_rowsum), __float_as_uint(ds_rowsum), false, false);
+            rs = __uint_as_float(r.x) + __uint_as_float(r.y);
+        }
+        const float* cen = a.kcen + (int64_t)bh * D;
 #pragma unroll
         for (int d = 0; d < DB; d++)
 #pragma unroll
@@ -456,8 +462,16 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
                 const int ch = d * 32 + g * 8 + half * 4;
                 u32x2 w = {0u, 0u};
                 if (live) {
-                    w.x = pack_bf16(acc1[d][g * 4] * a.scale, acc1[d][g * 4 + 1] * a.scale);
-                    w.y = pack_bf16(acc1[d][g * 4 + 2] * a.scale, acc1[d][g * 4 + 3] * a.scale);
+                    float y[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) y[e] = acc1[d][g * 4 + e];
+                    if constexpr (PASS == 0) {
+                        const v4f c4 = *reinterpret_cast<const v4f*>(cen + ch);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) y[e] -= rs * c4[e];
+                    }
+                    w.x = pack_bf16(y[0] * a.scale, y[1] * a.scale);
+                    w.y = pack_bf16(y[2] * a.scale, y[3] * a.scale);
                 }
                 *reinterpret_cast<u32x2*>(o1 + ch) = w;
                 if constexpr (PASS == 1) {

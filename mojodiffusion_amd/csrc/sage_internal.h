@@ -137,6 +137,7 @@ struct BwdArgs {
     // workspace
     uint16_t *kT, *qT, *doT;                     // [B,H,n_pad/64,D,64] bf16, rows in v_slot_f16 order, zero past valid
     float *lse2, *delta;                         // [B,H,nq_pad]: Stats*log2(e) (+inf past valid), rowsum(dO*O)
+    float* kcen;                                 // [B,H,D]: a vector close to the mean key (see sage_bwd.hip)
     int64_t nq_pad, nkv_pad;                     // multiples of 64
 };
 hipError_t launch_bwd(const BwdArgs& a, hipStream_t st);
