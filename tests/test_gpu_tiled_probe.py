@@ -173,3 +173,31 @@ def test_qwen_keymask_parity_gate(storage):
         # serenitymojo/parity.mojo:41-106: cosine >= 0.999 and a max-abs bar between the two paths
         cos, _ = _cos_ratio(key, full)
         assert cos >= 0.9999 and (key.float() - full.float()).abs().max() <= 2e-2, (real, cos)
+
+
+def test_reference_golden_dh128_through_the_gpu_path():
+    """ops/parity/sdpa_math_parity.mojo on the GPU path: the reference's golden output for its
+    closed-form inputs at [1,8,32,128] (ops/parity/sdpa_math_ref.txt, tag dh128; H=32 BSHD
+    indexing), and `sdpa_nomask` against `sdpa` with a zero mask (:136-237).  F32 storage in, as the
+    reference test has it; the bars of the quantized path: cosine >= 0.999, max-abs <= 2e-2."""
+    import os
+    import torch
+    from mojodiffusion_amd import attention_sage as A
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sdpa_math_ref.npz"))["dh128"]
+    B, S, H, D = 1, 8, 32, 128
+    i = np.arange(B * S * H * D, dtype=np.int64)
+    q = _dev((((i * 7) % 13).astype(np.float32) - 6.0) * np.float32(0.05), (B, S, H, D), torch.float32)
+    k = _dev((((i * 5) % 11).astype(np.float32) - 5.0) * np.float32(0.05), (B, S, H, D), torch.float32)
+    v = _dev((((i * 3) % 9).astype(np.float32) - 4.0) * np.float32(0.05), (B, S, H, D), torch.float32)
+    scale = 1.0 / float(np.sqrt(D))
+    want = torch.from_numpy(gold.reshape(B, S, H, D)).cuda()
+    got = A.sdpa_nomask(q, k, v, scale)
+    assert got.dtype == torch.float32
+    cos, ratio = _cos_ratio(got, want)
+    assert cos >= COS and float((got - want).abs().max()) <= 2e-2, (cos, ratio, float((got - want).abs().max()))
+    zero = torch.zeros((B, H, S, S), dtype=torch.float32, device="cuda")
+    masked = A.sdpa(q, k, v, zero, scale)
+    cos, _ = _cos_ratio(masked, got)
+    assert cos >= 0.9999 and float((masked - got).abs().max()) <= 1e-2, cos
+    cos, _ = _cos_ratio(masked, want)
+    assert cos >= COS, cos
