@@ -331,6 +331,14 @@ int mi355_sage_attn_fwd(
  * the first such call of a stream, never while that stream is being captured). */
 int mi355_sage_set_attn_split(int mode);
 
+/* How long a workgroup of the split schedule polls for another workgroup's partial result before
+ * it gives up and writes NaN into its rows (the launch never hangs; no counterpart in the
+ * reference).  polls > 0: that many polls of about a microsecond (default 262144; the longest
+ * wait that can legitimately occur is one row tile's worth of work, a few milliseconds); 0: back
+ * to the default; polls < 0: test mode — no workgroup announces its result and every waiting one
+ * gives up after -polls polls, which is how the give-up path is exercised without a hang. */
+int mi355_sage_set_attn_split_wait(int polls);
+
 /* Backward.  Replaces flame_cudnn_sdpa_bwd_bf16 (serenitymojo/ops/cshim/cudnn_sdpa_bwd.cpp:325-347;
  * Mojo callers ops/attention_flash.mojo:345-433, :478-535, :538-607): identical parameter list up
  * to `stream`, then the workspace pair.  Q, K, V, O, dO bf16 and dQ, dK, dV bf16, each a logical

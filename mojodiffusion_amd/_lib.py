@@ -50,6 +50,7 @@ SIGNATURES = {
     "mi355_sage_attn_fwd": (_int, [_vp, _vp, _int, _vp, _vp, _int, _vp, _vp, _int] + [_int] * 8
                             + [_vp, _i64p, _i64, _vp, _vp, _vp]),
     "mi355_sage_set_attn_split": (_int, [_int]),
+    "mi355_sage_set_attn_split_wait": (_int, [_int]),
     "mi355_sage_version": (ctypes.c_char_p, []),
 }
 

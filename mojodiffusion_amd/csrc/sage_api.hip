@@ -676,6 +676,12 @@ int mi355_sage_set_attn_split(int mode) {
     return MI355_SAGE_OK;
 }
 
+int mi355_sage_set_attn_split_wait(int polls) {
+    if (polls < -(1 << 24) || polls > (1 << 24)) return MI355_SAGE_EINVAL;
+    attn_split_wait(polls);
+    return MI355_SAGE_OK;
+}
+
 // ---- backward ---------------------------------------------------------------------------------
 struct BwdCarve { size_t kT, qT, doT, lse2, delta, kcen, total; };
 static BwdCarve bwd_carve(int B, int H, int Nq, int Nkv, int D) {

@@ -132,7 +132,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     uint16_t* __restrict__ o, int64_t osb, int64_t osh, int64_t osn,
     float* __restrict__ stats, int n_qtiles, int total_wg,
     const uint16_t* __restrict__ amask, int64_t amb, int64_t amh, int64_t amn,
-    int split_groups, float* split_part, int* split_flags) {
+    int split_groups, float* split_part, int* split_flags, int split_wait) {
     constexpr int VB = (VARIANT == 0) ? 2 : 1;          // bytes per V element
     constexpr int KSTEPS = D / 32;                      // int8 MFMA steps over the head dim
     constexpr int DB = D / 32;                          // 32-channel output blocks
@@ -590,7 +590,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         part[DB * 16 * 512 + 512 + lane_off] = VARIANT == 0 ? l_run : lacc[0];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == 0) __hip_atomic_store(split_flags + bid, 1 + my_xcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // (split_wait < 0: a test of the bounded wait below, in which nobody raises a flag)
+        if (tid == 0 && split_wait > 0) __hip_atomic_store(split_flags + bid, 1 + my_xcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         continue;
     }
     float poison = 0.0f;
@@ -608,7 +609,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             // are poisoned with NaN rather than left to hang or to read stale data.
             int spins = 0, flag;
             while ((flag = __hip_atomic_load(split_flags + pb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) == 0) {
-                if (++spins > (1 << 22)) break;
+                if (++spins > (split_wait < 0 ? -split_wait : split_wait)) break;
                 __builtin_amdgcn_s_sleep(16);
             }
             asm volatile("" ::: "memory");
@@ -679,6 +680,12 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
 #endif
 }
 
+// Polls of a hand-over flag before a workgroup gives up and poisons its rows (about a microsecond
+// each: a third of a second, where the longest legitimate wait is a few milliseconds).  Negative:
+// test mode — producers raise no flags, consumers give up after that many polls.
+static std::atomic<int> g_split_wait{1 << 18};
+void attn_split_wait(int polls) { g_split_wait.store(polls == 0 ? (1 << 18) : polls); }
+
 __global__ void split_clear_kernel(int* flags, int n) {
     for (int i = threadIdx.x; i < n; i += blockDim.x) flags[i] = 0;
 }
@@ -703,7 +710,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK, SPLIT>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
                        a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,          \
                        a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,               \
-                       (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags)
+                       (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags, g_split_wait.load())
 #define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                   \
     do {                                                   \
         if (split > 0) SAGE_LAUNCH_ATTN2(STATS, ADDMASK, true); \

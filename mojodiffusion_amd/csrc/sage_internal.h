@@ -123,6 +123,7 @@ size_t attn_split_bytes(int workgroups, int D);
 constexpr size_t kSplitFlagBytes = 4096;     // one int per workgroup in front of the state slots
 constexpr int kSplitMaxWorkgroups = 1024;
 void attn_split_override(int mode);          // 0: by shape (default); -1: never; n > 0 (multiple of 8): always n
+void attn_split_wait(int polls);             // bound of the hand-over wait; 0: default; < 0: test mode (no flag is raised)
 
 // ---- backward (sage_bwd.hip) -------------------------------------------------
 // bf16 flash backward: Q, K, V, O, dO and the forward's log-sum-exp in, dQ, dK, dV out.

@@ -170,3 +170,32 @@ def test_split_mode_argument():
     for bad in (-2, 12, 1032):
         assert L.mi355_sage_set_attn_split(bad) == -1
     assert L.mi355_sage_set_attn_split(0) == 0
+
+
+def test_a_partial_result_that_never_arrives_poisons_rows_and_nothing_hangs(split):
+    """The give-up path of the hand-over wait, forced from the host: in test mode no workgroup
+    announces its partial result, every workgroup that needs one stops polling after 64 polls and
+    writes NaN into its rows.  The launch ends, rows of items that were not cut stay right, and
+    the next ordinary call is unaffected."""
+    import torch
+    import gpu_harness as H
+    from test_gpu_attn import _one_shot
+    L = _lib.lib()
+    w = WORKLOADS[2].scaled(B=2, H=3, S=1100)               # 30 items of 18 steps; 24 workgroups: spans of 24 steps
+    q, k, v = make_inputs(w)
+    split(24)
+    good = bf16_bits_to_f32(_one_shot(q, k, v, w.scale, 0))
+    assert L.mi355_sage_set_attn_split_wait(-64) == 0
+    try:
+        bad = bf16_bits_to_f32(_one_shot(q, k, v, w.scale, 0))
+    finally:
+        assert L.mi355_sage_set_attn_split_wait(0) == 0
+    nan_rows = np.isnan(bad).any(axis=-1)                   # [B,S,H]
+    assert nan_rows.any() and not nan_rows.all()
+    # poisoned rows come as whole row tiles of a head; everything else is bit-identical
+    np.testing.assert_array_equal(bad[~nan_rows], good[~nan_rows])
+    assert np.isnan(bad[nan_rows]).all()
+    again = bf16_bits_to_f32(_one_shot(q, k, v, w.scale, 0))
+    np.testing.assert_array_equal(again, good)
+    for bad_arg in (-(1 << 25), 1 << 25):
+        assert L.mi355_sage_set_attn_split_wait(bad_arg) == -1
