@@ -14,8 +14,10 @@
  *   - q/k/v/o are bf16; the innermost (D) stride must be 1 and every row start
  *     must be 16-byte aligned (callers hand out 16-byte-aligned scratch views,
  *     serenitymojo/scratch_ring.mojo:49);
- *   - D is 64 or 128; attention is full and non-causal; trailing keys (real_N_kv) or one
- *     range of keys (_keymask) can be masked; N_q may differ from N_kv;
+ *   - D is 64, 128 or — forward only and without the fused RMSNorm / RoPE, as the reference's
+ *     Ideogram-4 arm uses it (serenitymojo/models/dit/ideogram4_dit.mojo:29-49) — 256;
+ *     attention is full and non-causal; trailing keys (real_N_kv) or one range of keys
+ *     (_keymask) can be masked; N_q may differ from N_kv;
  *   - return 0 on success; -1 for a null pointer, a non-positive dimension or
  *     null strides (serenitymojo/ops/cshim/cudnn_sdpa.cpp:391-393); -2 for an
  *     unsupported configuration; -3 for a workspace that is too small; a

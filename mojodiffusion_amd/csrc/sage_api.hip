@@ -37,7 +37,9 @@ inline size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
         }                                                                           \
     } while (0)
 
-bool dims_ok(int D) { return D == 64 || D == 128; }
+// Forward: 64, 128 and (four-wave workgroups, no fused pre-ops) 256 channels per head; backward: 64, 128.
+bool dims_ok(int D) { return D == 64 || D == 128 || D == 256; }
+bool bwd_dims_ok(int D) { return D == 64 || D == 128; }
 
 // Row starts must be 16-byte aligned and the head dim contiguous.
 int check_view(const char* name, const void* p, const int64_t* s, int64_t off) {
@@ -96,7 +98,7 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.rowinv_q = take((size_t)B * Nq * sizeof(float));        // whole-row RMSNorm statistic per token (optional pre-op)
     c.rowinv_k = take((size_t)B * Nkv * sizeof(float));
     // hand-over slots of the attention kernel's split scheduling (shapes that use it only)
-    c.split = take(attn_split_bytes(attn_split_workgroups(B, H, Nq, Nkv), D));
+    c.split = take(attn_split_bytes(attn_split_workgroups(B, H, Nq, Nkv, D), D));
     c.total = off;
     return c;
 }
@@ -287,7 +289,8 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
     if (!qs || !ks || !vs || !os) return MI355_SAGE_EINVAL;
     if (causal) { SAGE_LOG("causal attention is not supported"); return MI355_SAGE_EUNSUPPORTED; }
-    if (!dims_ok(D)) { SAGE_LOG("head dim %d not supported (64 or 128)", D); return MI355_SAGE_EUNSUPPORTED; }
+    if (!dims_ok(D)) { SAGE_LOG("head dim %d not supported (64, 128 or 256)", D); return MI355_SAGE_EUNSUPPORTED; }
+    if (D == 256 && pre.q.gain != nullptr) { SAGE_LOG("the fused RMSNorm / RoPE are built for head dims 64 and 128"); return MI355_SAGE_EUNSUPPORTED; }
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
     if (!blk_ok(blkq) || !blk_ok(blkk)) { SAGE_LOG("block sizes must be 32, 64 or 128"); return MI355_SAGE_EUNSUPPORTED; }
     if (k_flags & ~3) return MI355_SAGE_EUNSUPPORTED;
@@ -506,6 +509,7 @@ static int quant_qk_entry(const void* Q, const void* K, int B, int H, int N_q, i
     if (!q_strides || !k_strides) return MI355_SAGE_EINVAL;
     if ((k_flags & 3) && !scratch) return MI355_SAGE_EINVAL;
     if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk) || (k_flags & ~3)) return MI355_SAGE_EUNSUPPORTED;
+    if (D == 256 && pre.q.gain != nullptr) return MI355_SAGE_EUNSUPPORTED;
     const ScratchCarve sc = scratch_carve(B, H, N_kv, D);
     if ((k_flags & 3) && scratch_bytes < sc.total) return MI355_SAGE_EWORKSPACE;
     if (pre.q.gain != nullptr && (pre.q.cos != nullptr || pre.full_row) && N_q != N_kv) return MI355_SAGE_EUNSUPPORTED;
@@ -664,7 +668,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     a.stats = static_cast<float*>(stats);
     // Same scheduling, hence the same bits, as the one-shot calls: shapes that are split over a
     // fixed number of workgroups need hand-over slots, kept per (device, stream) by the library.
-    const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid), D);
+    const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid, D), D);
     if (split_bytes > 0 && (rc = internal_workspace(g_split_ws, split_bytes, static_cast<hipStream_t>(stream), &a.split))) return rc;
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
@@ -701,7 +705,7 @@ static BwdCarve bwd_carve(int B, int H, int Nq, int Nkv, int D) {
 }
 
 size_t mi355_sage_bwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D) {
-    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || !dims_ok(D)) return 0;
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || !bwd_dims_ok(D)) return 0;
     return bwd_carve(B, H, N_q, N_kv, D).total;
 }
 
@@ -722,7 +726,7 @@ int mi355_sage_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const 
     if (!q_strides || !k_strides || !v_strides || !o_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
         return MI355_SAGE_EINVAL;
     if (causal) { SAGE_LOG("causal attention is not supported"); return MI355_SAGE_EUNSUPPORTED; }
-    if (!dims_ok(D)) { SAGE_LOG("head dim %d is not supported (64 or 128)", D); return MI355_SAGE_EUNSUPPORTED; }
+    if (!bwd_dims_ok(D)) { SAGE_LOG("backward: head dim %d is not supported (64 or 128)", D); return MI355_SAGE_EUNSUPPORTED; }
     int rc;
     if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off)) ||
         (rc = check_view("V", V, v_strides, v_off)) || (rc = check_view("O", O, o_strides, o_off)) ||

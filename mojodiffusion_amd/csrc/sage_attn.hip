@@ -89,6 +89,15 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 constexpr int kMagicI = 0x3E22F983;
 constexpr float kMagicF = 0.15915494309189532f;        // the same 32 bits
 constexpr float kMagicUnit = 67108864.0f;               // 2^26: accumulator-as-float steps per integer
+// With 256 channels |dot| can reach 256*127*127 = 4129024, more than the mantissa of 1/(2*pi) has
+// room for below it.  0.1875 = 2^-3 * (1 + 2^22 * 2^-23) leaves 2^22 = 4194304 either way at the
+// same step of 2^-26; it is no inline operand, so that instantiation keeps it in registers.
+constexpr int kMagicWideI = 0x3E400000;
+constexpr float kMagicWideF = 0.1875f;
+template <int D> struct Magic {
+    static constexpr int I = D > 128 ? kMagicWideI : kMagicI;
+    static constexpr float F = D > 128 ? kMagicWideF : kMagicF;
+};
 
 // First matrix instruction of a score chain: accumulator input = the inline constant above.
 // (The compiler keeps a splat constant in 16 registers and copies them into the accumulator
@@ -96,10 +105,17 @@ constexpr float kMagicUnit = 67108864.0f;               // 2^26: accumulator-as-
 // following instructions of the chain are compiler-visible builtins that accumulate in place,
 // so everything that reads the finished scores is ordered against a matrix instruction the
 // compiler knows about.
+template <int D>
 __device__ __forceinline__ v16i mfma_i8_from_magic(const v4i& a, const v4i& b) {
-    v16i d;
-    asm("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0.15915494" : "=&v"(d) : "v"(a), "v"(b));
-    return d;
+    if constexpr (D > 128) {
+        constexpr int M = kMagicWideI;
+        const v16i c = {M, M, M, M, M, M, M, M, M, M, M, M, M, M, M, M};
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    } else {
+        v16i d;
+        asm("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0.15915494" : "=&v"(d) : "v"(a), "v"(b));
+        return d;
+    }
 }
 
 // A row's reference maximum is only refreshed (and the accumulators rescaled) when a tile
@@ -123,7 +139,7 @@ template <int VARIANT> struct Lazy {
 // global loads share the vector-memory counter with the tile copies, i.e. it waits for all of
 // them at the midpoint: it is bound by the N_q x N_kv bias it has to read, not by the copies.
 template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT>
-__global__ __launch_bounds__(512, 2) void sage_attn_kernel(
+__global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
@@ -138,11 +154,15 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     constexpr int DB = D / 32;                          // 32-channel output blocks
     constexpr int K_BYTES = kTileKV * D;                // K tile
     constexpr int V_BYTES = D * kTileKV * VB;           // V^T tile
-    constexpr int NW = 8;                               // waves per workgroup
+    // 256 channels: the output accumulators alone take 128 registers per lane, so a wave gets a SIMD
+    // to itself (up to 512 registers) and a workgroup is 4 waves = 128 query rows.
+    constexpr int NW = D > 128 ? 4 : 8;                 // waves per workgroup
+    constexpr int THREADS = NW * 64;
+    constexpr int ROWS_WG = NW * 32;                    // query rows per workgroup
     constexpr int K_NCH = K_BYTES / 1024, V_NCH = V_BYTES / 1024;      // 1 KiB copies per tile
     constexpr int K_CH = (K_NCH + NW - 1) / NW;         // copies per wave (short tiles: some waves repeat a copy)
     constexpr int V_CH = (V_NCH + NW - 1) / NW;
-    constexpr int LEAD = 2;                             // tile copies run this many iterations ahead
+    constexpr int LEAD = D > 128 ? 1 : 2;               // tile copies run this many iterations ahead (LDS: 160 KiB)
     constexpr int NSK = LEAD + 1, NSV = LEAD + 2;       // ring depths
     constexpr int K_CPR = D / 16;                       // chunks per K row
     constexpr int V_CPR = kTileKV * VB / 16;            // chunks per V^T row
@@ -153,7 +173,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     constexpr int FPU = VARIANT == 0 ? 1 : 2;           // 16-byte V fragments per PV instruction
     constexpr int PD = VARIANT == 0 ? 2 : 1;            // V fragment prefetch distance (units)
     constexpr int PW = VARIANT == 0 ? 16 : 8;           // dwords of packed P per tile
-    static_assert(32 % NUNIT == 0 && EPU % 2 == 0, "unit split");
+    static_assert(32 % NUNIT == 0 && (EPU % 2 == 0 || EPU == 1), "unit split");
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NSK][K_BYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][V_BYTES];
@@ -193,9 +213,8 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const unsigned long long probe_r0 = __builtin_amdgcn_s_memrealtime();
     const unsigned long long probe_t0 = __builtin_readcyclecounter();
 #endif
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31, half = lane >> 5;
 
     // ---- one segment = key tiles [t_off, t_off + ntiles) of one item, last segment of the span first
     // (the instantiation without splitting is straight-line code: one segment, the whole item)
@@ -215,12 +234,15 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const int qt = (int)((uint32_t)wg % (uint32_t)qtiles_div);
     const int64_t bh = (uint32_t)wg / (uint32_t)qtiles_div;
     const int b = (int)((uint32_t)bh / (uint32_t)heads_div), h = (int)((uint32_t)bh % (uint32_t)heads_div);
-    // (through an empty statement: the per-lane addresses derived from the row are formed in the
-    // segment that uses them instead of being carried in registers across the main loop)
-    int row_in_tile = wave * 32 + l32;
-    if constexpr (SPLIT) asm volatile("" : "+v"(row_in_tile));
-    const int qrow = qt * kTileQ + row_in_tile;         // this lane's query (padded index)
-    __syncthreads();                                    // every wave has left the previous segment's LDS
+    // (through an empty statement: what is derived from the lane number — row addresses, fragment
+    // and copy offsets — is formed in the segment that uses it instead of being carried in registers
+    // from before the loop over the segments and across the hand-over code at its end)
+    int lane = tid & 63;
+    if constexpr (SPLIT) asm volatile("" : "+v"(lane));
+    const int l32 = lane & 31, half = lane >> 5;
+    const int row_in_tile = wave * 32 + l32;
+    const int qrow = qt * ROWS_WG + row_in_tile;        // this lane's query (padded index)
+    if constexpr (SPLIT) __syncthreads();               // every wave has left the previous segment's LDS
 
     // Q^T fragments: 16 bytes of the head dim per step, resident for the whole kernel.
     v4i qf[KSTEPS];
@@ -239,7 +261,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     const float* ksc = kscale + bh * (nkv_pad / blkk);
     const int nks = (int)(nkv_pad / blkk);
     const int ush = blkk == 32 ? 0 : (blkk == 64 ? 1 : 2);      // log2(32-key blocks per scale block)
-    for (int i = row_in_tile + half * 256; i < nks; i += 64 * NW) lds_ks[i] = ksc[i];     // (indices 0..511, once each)
+    for (int i = row_in_tile + half * ROWS_WG; i < nks; i += THREADS) lds_ks[i] = ksc[i];     // (each thread a distinct index below THREADS)
     auto kscale_of = [&](int u32blk) -> float { return lds_ks[u32blk >> ush]; };
 
     // tile indices below are relative to the segment's first tile
@@ -373,7 +395,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int st = 0; st < KSTEPS; st++)
-                s[kb] = st == 0 ? mfma_i8_from_magic(kf[kb][0], qf[0])
+                s[kb] = st == 0 ? mfma_i8_from_magic<D>(kf[kb][0], qf[0])
                                 : __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], s[kb], 0, 0, 0);
 
         float f[2], c0[2];
@@ -398,7 +420,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         if constexpr (ADDMASK) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
-                const float base = -(kMagicF * f[kb]);
+                const float base = -(Magic<D>::F * f[kb]);
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const int key = key0 + kb * 32 + g * 8 + half * 4;
@@ -442,7 +464,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
                     mb = max(max(mb, s[kb][i + 2]), s[kb][i + 3]);
                 }
                 const int mi = max(max(ma, mb), max(s[kb][14], s[kb][15]));
-                const float mk = mi < 0 ? -INFINITY : (float)(mi - kMagicI) * (f[kb] * (1.0f / kMagicUnit));
+                const float mk = mi < 0 ? -INFINITY : (float)(mi - Magic<D>::I) * (f[kb] * (1.0f / kMagicUnit));
                 mt = fmaxf(mt, mk);
             }
             const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);
@@ -456,7 +478,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         };
         if (!OPT) decide(Lazy<VARIANT>::tau);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(kMagicF, f[kb], m_used);
+        for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
         const float l_before = l_run;
 
         // Exponentials of scores n, n+1 of this lane (n counts through kb, then i).
@@ -484,8 +506,13 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             }
         };
         auto exp_group = [&](int g) {                  // the EPU scores that go with PV unit g
+            if constexpr (EPU == 1) {                  // one score per unit: a pair with every second unit
+                if (g & 1) return;
+                exp_pair(g);
+            } else {
 #pragma unroll
-            for (int e = 0; e < EPU; e += 2) exp_pair(g * EPU + e);
+                for (int e = 0; e < EPU; e += 2) exp_pair(g * EPU + e);
+            }
             // Pin the group here: an empty volatile statement that consumes the results keeps the
             // compiler from sinking the exponentials below the matrix instructions they are meant
             // to overlap with.
@@ -521,7 +548,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
                 l_run = l_before;
                 decide(0.0f);
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(kMagicF, f[kb], m_used);
+                for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
 #pragma unroll
                 for (int n = 0; n < 32; n += 2) exp_pair(n);
             }
@@ -573,7 +600,7 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
     // write-back or invalidation — device-scope fences would throw the K/V tiles out of the L2 for
     // everybody.  That both sides sit on the same XCD follows from the round-robin placement of
     // workgroup ids; the flag carries the producer's XCD number so that the consumer can check.
-    constexpr int PART_FLOATS = (DB * 16 + 2) * 512;    // one workgroup's slot of split_part
+    constexpr int PART_FLOATS = (DB * 16 + 2) * THREADS;    // one workgroup's slot of split_part
     const int my_xcd = SPLIT ? (int)__builtin_amdgcn_s_getreg(20 | (3 << 11)) : 0;     // XCC_ID, bits 3:0
     if (SPLIT && !seg_finishes) {
         // ---- this item ends in another workgroup's span: hand over the running state ----------
@@ -583,11 +610,13 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
         uint32_t lane_off = (uint32_t)tid;
         asm volatile("" : "+v"(lane_off));
 #pragma unroll
-        for (int d = 0; d < DB; d++)
+        for (int d = 0; d < DB; d++) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) part[(d * 16 + i) * 512 + lane_off] = oacc[d][i];
-        part[DB * 16 * 512 + lane_off] = m_used;
-        part[DB * 16 * 512 + 512 + lane_off] = VARIANT == 0 ? l_run : lacc[0];
+            for (int i = 0; i < 16; i++) part[(d * 16 + i) * THREADS + lane_off] = oacc[d][i];
+            __builtin_amdgcn_sched_barrier(0);          // one block at a time (keeps the live registers down)
+        }
+        part[DB * 16 * THREADS + lane_off] = m_used;
+        part[DB * 16 * THREADS + THREADS + lane_off] = VARIANT == 0 ? l_run : lacc[0];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         // (split_wait < 0: a test of the bounded wait below, in which nobody raises a flag)
@@ -616,15 +645,17 @@ __global__ __launch_bounds__(512, 2) void sage_attn_kernel(
             if (flag != 1 + my_xcd) poison = __builtin_nanf("");
             const float* part = split_part + (int64_t)pb * PART_FLOATS;
             auto peer = [&](int idx) { return __hip_atomic_load(part + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-            const float m_p = peer(DB * 16 * 512 + lane_off), l_p = peer(DB * 16 * 512 + 512 + lane_off);
+            const float m_p = peer(DB * 16 * THREADS + lane_off), l_p = peer(DB * 16 * THREADS + THREADS + lane_off);
             const float m_new = fmaxf(m_used, m_p);
             const float ca = __builtin_amdgcn_exp2f(m_used - m_new), cb = __builtin_amdgcn_exp2f(m_p - m_new);
             if constexpr (VARIANT == 0) l_run = l_run * ca + l_p * cb;
             else lacc[0] = lacc[0] * ca + l_p * cb;
 #pragma unroll
-            for (int d = 0; d < DB; d++)
+            for (int d = 0; d < DB; d++) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) oacc[d][i] = oacc[d][i] * ca + peer((d * 16 + i) * 512 + lane_off) * cb;
+                for (int i = 0; i < 16; i++) oacc[d][i] = oacc[d][i] * ca + peer((d * 16 + i) * THREADS + lane_off) * cb;
+                __builtin_amdgcn_sched_barrier(0);
+            }
             m_used = m_new;
             need = ps0;
         }
@@ -692,10 +723,11 @@ __global__ void split_clear_kernel(int* flags, int n) {
 
 template <int D, int VARIANT>
 static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
-    const int n_qtiles = (int)(a.nq_pad / kTileQ);
+    constexpr int kThreads = D > 128 ? 256 : 512;             // 32 query rows per wave
+    const int n_qtiles = (int)(a.nq_pad / (kThreads / 2));
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    const int split = attn_split_workgroups(a.B, a.H, a.Nq, a.kv_valid);
+    const int split = D > 128 ? 0 : attn_split_workgroups(a.B, a.H, a.Nq, a.kv_valid, D);
     int* flags = nullptr;
     float* part = nullptr;
     if (split > 0) {
@@ -705,16 +737,20 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
         // (a kernel, not a memset: the call may be recorded into a graph)
         hipLaunchKernelGGL(split_clear_kernel, dim3(1), dim3(256), 0, st, flags, split);
     }
-    dim3 grid((unsigned)(split > 0 ? split : total)), block(512);
+    dim3 grid((unsigned)(split > 0 ? split : total)), block(kThreads);
 #define SAGE_LAUNCH_ATTN2(STATS, ADDMASK, SPLIT)                                                                         \
     hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK, SPLIT>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
                        a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,          \
                        a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,               \
                        (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags, g_split_wait.load())
-#define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                   \
-    do {                                                   \
-        if (split > 0) SAGE_LAUNCH_ATTN2(STATS, ADDMASK, true); \
-        else SAGE_LAUNCH_ATTN2(STATS, ADDMASK, false);     \
+#define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                                  \
+    do {                                                                  \
+        if constexpr (D <= 128) {                                         \
+            if (split > 0) SAGE_LAUNCH_ATTN2(STATS, ADDMASK, true);       \
+            else SAGE_LAUNCH_ATTN2(STATS, ADDMASK, false);                \
+        } else {                                                          \
+            SAGE_LAUNCH_ATTN2(STATS, ADDMASK, false);                     \
+        }                                                                 \
     } while (0)
     if (a.amask != nullptr) {
         if (a.stats != nullptr) SAGE_LAUNCH_ATTN(true, true);
@@ -743,10 +779,11 @@ static std::atomic<int> g_split_mode{0};       // 0: by shape; -1: never; n > 0:
 
 void attn_split_override(int mode) { g_split_mode.store(mode); }
 
-int attn_split_workgroups(int B, int H, int Nq, int kv_valid) {
+int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D) {
 #ifdef SAGE_CLOCK_PROBE
     return 0;                                  // the measurement build reports per-item clocks
 #else
+    if (D > 128) return 0;                     // four-wave workgroups: one per item
     const int64_t items = pad_to(Nq, kTileQ) / kTileQ * B * H;
     const int64_t ntiles = (kv_valid + kTileKV - 1) / kTileKV;
     const int mode = g_split_mode.load();
@@ -766,13 +803,14 @@ int attn_split_workgroups(int B, int H, int Nq, int kv_valid) {
 
 size_t attn_split_bytes(int workgroups, int D) {
     if (workgroups <= 0) return 0;
-    return kSplitFlagBytes + (size_t)workgroups * ((D / 32) * 16 + 2) * 512 * sizeof(float);
+    return kSplitFlagBytes + (size_t)workgroups * ((D / 32) * 16 + 2) * (D > 128 ? 256 : 512) * sizeof(float);
 }
 
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st) {
     if (a.nkv_pad / a.blkk > kMaxKScales) return hipErrorInvalidValue;      // K scales would not fit the LDS staging
     if (a.D == 128) return a.variant == 0 ? launch_attn_dv<128, 0>(a, st) : launch_attn_dv<128, 1>(a, st);
     if (a.D == 64) return a.variant == 0 ? launch_attn_dv<64, 0>(a, st) : launch_attn_dv<64, 1>(a, st);
+    if (a.D == 256) return a.variant == 0 ? launch_attn_dv<256, 0>(a, st) : launch_attn_dv<256, 1>(a, st);
     return hipErrorInvalidValue;
 }
 

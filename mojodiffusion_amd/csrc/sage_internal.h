@@ -118,7 +118,7 @@ hipError_t launch_attn(const AttnArgs& a, hipStream_t st);
 // Shapes whose items do not fill whole rounds of workgroups are spread evenly over a fixed number
 // of workgroups that hand partial results to each other through `split`.  Number of workgroups
 // (a multiple of 8), or 0 for one workgroup per item; depends on the shape only.
-int attn_split_workgroups(int B, int H, int Nq, int kv_valid);
+int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D);
 size_t attn_split_bytes(int workgroups, int D);
 constexpr size_t kSplitFlagBytes = 4096;     // one int per workgroup in front of the state slots
 constexpr int kSplitMaxWorkgroups = 1024;

@@ -285,14 +285,17 @@ struct KGroupSmem {
     float leafmax[16][D + 1];
 };
 
-template <int D, bool PRE>
+// D is the number of channels this call covers, starting at channel col0 of a head of DFULL
+// channels (the statistics are per channel, so a 256-channel head is done as two windows of 128).
+template <int D, bool PRE, int DFULL = D>
 __device__ __forceinline__ void kstats_group_body(
     int g, int h, int b, int tid, const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int ngroups, const KeyMask& km, double* __restrict__ part_sum, float* __restrict__ part_mm,
-    KGroupSmem<D>& sm, const PreOp& pre) {
+    KGroupSmem<D>& sm, const PreOp& pre, int col0 = 0) {
+    static_assert(!PRE || DFULL == D, "the fused pre-ops need the whole row in one call");
     constexpr int CPR = D / 8;
     const int leaf = tid / CPR, col = (tid % CPR) * 8;
-    const uint16_t* src = k + b * sb + h * sh + col;
+    const uint16_t* src = k + b * sb + h * sh + col0 + col;
     const int s0 = g * kGroup + leaf * kLeaf;
 
     u32x4 w[kLeaf];
@@ -335,7 +338,7 @@ __device__ __forceinline__ void kstats_group_body(
             gmn = fminf(gmn, sm.leafmin[u][tid]);
             gmx = fmaxf(gmx, sm.leafmax[u][tid]);
         }
-        const int64_t o = (((int64_t)b * H + h) * ngroups + g) * D + tid;
+        const int64_t o = (((int64_t)b * H + h) * ngroups + g) * DFULL + col0 + tid;
         part_sum[o] = gsum;
         part_mm[2 * o] = gmn;
         part_mm[2 * o + 1] = gmx;
@@ -357,7 +360,8 @@ __device__ __forceinline__ uint16_t f32_to_f16_sat(float x) {
 // touch every bank once (D = 128: 16 chunks; D = 64: 8 chunks, XOR with slot/8 instead).
 template <int D>
 __device__ __forceinline__ int v_tile_chunk(int slot, int chunk) {
-    return D == 128 ? (chunk ^ (((slot >> 3) & 7) << 1)) : (chunk ^ ((slot >> 3) & 7));
+    // (D = 256: 32 chunks, XOR with 4*(slot/8))
+    return D == 256 ? (chunk ^ (((slot >> 3) & 7) << 2)) : D == 128 ? (chunk ^ (((slot >> 3) & 7) << 1)) : (chunk ^ ((slot >> 3) & 7));
 }
 
 template <int D>
@@ -513,11 +517,12 @@ __device__ __forceinline__ void quant_v_fp8_body(
 // ---------------------------------------------------------------------------
 template <int D, bool PRE>
 __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
-    constexpr int GPW = 256 / (16 * (D / 8));             // K groups per workgroup
+    constexpr int DK = D > 128 ? 128 : D;                 // channels per K statistics call
+    constexpr int GPW = 256 / (16 * (DK / 8));            // K groups per workgroup (D = 256: one group, one half of the channels)
     union Smem {
         uint16_t tile[64 * D];
         float red[256 / (D / 8)][D + 1];
-        KGroupSmem<D> kg[GPW];
+        KGroupSmem<DK> kg[GPW];
     };
     __shared__ __attribute__((aligned(16))) Smem sm;
     const int per_bh = a.nv_units + a.nk_wg;
@@ -528,6 +533,10 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
             quant_v_f16_body<D>(r, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km, a.v16, sm.tile);
         else
             v_absmax_group_body<D>(r, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.ngroups, a.km, a.vpart, sm.red);
+    } else if constexpr (D > 128) {
+        const int u = r - a.nv_units;                     // (group, channel half)
+        kstats_group_body<DK, false, D>(u >> 1, h, b, threadIdx.x, a.k.p, a.k.sb, a.k.sh, a.k.sn, a.Nkv, a.H, a.ngroups,
+                                        a.km, a.kpart_sum, a.kpart_mm, sm.kg[0], a.pre_k, (u & 1) * DK);
     } else {
         const int sub = threadIdx.x / (16 * (D / 8));
         const int g = (r - a.nv_units) * GPW + sub;
@@ -585,8 +594,8 @@ hipError_t launch_row_inv(const View& q, const View& k, int B, int H, int Nq, in
 hipError_t launch_prep(const PrepArgs& a_in, int B, int D, hipStream_t st) {
     PrepArgs a = a_in;
     a.ngroups = (a.Nkv + kGroup - 1) / kGroup;
-    const int gpw = D == 128 ? 1 : 2;
-    a.nk_wg = a.kpart_sum != nullptr ? (a.ngroups + gpw - 1) / gpw : 0;
+    // K groups per workgroup: 2 at D = 64, 1 at D = 128; at D = 256 a group takes two workgroups
+    a.nk_wg = a.kpart_sum == nullptr ? 0 : D == 256 ? a.ngroups * 2 : D == 128 ? a.ngroups : (a.ngroups + 1) / 2;
     a.nv_units = a.vmode == 0 ? (int)(a.nkv_pad / 64) : (a.vmode == 1 ? a.ngroups : 0);
     const int64_t total = (int64_t)B * a.H * (a.nv_units + a.nk_wg);
     if (total == 0) return hipSuccess;
@@ -597,6 +606,7 @@ hipError_t launch_prep(const PrepArgs& a_in, int B, int D, hipStream_t st) {
     else if (D == 128) hipLaunchKernelGGL((prep_kernel<128, false>), grid, block, 0, st, a);
     else if (D == 64 && has_pre) hipLaunchKernelGGL((prep_kernel<64, true>), grid, block, 0, st, a);
     else if (D == 64) hipLaunchKernelGGL((prep_kernel<64, false>), grid, block, 0, st, a);
+    else if (D == 256 && !has_pre) hipLaunchKernelGGL((prep_kernel<256, false>), grid, block, 0, st, a);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -715,6 +725,7 @@ hipError_t launch_quant(const QuantArgs& a_in, int B, int D, hipStream_t st) {
     else if (D == 128) hipLaunchKernelGGL((quant_kernel<128, false>), grid, block, 0, st, a);
     else if (D == 64 && has_pre) hipLaunchKernelGGL((quant_kernel<64, true>), grid, block, 0, st, a);
     else if (D == 64) hipLaunchKernelGGL((quant_kernel<64, false>), grid, block, 0, st, a);
+    else if (D == 256 && !has_pre) hipLaunchKernelGGL((quant_kernel<256, false>), grid, block, 0, st, a);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

@@ -10,7 +10,7 @@
 Same dtype flow as the reference arms: BF16 q/k/v go straight in; anything else is cast to BF16
 at the op boundary and the result cast back to q's dtype; the returned tensor owns its memory.
 There is no other backend behind these functions: with an arm switched off, or for a head dim the
-library does not cover, they raise.
+library does not cover (64, 128 and, forward only, 256 are covered), they raise.
 """
 import torch
 
@@ -21,8 +21,8 @@ ZIMAGE_SDPA_SAGE = True
 LTX2_SDPA_SAGE = True
 KREA2_SDPA_SAGE = True
 KLEIN_SDPA_SAGE = True
-# Ideogram-4 attends with Dh = 256 (ideogram4_dit.mojo:39-40); the kernels cover 64 and 128.
-IDEOGRAM4_SDPA_SAGE = False
+# Ideogram-4 attends with Dh = 256 (ideogram4_dit.mojo:39-40): forward only, as in the reference.
+IDEOGRAM4_SDPA_SAGE = True
 
 
 def _product_fwd(name, enabled, q, k, v, scale, variant, rect):

@@ -39,9 +39,11 @@ def test_product_fwd_arms_bf16_and_f32(oracle):
     qs = qd[:, :200].contiguous()
     got = M.ltx2_sdpa_product_fwd_rect(qs.float(), kd.float(), vd.float(), w.scale)
     np.testing.assert_array_equal(got.cpu().numpy(), A.sdpa_flash_train_fwd_rect(qs, kd, vd, w.scale).o.float().cpu().numpy())
-    # Ideogram-4 attends with Dh = 256: no arm, and no silent fallback
+    # the Ideogram-4 arm (Dh = 256 in that model) is the same function
+    np.testing.assert_array_equal(Hh.to_bits(M.ideogram4_sdpa_product_fwd(qd, kd, vd, w.scale)), Hh.to_bits(want))
+    # a head dim the library does not cover: no silent fallback
     with pytest.raises(A.Error):
-        M.ideogram4_sdpa_product_fwd(qd, kd, vd, w.scale)
+        M.zimage_sdpa_product_fwd(qd[..., :96].contiguous(), kd[..., :96].contiguous(), vd[..., :96].contiguous(), w.scale)
     # a switched-off arm fails loudly too
     M.ZIMAGE_SDPA_SAGE = False
     try:

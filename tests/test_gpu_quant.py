@@ -56,7 +56,8 @@ def test_quant_bit_exact_at_full_sequence_length(oracle, wid):
 
 
 @pytest.mark.parametrize("D,S,mask,smooth,balance", [(128, 700, (300, 512), True, True), (128, 333, (0, 64), True, True),
-                                                     (64, 520, (500, 520), True, False), (128, 200, (17, 150), False, True)])
+                                                     (64, 520, (500, 520), True, False), (128, 200, (17, 150), False, True),
+                                                     (256, 600, (100, 333), True, True)])
 def test_quant_with_masked_key_range(oracle, D, S, mask, smooth, balance):
     """Keys [lo, hi) take no part: not in the K statistics, not in their scale blocks (code 0),
     not in the V scales (bytes 0) — also when the range cuts through blocks and groups."""
@@ -80,7 +81,8 @@ def test_quant_with_masked_key_range(oracle, D, S, mask, smooth, balance):
 
 @pytest.mark.parametrize("D,blkq,blkk,S,smooth", [
     (64, 32, 32, 96, True), (64, 128, 128, 300, False), (128, 32, 64, 1, True),
-    (128, 64, 32, 65, True), (128, 128, 64, 257, False), (64, 64, 64, 1024, True)])
+    (128, 64, 32, 65, True), (128, 128, 64, 257, False), (64, 64, 64, 1024, True),
+    (256, 128, 64, 1153, True), (256, 32, 32, 300, True), (256, 64, 128, 77, False)])
 def test_quant_qk_bit_exact_shapes(oracle, D, blkq, blkk, S, smooth):
     import gpu_harness as H
     rng = np.random.default_rng(S * 7 + D)
@@ -143,7 +145,7 @@ def test_quant_qk_bhsd_strides_and_offsets(oracle):
             np.testing.assert_array_equal(a["vscale"], b["vscale"])
 
 
-@pytest.mark.parametrize("D,S", [(128, 1100), (64, 1024), (128, 64), (64, 7)])
+@pytest.mark.parametrize("D,S", [(128, 1100), (64, 1024), (128, 64), (64, 7), (256, 1153), (256, 50)])
 def test_quant_v_bit_exact(oracle, D, S):
     import gpu_harness as H
     rng = np.random.default_rng(S + D)
