@@ -6,15 +6,18 @@
 //     dV = P^T dO,   dS = P * (dO V^T - Delta),   dQ = scale * dS K,   dK = scale * dS^T Q,
 // with v_mfma_f32_32x32x16_bf16, fp32 accumulation, P and dS rounded to bf16 as matrix operands.
 //
-// Three launches:
+// Two launches:
 //   1. bwd_prep_kernel     Delta and Stats * log2(e) per query row (padding rows: +inf, so their
 //                          probabilities vanish), and transposed copies K^T, Q^T, dO^T in tiles of
 //                          64 rows whose rows sit in the slot order of the matrix instruction's
 //                          operand layout (v_slot_f16); and a vector c close to the mean key.
-//   2. bwd_pass_kernel<0>  owner = 256 query rows per workgroup (8 waves), loop over key tiles  -> dQ,
-//                          as scale * (dS K - rowsum(dS) c) = scale * dS (K - c)
-//   3. bwd_pass_kernel<1>  owner = 128 keys per workgroup (4 waves), loop over query tiles     -> dK, dV
-// In both passes a wave owns 32 rows ("x"), keeps their two bf16 row blocks resident as B operands
+//   2. bwd_fused_kernel    one grid of two kinds of 8-wave workgroups, the longer kind first:
+//        dQ     owner = 256 query rows, loop over key tiles, as scale * (dS K - rowsum(dS) c)
+//               = scale * dS (K - c)                                          (bwd_pass_body<D,0,8>)
+//        dK,dV  owner = 128 keys, loop over query tiles; pairs of waves share 32 keys, one wave
+//               carrying P and dV, the other dS and dK                        (bwd_dkdv_body)
+//               (head dim 64: 256 keys, every wave both products — bwd_pass_body<D,1,8>)
+// In both kinds a wave owns 32 rows ("x"), keeps their bf16 row blocks resident as B operands
 // and walks the other side ("y") in tiles of 64 rows staged in LDS by register-bypassing copies,
 // double buffered, one barrier per tile.  A 32x32 block of scores T[y,x] lands in the accumulator
 // layout with the owner row as the lane's column, which is exactly the B-operand layout of the
@@ -22,6 +25,7 @@
 // instruction, and the only transposed operands (rows = head channel, k = y) are the ones read
 // from the transposed copies of launch 1.
 #include "sage_internal.h"
+#include <type_traits>
 
 namespace sage {
 
@@ -32,6 +36,7 @@ typedef unsigned v2u __attribute__((ext_vector_type(2)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef __fp16 v2h __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -196,10 +201,20 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Launches 2 and 3.
+// Launch 2, the form in which one wave carries every product of its 32 owner rows: the dQ
+// workgroups (PASS 0), and the dK/dV workgroups at head dim 64 (PASS 1).
 // ---------------------------------------------------------------------------------------------
+template <int D, int PASS>
+struct PassLds {
+    static constexpr int TILE_BYTES = 64 * D * 2;
+    static constexpr int NTR = PASS == 0 ? 1 : 2;
+    uint8_t nat[2][2][TILE_BYTES];
+    uint8_t tr[2][NTR][TILE_BYTES];
+    float row[2][2][64];
+};
+
 template <int D, int PASS, int NW>
-__global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdArgs a) {
+__device__ __forceinline__ void bwd_pass_body(const BwdArgs& a, PassLds<D, PASS>& L, int block) {
     constexpr int XROWS = NW * 32;                  // owner rows per workgroup
     constexpr int CPR = D / 8;                      // 16-byte chunks per natural row
     constexpr int TILE_BYTES = 64 * D * 2;          // natural and transposed tiles have the same size
@@ -208,25 +223,19 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
     constexpr int KS = D / 16;                      // matrix-instruction steps over the head dim
     constexpr int DB = D / 32;                      // 32-channel output blocks
     constexpr int NTR = PASS == 0 ? 1 : 2;          // transposed operands per tile
-    // The dK/dV pass needs more than 256 registers per lane.  Its gradient accumulators are only
-    // ever touched by matrix instructions inside the loop, so they are steered into the
-    // accumulation registers (an empty statement with an "a" constraint per tile); left to itself
-    // the compiler parks the SCORE accumulators there, which the vector ALU reads element by
-    // element, and pays a copy for every one.
-    constexpr bool ACC_IN_AGPR = PASS == 1 && NW == 4;
     static_assert(RUNS % NW == 0, "tile copies must divide over the waves");
 
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_nat[2][2][TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_tr[2][NTR][TILE_BYTES];
-    __shared__ __attribute__((aligned(256))) float lds_row[2][2][64];
+    auto& lds_nat = L.nat;
+    auto& lds_tr = L.tr;
+    auto& lds_row = L.row;
 
     const int Nx = PASS == 0 ? a.Nq : a.Nkv;
     const int valid_x = PASS == 0 ? a.valid_q : a.valid_kv;
     const int Ny = PASS == 0 ? a.Nkv : a.Nq;
     const int valid_y = PASS == 0 ? a.valid_kv : a.valid_q;
     const int x_tiles = (Nx + XROWS - 1) / XROWS;
-    const int xt = blockIdx.x % x_tiles;
-    const int bh = blockIdx.x / x_tiles;
+    const int xt = block % x_tiles;
+    const int bh = block / x_tiles;
     const int b = bh / a.H, h = bh % a.H;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -334,10 +343,6 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
         dma_wait_all();
         __syncthreads();                 // tile t is visible; every wave is done with the other stage
         if (t + 1 < ntiles) copy_tile(t + 1, stage ^ 1);
-        if constexpr (ACC_IN_AGPR) {
-#pragma unroll
-            for (int d = 0; d < DB; d++) asm volatile("" : "+a"(acc1[d]), "+a"(acc2[d]));
-        }
         const uint8_t* n1 = &lds_nat[stage][0][0];
         const uint8_t* n2 = &lds_nat[stage][1][0];
         const uint8_t* r1 = &lds_tr[stage][0][0];
@@ -363,10 +368,6 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
             if (ks + 1 < KS) scores_load(blk, ks + 1);
             tacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f1[ks & 1]), __builtin_bit_cast(v8bf, b1[ks]), tacc[blk], 0, 0, 0);
             gacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f2[ks & 1]), __builtin_bit_cast(v8bf, b2[ks]), gacc[blk], 0, 0, 0);
-            // The vector ALU reads every element of the finished scores: keep them in ordinary
-            // registers.  (Only a register-class hint: the matrix instructions stay compiler-visible
-            // builtins, so the wait states between them and their readers are still inserted.)
-            if (ACC_IN_AGPR && ks == KS - 1) asm volatile("" : "+v"(tacc[blk]), "+v"(gacc[blk]));
         };
         // elements i, i+1 of a block (i even): y rows (i>>2)*8 + half*4 + (i&3) (+1), column = owner row
         auto softmax_pair = [&](int blk, int i) {
@@ -486,16 +487,284 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 2 : 1) void bwd_pass_kernel(BwdA
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Launch 2, dK/dV workgroups at head dim 128.  The single-wave form above would keep 128
+// accumulator and 64 operand registers per lane and so run one wave per SIMD.  Here a PAIR of waves
+// shares 32 keys:
+//   the P wave keeps the keys' K rows and the dV accumulators:  T = Q K^T -> P = exp2(cT - lse) -> dV += P^T dO
+//   the S wave keeps the keys' V rows and the dK accumulators:  G = dO V^T, dS = P (G - Delta)  -> dK += dS^T Q
+// No product is computed twice and every fragment is read from LDS once.  P goes from the P wave
+// to the S wave through LDS, in the lane layout of the accumulator, which both waves share — as
+// fp16 (11 significant bits, truncated): dS is P times a difference and is itself rounded to bf16,
+// and a bf16 P underneath would add a second error of the same size to every term of dK.  The S wave runs one query tile behind the P wave, so the hand-over is ordered by the
+// workgroup barrier that every tile has anyway; the tiles the S wave reads (dO, Q^T, Delta) are
+// copied one iteration later than the P wave's (Q, dO^T, lse), which keeps every ring at two slots.
+// There is room for one hand-over slot only (160 KiB of LDS): before the P wave overwrites it, it
+// checks a per-pair counter that the S wave advances as soon as it holds the previous tile's P in
+// registers — at the top of the iteration, half a tile before the P wave gets there.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct DkDvLds {
+    static constexpr int TILE_BYTES = 64 * D * 2;
+    uint8_t nat[2][2][TILE_BYTES];                  // [stage][0: Q | 1: dO], natural rows
+    uint8_t tr[2][2][TILE_BYTES];                   // [stage][0: Q^T | 1: dO^T]
+    u32x4 p[4][2][2][64];                           // [pair][32-row block][values 0-7 | 8-15][lane], fp16 pairs
+    float row[2][2][64];                            // [stage][0: lse | 1: Delta]
+    int taken[4];                                   // per pair: the S wave holds P of every tile below this
+};
+
+template <int D, int ROLE>
+__device__ __forceinline__ void dkdv_role(const BwdArgs& a, DkDvLds<D>& L, int bh, int xt, int wave, int lane) {
+    constexpr int NW = 8;
+    constexpr int CPR = D / 8;
+    constexpr int TILE_BYTES = 64 * D * 2;
+    constexpr int RUNS = TILE_BYTES / 1024;
+    constexpr int RPW = RUNS / NW;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    static_assert(RUNS % NW == 0, "tile copies must divide over the waves");
+    const int b = bh / a.H, h = bh % a.H;
+    const int pair = wave & 3;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int x = xt * 128 + pair * 32 + l32;
+    const int xc = min(x, a.Nkv - 1);
+
+    // owner side: the P wave keeps K rows, the S wave V rows (B operands: column = key, k = head channel)
+    const View& xv = ROLE == 0 ? a.k : a.v;
+    v4i bx[KS];
+    {
+        const uint16_t* px = xv.p + b * xv.sb + h * xv.sh + (int64_t)xc * xv.sn + half * 8;
+#pragma unroll
+        for (int s = 0; s < KS; s++) bx[s] = *reinterpret_cast<const v4i*>(px + s * 16);
+    }
+#pragma unroll
+    for (int s = 0; s < KS; s++) asm volatile("" : "+v"(bx[s]));     // the wait for these loads stays out of the loop
+    dma_wait_all();
+
+    const uint8_t* yq = reinterpret_cast<const uint8_t*>(a.q.p + b * a.q.sb + h * a.q.sh);
+    const uint8_t* yg = reinterpret_cast<const uint8_t*>(a.dout.p + b * a.dout.sb + h * a.dout.sh);
+    const uint8_t* tq = reinterpret_cast<const uint8_t*>(a.qT) + (int64_t)bh * a.nq_pad * D * 2;
+    const uint8_t* tg = reinterpret_cast<const uint8_t*>(a.doT) + (int64_t)bh * a.nq_pad * D * 2;
+    const uint8_t* rows_l = reinterpret_cast<const uint8_t*>(a.lse2 + (int64_t)bh * a.nq_pad);
+    const uint8_t* rows_d = reinterpret_cast<const uint8_t*>(a.delta + (int64_t)bh * a.nq_pad);
+    const int ntiles = xt * 128 < a.valid_kv ? (a.valid_q + 63) / 64 : 0;
+
+    int nat_row[RPW], nat_col[RPW];
+    uint32_t tr_src[RPW];
+#pragma unroll
+    for (int i = 0; i < RPW; i++) {
+        const int P = (i * NW + wave) * 64 + lane;
+        const int row = P / CPR, pos = P % CPR;
+        nat_row[i] = row;
+        nat_col[i] = nat_pos<CPR>(row, pos) * 16;
+        tr_src[i] = (uint32_t)tr_off(P);
+    }
+    const uint32_t nat_base = lds_addr(&L.nat[0][0][0]), tr_base = lds_addr(&L.tr[0][0][0]);
+    const uint32_t row_base = lds_addr(&L.row[0][0][0]);
+    const uint32_t sq = (uint32_t)(a.q.sn * 2), sg = (uint32_t)(a.dout.sn * 2);
+    // what the P wave reads of query tile t: Q rows, dO^T, lse
+    auto copy_for_p = [&](int t, int stage) {
+#pragma unroll
+        for (int i = 0; i < RPW; i++) {
+            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], a.Nq - 1);
+            const uint32_t dst = (uint32_t)((i * NW + wave) * 1024);
+            dma16(yq, row * sq + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 0) * TILE_BYTES + dst));
+            dma16(tg + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * 2 + 1) * TILE_BYTES + dst));
+        }
+        if (wave == 0) dma4(rows_l + (int64_t)t * 256, lane * 4, __builtin_amdgcn_readfirstlane(row_base + (stage * 2 + 0) * 256));
+    };
+    // what the S wave reads of query tile t: dO rows, Q^T, Delta
+    auto copy_for_s = [&](int t, int stage) {
+#pragma unroll
+        for (int i = 0; i < RPW; i++) {
+            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], a.Nq - 1);
+            const uint32_t dst = (uint32_t)((i * NW + wave) * 1024);
+            dma16(yg, row * sg + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 1) * TILE_BYTES + dst));
+            dma16(tq + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * 2 + 0) * TILE_BYTES + dst));
+        }
+        if (wave == 1) dma4(rows_d + (int64_t)t * 256, lane * 4, __builtin_amdgcn_readfirstlane(row_base + (stage * 2 + 1) * 256));
+    };
+
+    int nat_frag[2][KS];
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int s = 0; s < KS; s++) nat_frag[blk][s] = nat_off<CPR>(blk * 32 + l32, s * 2 + half);
+    int tr_frag[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) tr_frag[j] = tr_off(l32 * 8 + j * 2 + half);
+
+    v16f acc[DB];
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[d][i] = 0.0f;
+    const float c = a.scale * kLog2e;
+    // (an LDS pointer by type: through a generic one the accesses become flat instructions, whose waits
+    // also wait for the tile copies in flight)
+    volatile __attribute__((address_space(3))) int* taken = (volatile __attribute__((address_space(3))) int*)&L.taken[pair];
+
+    if (ntiles > 0) copy_for_p(0, 0);
+    // iteration `it`: the P wave works on query tile it, the S wave on tile it - 1
+    for (int it = 0; ntiles > 0 && it <= ntiles; it++) {
+        const int stage = it & 1;
+        dma_wait_all();
+        __syncthreads();                 // this iteration's tiles and the previous one's P are visible; the other stage is free
+        if (it + 1 < ntiles) copy_for_p(it + 1, stage ^ 1);
+        if (it < ntiles) copy_for_s(it, stage ^ 1);
+        if (ROLE == 0 ? it >= ntiles : it == 0) continue;
+
+        const uint8_t* nt = &L.nat[stage][ROLE][0];
+        const uint8_t* rt = &L.tr[stage][1 - ROLE][0];
+        const float* rowv = &L.row[stage][ROLE][0];
+        uint32_t hp[2][8];               // S wave: the P wave's probabilities of this tile
+        if constexpr (ROLE == 1) {
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const u32x4 w = L.p[pair][blk][j][lane];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) hp[blk][j * 4 + e] = w[e];
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) asm volatile("" : "+v"(hp[blk][e]));
+            if (lane == 0) *taken = it;
+        }
+        v16f sacc[2];
+        uint32_t pk[2][8];               // P (P wave) or dS (S wave), packed bf16 pairs: the next product's B operand
+        uint32_t ph[2][8];               // P wave: the same P as fp16 pairs, for the S wave
+        float rv[4];
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) sacc[blk][i] = 0.0f;
+        v4i f[2];
+        auto scores_load = [&](int blk, int ks) { f[ks & 1] = *reinterpret_cast<const v4i*>(nt + nat_frag[blk][ks]); };
+        auto scores_step = [&](int blk, int ks) {
+            if (ks + 1 < KS) scores_load(blk, ks + 1);
+            sacc[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, f[ks & 1]), __builtin_bit_cast(v8bf, bx[ks]), sacc[blk], 0, 0, 0);
+        };
+        // elements i, i+1 of a block (i even): query rows (i>>2)*8 + half*4 + (i&3) (+1), column = key
+        auto value_pair = [&](int blk, int i) {
+            const int g = i >> 2;
+            if ((i & 3) == 0) {
+                const v4f vr = *reinterpret_cast<const v4f*>(rowv + blk * 32 + g * 8 + half * 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) rv[e] = vr[e];
+            }
+            float y[2];
+            if constexpr (ROLE == 0) {
+#pragma unroll
+                for (int e = 0; e < 2; e++) y[e] = __builtin_amdgcn_exp2f(fmaf(sacc[blk][i + e], c, -rv[(i & 3) + e]));
+                ph[blk][i >> 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(y[0], y[1]));
+            } else {
+                const v2h w = __builtin_bit_cast(v2h, hp[blk][i >> 1]);
+                y[0] = (float)w[0] * (sacc[blk][i] - rv[i & 3]);
+                y[1] = (float)w[1] * (sacc[blk][i + 1] - rv[(i & 3) + 1]);
+            }
+            pk[blk][i >> 1] = pack_bf16(y[0], y[1]);
+        };
+        constexpr int ACC_M = 2 * DB;
+        auto acc_step = [&](int blk, int m) {
+            const int j2 = m / DB, d = m % DB;
+            const int j = blk * 2 + j2;
+            const v4i sb = {(int)pk[blk][j2 * 4], (int)pk[blk][j2 * 4 + 1], (int)pk[blk][j2 * 4 + 2], (int)pk[blk][j2 * 4 + 3]};
+            const v4i fa = *reinterpret_cast<const v4i*>(rt + tr_frag[j] + d * 32 * 128);
+            acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, fa), __builtin_bit_cast(v8bf, sb), acc[d], 0, 0, 0);
+        };
+        auto hand_over = [&](int blk) {
+            if constexpr (ROLE == 0) {
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    L.p[pair][blk][j][lane] = u32x4{ph[blk][j * 4], ph[blk][j * 4 + 1], ph[blk][j * 4 + 2], ph[blk][j * 4 + 3]};
+            }
+        };
+        scores_load(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) scores_step(0, ks);
+        scores_load(1, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            scores_step(1, ks);
+#pragma unroll
+            for (int q = 0; q < 8 / KS; q++) value_pair(0, (ks * (8 / KS) + q) * 2);
+        }
+        if constexpr (ROLE == 0) {
+            // the slot still holds the previous tile's P until the S wave has it in registers
+            while (__builtin_amdgcn_readfirstlane(*taken) < it) __builtin_amdgcn_s_sleep(1);
+            asm volatile("" ::: "memory");
+        }
+        hand_over(0);
+#pragma unroll
+        for (int m = 0; m < ACC_M; m++) {
+            acc_step(0, m);
+#pragma unroll
+            for (int q = 0; q < 8 / ACC_M; q++) value_pair(1, (m * (8 / ACC_M) + q) * 2);
+        }
+        hand_over(1);
+#pragma unroll
+        for (int m = 0; m < ACC_M; m++) acc_step(1, m);
+    }
+
+    if (x < a.Nkv) {
+        const bool live = x < a.valid_kv;
+        uint16_t* o = ROLE == 0 ? a.dv + b * a.dv_sb + h * a.dv_sh + (int64_t)x * a.dv_sn
+                                : a.dk + b * a.dk_sb + h * a.dk_sh + (int64_t)x * a.dk_sn;
+        const float mul = ROLE == 0 ? 1.0f : a.scale;
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                u32x2 w = {0u, 0u};
+                if (live) {
+                    w.x = pack_bf16(acc[d][g * 4] * mul, acc[d][g * 4 + 1] * mul);
+                    w.y = pack_bf16(acc[d][g * 4 + 2] * mul, acc[d][g * 4 + 3] * mul);
+                }
+                *reinterpret_cast<u32x2*>(o + d * 32 + g * 8 + half * 4) = w;
+            }
+    }
+}
+
+template <int D>
+__device__ __forceinline__ void bwd_dkdv_body(const BwdArgs& a, DkDvLds<D>& L, int block) {
+    const int x_tiles = (a.Nkv + 127) / 128;
+    const int xt = block % x_tiles, bh = block / x_tiles;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    if (tid < 4) L.taken[tid] = 0;                  // ordered before the first use by the loop's first barrier
+    if (wave < 4) dkdv_role<D, 0>(a, L, bh, xt, wave, lane);
+    else dkdv_role<D, 1>(a, L, bh, xt, wave, lane);
+}
+
+// One grid for both: the first n_dq workgroups are the dQ pass (the longer ones first), the rest
+// the dK/dV pass.  Both take a whole CU (8 waves, most of the LDS); in one grid the second
+// kind starts on a CU as soon as the first kind runs out, instead of after its last workgroup.
+template <int D>
+__global__ __launch_bounds__(512, 2) void bwd_fused_kernel(BwdArgs a, int n_dq) {
+    constexpr bool PAIRED = D > 64;                 // below, the single-wave form already fits two waves per SIMD
+    using KvLds = std::conditional_t<PAIRED, DkDvLds<D>, PassLds<D, 1>>;
+    constexpr size_t BYTES = sizeof(KvLds) > sizeof(PassLds<D, 0>) ? sizeof(KvLds) : sizeof(PassLds<D, 0>);
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[BYTES];
+    const int block = (int)blockIdx.x;
+    if (block < n_dq) bwd_pass_body<D, 0, 8>(a, *reinterpret_cast<PassLds<D, 0>*>(smem), block);
+    else if constexpr (PAIRED) bwd_dkdv_body<D>(a, *reinterpret_cast<DkDvLds<D>*>(smem), block - n_dq);
+    else bwd_pass_body<D, 1, 8>(a, *reinterpret_cast<PassLds<D, 1>*>(smem), block - n_dq);
+}
+
 template <int D>
 static hipError_t launch_bwd_d(const BwdArgs& a, hipStream_t st) {
     const int64_t bh = (int64_t)a.B * a.H;
     const int64_t prep = bh * (a.nkv_pad / 64 + 3 * (a.nq_pad / 64));
-    constexpr int NWQ = 8, NWK = 4;                 // waves per workgroup of the dQ pass / the dK, dV pass
-    const int64_t gq = bh * ((a.Nq + NWQ * 32 - 1) / (NWQ * 32)), gk = bh * ((a.Nkv + NWK * 32 - 1) / (NWK * 32));
-    if (prep > 0x7FFFFFFF || gq > 0x7FFFFFFF || gk > 0x7FFFFFFF) return hipErrorInvalidValue;
+    // dQ: 256 query rows per workgroup; dK, dV: 128 keys (wave pairs) or 256 keys (single-wave form)
+    constexpr int KEYS_WG = D > 64 ? 128 : 256;
+    const int64_t gq = bh * ((a.Nq + 255) / 256), gk = bh * ((a.Nkv + KEYS_WG - 1) / KEYS_WG);
+    if (prep > 0x7FFFFFFF || gq + gk > 0x7FFFFFFF) return hipErrorInvalidValue;
     hipLaunchKernelGGL((bwd_prep_kernel<D>), dim3((unsigned)prep), dim3(256), 0, st, a);
-    hipLaunchKernelGGL((bwd_pass_kernel<D, 0, NWQ>), dim3((unsigned)gq), dim3(NWQ * 64), 0, st, a);
-    hipLaunchKernelGGL((bwd_pass_kernel<D, 1, NWK>), dim3((unsigned)gk), dim3(NWK * 64), 0, st, a);
+    hipLaunchKernelGGL((bwd_fused_kernel<D>), dim3((unsigned)(gq + gk)), dim3(512), 0, st, a, (int)gq);
     return hipGetLastError();
 }
 
