@@ -11,6 +11,8 @@
 //                  (global_load_lds), the workgroup barrier of every tile
 //   loop<4 waves>  the same loop as 128-row workgroups, one or two per CU; and with 64 rows per
 //                  wave (every LDS fragment feeds two matrix instructions, one wave per SIMD)
+//   loop_sp        64 rows per wave, one wave per SIMD, pipelined over three tiles: the scores of
+//                  tile t+1 are issued between the exponentials of tile t and P.V of tile t-1
 //   pingpong       waves 0-3 and 4-7 alternate between a matrix phase (24 matrix instructions back
 //                  to back) and a vector phase (the exponentials), half a tile apart, a barrier
 //                  between phases
@@ -171,6 +173,112 @@ __global__ __launch_bounds__(NW * 64, RB == 1 ? 2 : 1) void loop_kernel(int tile
     if (lane == 0) stamps[blockIdx.x * 8 + wave] = Stamp{t1 - t0, at_barrier, r0, r1};
 }
 
+// 64 rows per wave, one wave per SIMD, software-pipelined over three tiles: the scores of tile t+1
+// (16 matrix instructions) are issued inside iteration t, spread between the exponentials of tile t
+// and P.V of tile t-1, so that every one of the 48 matrix instructions of a tile has vector work
+// behind it in program order.  Every LDS fragment feeds two matrix instructions.
+template <int FEAT>
+__global__ __launch_bounds__(256, 1) void loop_sp_kernel(int tiles, const uint8_t* kg_all, const uint8_t* vg_all, float* out, Stamp* stamps) {
+    constexpr int NW = 4, LEAD = 2, NSK = LEAD + 2, NSV = LEAD + 2, KCH = 8 / NW, VCH = 16 / NW;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NSK][8192];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][16384];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const uint8_t* kg = kg_all + (size_t)(blockIdx.x % HEADS) * tiles * 8192;
+    const uint8_t* vg = vg_all + (size_t)(blockIdx.x % HEADS) * tiles * 16384;
+    for (int i = tid; i < NSK * 8192 / 4; i += NW * 64) ((unsigned*)lds_k)[i] = (i * 2654435761u >> 3) & 0x3B3F3B3Fu;
+    for (int i = tid; i < NSV * 16384 / 4; i += NW * 64) ((unsigned*)lds_v)[i] = (i * 2654435761u >> 3) & 0x3BFF3BFFu;
+    __syncthreads();
+    int koff[4], voff[4];
+    for (int s = 0; s < 4; s++) koff[s] = swz(l32 * 8 + s * 2 + half), voff[s] = swz(l32 * 8 + s * 2 + half);
+    int ksrc[KCH], vsrc[VCH];
+    uint32_t kdst[KCH], vdst[VCH];
+    for (int i = 0; i < KCH; i++) { ksrc[i] = swz((i * NW + wave) * 64 + lane); kdst[i] = lds_addr(&lds_k[0][0]) + (i * NW + wave) * 1024; }
+    for (int i = 0; i < VCH; i++) { vsrc[i] = swz((i * NW + wave) * 64 + lane); vdst[i] = lds_addr(&lds_v[0][0]) + (i * NW + wave) * 1024; }
+
+    v4i qf[4], kf0[2][4], vf[16];
+    init_operands(qf, kf0, vf);
+    v4i kf[8];
+    for (int i = 0; i < 8; i++) kf[i] = kf0[i >> 2][i & 3];
+    v4i qf2[2][4];
+    for (int r = 0; r < 2; r++)
+        for (int st = 0; st < 4; st++) qf2[r][st] = qf[st] ^ v4i{r, 0, r, 0};
+    v16f o[2][4] = {};
+    float l[2] = {}, f = 1e-9f, c = -0.25f;
+    unsigned p[2][2][16] = {};
+    v16i s[2][2][2] = {};          // [tile parity][row block][key block]
+    unsigned long long at_barrier = 0;
+    auto mid = [&](int t) {
+        if constexpr (FEAT & COPY) dma_wait<(LEAD - 1) * (KCH + VCH)>();
+        if (FEAT & BARRIER) {
+            const unsigned long long b0 = __builtin_readcyclecounter();
+            __builtin_amdgcn_s_barrier();
+            at_barrier += __builtin_readcyclecounter() - b0;
+        }
+        if constexpr (FEAT & COPY) {
+            const int tk = min(t + LEAD + 2, tiles - 1), tv = min(t + LEAD, tiles - 1);
+#pragma unroll
+            for (int i = 0; i < KCH; i++) dma16(kg + (size_t)tk * 8192, ksrc[i], __builtin_amdgcn_readfirstlane(kdst[i] + ((t + LEAD + 2) % NSK) * 8192));
+#pragma unroll
+            for (int i = 0; i < VCH; i++) dma16(vg + (size_t)tv * 16384, vsrc[i], __builtin_amdgcn_readfirstlane(vdst[i] + ((t + LEAD) % NSV) * 16384));
+        }
+    };
+    auto read_kf = [&](int slot, int fi) {
+        if constexpr (FEAT & FRAG) kf[fi] = *reinterpret_cast<const v4i*>(&lds_k[slot][koff[fi & 3] + (fi >> 2) * 32 * 128]);
+    };
+    auto body = [&](int t, auto xtag) {
+        constexpr int X = decltype(xtag)::value;
+        const int slot_kn = (t + 1) % NSK, slot_kn2 = (t + 2) % NSK, slot_v = (t + NSV - 1) % NSV;
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            if ((FEAT & FRAG) && u + 2 < 16) vf[u + 2] = *reinterpret_cast<const v4i*>(&lds_v[slot_v][voff[(u + 2) >> 2] + ((u + 2) & 3) * 32 * 128]);
+            // K fragment fi serves score instructions 2*fi and 2*fi+1; fetched four units ahead
+            if ((u & 1) == 0 && u + 4 < 16) read_kf(slot_kn, (u + 4) >> 1);
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                const v4i pw = {(int)p[r][X ^ 1][(u >> 2) * 4], (int)p[r][X ^ 1][(u >> 2) * 4 + 1], (int)p[r][X ^ 1][(u >> 2) * 4 + 2], (int)p[r][X ^ 1][(u >> 2) * 4 + 3]};
+                o[r][u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vf[u]), __builtin_bit_cast(v8h, pw), o[r][u & 3], 0, 0, 0);
+                const int kb = u >> 3, i = (u & 7) * 2;
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[X][r][kb][i]), f, c));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[X][r][kb][i + 1]), f, c));
+                const v2h pr = {(_Float16)p0, (_Float16)p1};
+                const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
+                l[r] = __builtin_amdgcn_fdot2(pr, ones, l[r], false);
+                p[r][X][u] = __builtin_bit_cast(unsigned, pr);
+                asm volatile("" : "+v"(l[r]), "+v"(p[r][X][u]));
+            }
+            {
+                // score instruction u of tile t+1: key block u>>3, head-dim step (u&7)>>1, row block u&1
+                const int kb = u >> 3, st = (u & 7) >> 1, r = u & 1;
+                const v16i zero = {};
+                s[X ^ 1][r][kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb * 4 + st], qf2[r][st], st == 0 ? zero : s[X ^ 1][r][kb], 0, 0, 0);
+            }
+            if (u == 7) mid(t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (FEAT & FRAG) {
+            vf[0] = *reinterpret_cast<const v4i*>(&lds_v[t % NSV][voff[0]]);
+            vf[1] = *reinterpret_cast<const v4i*>(&lds_v[t % NSV][voff[0] + 32 * 128]);
+        }
+        read_kf(slot_kn2, 0);
+        read_kf(slot_kn2, 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();
+    const unsigned long long t0 = __builtin_readcyclecounter();
+    for (int t = 0; t < tiles; t += 2) {
+        body(t, std::integral_constant<int, 0>{});
+        body(t + 1, std::integral_constant<int, 1>{});
+    }
+    const unsigned long long t1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = __builtin_amdgcn_s_memrealtime();
+    dma_wait<0>();
+    float chk = 0.0f;
+    for (int r = 0; r < 2; r++) chk += o[r][0][0] + o[r][1][0] + o[r][2][0] + o[r][3][0] + l[r] + (float)s[0][r][0][0] + (float)s[0][r][1][0];
+    if (chk == 1.2345f) out[threadIdx.x] = chk;
+    if (lane == 0) stamps[blockIdx.x * 8 + wave] = Stamp{t1 - t0, at_barrier, r0, r1};
+}
+
 // Ping-pong: while waves 0-3 are in their matrix phase, waves 4-7 (the other wave of each SIMD) are in
 // their vector phase, and the other way round; a workgroup barrier ends every phase.
 __global__ __launch_bounds__(512, 2) void pingpong_kernel(int tiles, const uint8_t* kg_all, const uint8_t* vg_all, float* out, Stamp* stamps) {
@@ -327,6 +435,12 @@ int main() {
     if (run_loop<4, 1, FRAG | COPY | BARRIER>("128-row workgroups, two per CU", 512)) return 1;
     if (run_loop<4, 2, FRAG | COPY | BARRIER, 2>("64 rows per wave, 4 waves (one per SIMD), every fragment used twice", 256)) return 1;
     if (run_loop<4, 2, FRAG | COPY, 2>("   the same without the barrier", 256)) return 1;
+    for (int rep = 0; rep < 4; rep++) hipLaunchKernelGGL((loop_sp_kernel<FRAG | COPY | BARRIER>), dim3(256), dim3(256), 0, 0, TILES, d_k, d_v, d_out, d_stamps);
+    if (report("   the same, scores of tile t+1 inside iteration t (three-stage pipeline)", 4, 256, 2)) return 1;
+    for (int rep = 0; rep < 4; rep++) hipLaunchKernelGGL((loop_sp_kernel<0>), dim3(256), dim3(256), 0, 0, TILES, d_k, d_v, d_out, d_stamps);
+    if (report("   three-stage pipeline, instruction mix only", 4, 256, 2)) return 1;
+    for (int rep = 0; rep < 4; rep++) hipLaunchKernelGGL((loop_sp_kernel<FRAG>), dim3(256), dim3(256), 0, 0, TILES, d_k, d_v, d_out, d_stamps);
+    if (report("   three-stage pipeline, + LDS fragment reads", 4, 256, 2)) return 1;
     for (int rep = 0; rep < 4; rep++) hipLaunchKernelGGL(pingpong_kernel, dim3(256), dim3(512), 0, 0, TILES, d_k, d_v, d_out, d_stamps);
     if (report("ping-pong: matrix phase | vector phase, barrier between", 8, 256)) return 1;
     return 0;
