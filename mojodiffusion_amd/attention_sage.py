@@ -7,7 +7,9 @@ serenitymojo/ops/attention_flash.mojo (sdpa_flash_train_fwd :149-202, _rect
 serenitymojo/ops/attention.mojo (sdpa :1596-1647, sdpa_chunked :1650-1687,
 sdpa_nomask :1690-1718, sdpa_nomask_tiled :1762-1787, sdpa_qwen_keymask :1790-1857,
 sdpa_cross_nomask :1860-1894, sdpa_cross_masked :1897-1936, sdpa_nomask_slab
-:2144-2169).  Tensors are [B, S, H, Dh]; torch is
+:2144-2169), and the math-mode backward surface of serenitymojo/ops/attention_backward.mojo
+(sdpa_backward :435, _masked :566, _rect :928, _scratch :1099, _rect_slab :1477, _slab :1641) with
+its shape dispatchers (autograd_v2/ops_record.mojo:165, :463; attention_flash.mojo:610).  Tensors are [B, S, H, Dh]; torch is
 used only to own device memory and the stream.  What differs from the cuDNN path:
 no 128-padding copies are needed (ragged S is handled in the kernels), so the
 `*_pad` members of the result alias the caller's tensors.
@@ -218,6 +220,240 @@ def sdpa_flash_backward_raw(q_pad, k_pad, v_pad, o_pad, stats, d_out, scale):
         raise Error("%s: d_out must be BF16" % name)
     _require_cuda(name, q_pad, k_pad, v_pad, o_pad, d_out, stats)
     return _call_bwd(name, q_pad, k_pad, v_pad, o_pad, d_out, stats, scale, q_pad.shape[1], k_pad.shape[1])
+
+
+def sdpa_flash_backward_dispatch(q_pad, k_pad, v_pad, o_pad, stats, d_out, scale, B, S, H, Dh):
+    """attention_flash.mojo:610-633: the autograd engine's entry, runtime dims in.  The reference
+    looks the dims up in a table of compiled instantiations and raises for the others; the kernels
+    here take their dims at run time, so every shape the saved tensors really have is served."""
+    name = "sdpa_flash_backward_dispatch"
+    if tuple(q_pad.shape) != (B, S, H, Dh):
+        raise Error("%s: no bucket (B,S,H,Dh)=(%d,%d,%d,%d)" % (name, B, S, H, Dh))
+    return sdpa_flash_backward_raw(q_pad, k_pad, v_pad, o_pad, stats, d_out, scale)
+
+
+@dataclass
+class SdpaGrads:
+    """serenitymojo/ops/attention_backward.mojo:56-66."""
+    d_q: torch.Tensor
+    d_k: torch.Tensor
+    d_v: torch.Tensor
+
+
+class ScratchRingMark:
+    """serenitymojo/scratch_ring.mojo:20-25 (front positions only: nothing here allocates from the back)."""
+
+    def __init__(self, slab_index, offset):
+        self.slab_index = slab_index
+        self.offset = offset
+
+
+class ScratchRingAllocator:
+    """Counterpart of serenitymojo/scratch_ring.mojo:27-215: frame-scoped scratch in slabs the
+    caller owns.  alloc() bumps through the slabs (a new slab when the current one is full),
+    mark() / rewind() give the memory back in stack order; the caller rewinds only when nothing
+    queued later on another stream still reads what was allocated since the mark."""
+
+    def __init__(self, slab_bytes, device="cuda", alignment=256):
+        self.slab_bytes = int(slab_bytes)
+        self.device = device
+        self.alignment = alignment
+        self.slabs = []
+        self.slab_index = 0
+        self.offset = 0
+
+    def capacity_bytes(self):
+        return self.slab_bytes * len(self.slabs)
+
+    def used_bytes(self):
+        return self.slab_index * self.slab_bytes + self.offset
+
+    def mark(self):
+        return ScratchRingMark(self.slab_index, self.offset)
+
+    def reset(self):
+        self.slab_index = 0
+        self.offset = 0
+
+    def rewind(self, mark):
+        if (mark.slab_index, mark.offset) > (self.slab_index, self.offset):
+            raise Error("ScratchRingAllocator: rewind mark is ahead of the allocator")
+        self.slab_index = mark.slab_index
+        self.offset = mark.offset
+
+    def alloc(self, nbytes):
+        nbytes = int(nbytes)
+        if nbytes > self.slab_bytes:
+            raise Error("ScratchRingAllocator: request %d exceeds the slab size %d" % (nbytes, self.slab_bytes))
+        while True:
+            if self.slab_index == len(self.slabs):
+                self.slabs.append(torch.empty(self.slab_bytes, dtype=torch.uint8, device=self.device))
+            slab = self.slabs[self.slab_index]
+            base = slab.data_ptr()
+            start = (base + self.offset + self.alignment - 1) // self.alignment * self.alignment - base
+            if start + nbytes <= self.slab_bytes:
+                self.offset = start + nbytes
+                return slab[start:start + nbytes]
+            self.slab_index += 1
+            self.offset = 0
+
+
+def _math_bwd(name, q, k, v, d_out, scale, variant, alloc, out_alloc=None):
+    """The decomposed backward's contract on the flash kernels: the forward is recomputed by the
+    quantized kernel (its O and log-sum-exp), the gradients by the bf16 backward.  `alloc(nbytes)`
+    provides every intermediate (workspaces, O, Stats, bf16 staging); the three results, in q's
+    dtype, are fresh tensors, or come from `out_alloc(nbytes)` when that is given."""
+    if q.dtype != k.dtype or q.dtype != v.dtype or q.dtype != d_out.dtype:
+        raise Error("%s: q/k/v/d_out dtype mismatch" % name)
+    _require_cuda(name, q, k, v, d_out)
+    B, Sq, H, Dh = q.shape
+    Skv = k.shape[1]
+    if Dh not in (64, 128):
+        raise Error("%s: Dh=%d is not supported by the backward kernels (64 or 128)" % (name, Dh))
+    L = _lib.lib()
+    dev = q.device
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def staged(t):
+        if t.dtype == torch.bfloat16:
+            return t
+        out = alloc(t.numel() * 2).view(torch.bfloat16).view(t.shape)
+        out.copy_(t)
+        return out
+
+    qb, kb, vb, gb = staged(q), staged(k), staged(v), staged(d_out)
+    o = alloc(q.numel() * 2).view(torch.bfloat16).view(q.shape)
+    stats = alloc(B * H * Sq * 4).view(torch.float32).view(B, H, Sq, 1)
+    nfw = max(L.mi355_sage_workspace_bytes(B, H, Sq, Skv, Dh, variant), 256)
+    nbw = max(L.mi355_sage_bwd_workspace_bytes(B, H, Sq, Skv, Dh), 256)
+    ws = alloc(max(nfw, nbw))            # the forward is finished with it before the backward starts (one stream)
+    qs = _lib.strides_bhnd(Sq, H, Dh)
+    ks = _lib.strides_bhnd(Skv, H, Dh)
+    rc = L.mi355_sage_sdpa_bf16_train_fwd(
+        qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), o.data_ptr(), stats.data_ptr(),
+        B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, 0, 0, 0, 0, 0,
+        0, Sq, Skv, stream, variant, ws.data_ptr(), ws.numel())
+    if rc != 0:
+        raise Error("%s: forward shim rc=%d (B=%d Sq=%d Skv=%d H=%d Dh=%d)" % (name, rc, B, Sq, Skv, H, Dh))
+    same = q.dtype == torch.bfloat16
+
+    def result_like(t):
+        if out_alloc is None:
+            return torch.empty_like(t)
+        return out_alloc(t.numel() * t.element_size()).view(t.dtype).view(t.shape)
+
+    dq = result_like(q) if same else alloc(q.numel() * 2).view(torch.bfloat16).view(q.shape)
+    dk = result_like(k) if same else alloc(k.numel() * 2).view(torch.bfloat16).view(k.shape)
+    dv = result_like(v) if same else alloc(v.numel() * 2).view(torch.bfloat16).view(v.shape)
+    rc = L.mi355_sage_sdpa_bwd_bf16(
+        qb.data_ptr(), kb.data_ptr(), vb.data_ptr(), o.data_ptr(), gb.data_ptr(), stats.data_ptr(),
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+        B, H, Sq, Skv, Dh, float(scale), qs, ks, ks, qs, qs, qs, ks, ks,
+        0, 0, 0, 0, 0, 0, 0, 0, 0,
+        0, Sq, Skv, stream, ws.data_ptr(), ws.numel())
+    if rc != 0:
+        raise Error("%s: backward shim rc=%d (B=%d Sq=%d Skv=%d H=%d Dh=%d)" % (name, rc, B, Sq, Skv, H, Dh))
+    if same:
+        return SdpaGrads(dq, dk, dv)
+    outs = []
+    for g, like in ((dq, q), (dk, k), (dv, v)):
+        r = result_like(like)
+        r.copy_(g)
+        outs.append(r)
+    return SdpaGrads(*outs)
+
+
+def _torch_alloc(device):
+    return lambda nbytes: torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+
+
+def _check_bwd_rect(name, q, k, v, d_out):
+    """Shape checks in the order and with the messages of attention_backward.mojo:947-958."""
+    if q.dim() != 4:
+        raise Error("%s: q shape != [B,Sq,H,Dh]" % name)
+    B, Sq, H, Dh = q.shape
+    if k.dim() != 4 or k.shape[0] != B or k.shape[2] != H or k.shape[3] != Dh:
+        raise Error("%s: k shape != [B,Skv,H,Dh]" % name)
+    if v.shape != k.shape:
+        raise Error("%s: v shape != [B,Skv,H,Dh]" % name)
+    if d_out.shape != q.shape:
+        raise Error("%s: d_out shape != [B,Sq,H,Dh]" % name)
+
+
+def sdpa_backward_rect(q, k, v, d_out, scale, variant=PV_FP16):
+    """attention_backward.mojo:928-1096: gradients of full attention wrt q [B,Sq,H,Dh] and k, v
+    [B,Skv,H,Dh] from the inputs and the upstream gradient alone (no saved forward), in q's dtype."""
+    name = "sdpa_backward_rect"
+    if q.dtype != k.dtype or q.dtype != v.dtype or q.dtype != d_out.dtype:
+        raise Error("%s: q/k/v/d_out dtype mismatch" % name)
+    _check_bwd_rect(name, q, k, v, d_out)
+    return _math_bwd(name, q, k, v, d_out, scale, variant, _torch_alloc(q.device))
+
+
+def _check_bwd_square(name, q, k, v, d_out):
+    if q.dtype != k.dtype or q.dtype != v.dtype or q.dtype != d_out.dtype:
+        raise Error("%s: q/k/v/d_out dtype mismatch" % name)
+    if q.dim() != 4:
+        raise Error("%s: q shape != compile-time [B,S,H,Dh]" % name)
+    if k.shape != q.shape or v.shape != q.shape or d_out.shape != q.shape:
+        raise Error("%s: k/v/d_out shape does not match q [B,S,H,Dh]" % name)
+
+
+def sdpa_backward(q, k, v, d_out, scale, variant=PV_FP16):
+    """attention_backward.mojo:435-563: the square case."""
+    _check_bwd_square("sdpa_backward", q, k, v, d_out)
+    return _math_bwd("sdpa_backward", q, k, v, d_out, scale, variant, _torch_alloc(q.device))
+
+
+def sdpa_backward_masked(q, k, v, mask_f32, d_out, scale):
+    """attention_backward.mojo:566-740 takes an additive mask into the recomputed softmax.  The
+    backward kernels here know valid lengths only, so this call is refused instead of answered
+    without the mask."""
+    raise Error("sdpa_backward_masked: an additive mask is not supported by the backward kernels")
+
+
+def sdpa_backward_scratch(q, k, v, d_out, scale, scratch, variant=PV_FP16):
+    """attention_backward.mojo:1099-1268: the intermediates come from the caller's scratch ring
+    and are given back before the call returns; the three gradients are fresh tensors."""
+    mark = scratch.mark()
+    try:
+        _check_bwd_square("sdpa_backward_scratch", q, k, v, d_out)
+        g = _math_bwd("sdpa_backward_scratch", q, k, v, d_out, scale, variant, scratch.alloc)
+        # (results that were staged in the ring have been converted into fresh tensors by now)
+        return g
+    finally:
+        scratch.rewind(mark)
+
+
+def sdpa_backward_rect_slab(q, k, v, d_out, scale, slab, variant=PV_FP16):
+    """attention_backward.mojo:1477-1638: `sdpa_backward_rect` with every intermediate taken
+    from the step's slab (nothing is given back before the step's reset)."""
+    name = "sdpa_backward_rect"
+    if q.dtype != k.dtype or q.dtype != v.dtype or q.dtype != d_out.dtype:
+        raise Error("%s: q/k/v/d_out dtype mismatch" % name)
+    _check_bwd_rect(name, q, k, v, d_out)
+    return _math_bwd(name, q, k, v, d_out, scale, variant, slab.alloc, slab.alloc)
+
+
+def sdpa_backward_slab(q, k, v, d_out, scale, slab, variant=PV_FP16):
+    """attention_backward.mojo:1641-1768."""
+    _check_bwd_square("sdpa_backward", q, k, v, d_out)
+    return _math_bwd("sdpa_backward", q, k, v, d_out, scale, variant, slab.alloc, slab.alloc)
+
+
+def sdpa_backward_dispatch(q, k, v, d_out, scale, B, S, H, Dh, variant=PV_FP16):
+    """autograd_v2/ops_record.mojo:165-216: runtime dims -> instantiation.  No table here: the
+    dims only have to be the tensors' own."""
+    if tuple(q.shape) != (B, S, H, Dh):
+        raise Error("sdpa_backward_dispatch: no comptime bucket for (B,S,H,Dh)=(%d,%d,%d,%d)" % (B, S, H, Dh))
+    return sdpa_backward(q, k, v, d_out, scale, variant)
+
+
+def sdpa_backward_dispatch_slab(q, k, v, d_out, scale, B, S, H, Dh, slab, variant=PV_FP16):
+    """autograd_v2/ops_record.mojo:463-510."""
+    if tuple(q.shape) != (B, S, H, Dh):
+        raise Error("sdpa_backward_dispatch: no comptime bucket for (B,S,H,Dh)=(%d,%d,%d,%d)" % (B, S, H, Dh))
+    return sdpa_backward_slab(q, k, v, d_out, scale, slab, variant)
 
 
 def sdpa_nomask(q, k, v, scale, variant=PV_FP16):

@@ -348,3 +348,82 @@ def test_bwd_many_tiles_is_reproducible_and_close_to_fp32_autograd(B, S, H, D):
         assert torch.equal(a, b) and torch.equal(a, c), name
     for name, got, want in zip(("dQ", "dK", "dV"), runs[0], (Q.grad, K.grad, V.grad)):
         _check(name, got, want.cpu().numpy())
+
+
+def test_math_mode_backward_surface(oracle):
+    """The decomposed backward's call surface (serenitymojo/ops/attention_backward.mojo: sdpa_backward,
+    _rect, _scratch, _slab, _rect_slab; the dispatchers of autograd_v2/ops_record.mojo) served by the
+    quantized forward + the bf16 backward.  Gates: the reference's golden gradients
+    (ops/parity/sdpa_bwd_ref.txt) at the cosine bar of its bf16 run tightened to 0.999; the checker's
+    double-precision backward at cosine >= 0.999 for F32 tensors, rectangular; the allocator-backed
+    variants give the bits of the plain call and leave their allocators as the reference's do."""
+    A = attention_sage
+    ref = np.load(os.path.join(GOLD, "sdpa_bwd_ref.npz"))
+    for tag, (B, S, H, D) in (("dh128", (1, 8, 32, 128)), ("dh64", (1, 8, 8, 64))):
+        i = np.arange(B * S * H * D, dtype=np.int64)
+        shp = (B, S, H, D)
+        q = _bf16_round(((((i * 7) % 13) - 6.0) * 0.05).reshape(shp)).cuda()
+        k = _bf16_round(((((i * 5) % 11) - 5.0) * 0.05).reshape(shp)).cuda()
+        v = _bf16_round(((((i * 3) % 9) - 4.0) * 0.05).reshape(shp)).cuda()
+        g = _bf16_round(((((i * 2) % 7) - 3.0) * 0.05).reshape(shp)).cuda()
+        grads = A.sdpa_backward(q, k, v, g, float(1.0 / np.sqrt(D)))
+        torch.cuda.synchronize()
+        assert grads.d_q.dtype == torch.bfloat16
+        for name, got in (("dq", grads.d_q), ("dk", grads.d_k), ("dv", grads.d_v)):
+            want = ref[tag + "_" + name].reshape(shp)
+            assert _cos(got.float().cpu().numpy(), want) >= 0.999, (tag, name, _cos(got.float().cpu().numpy(), want))
+
+    # F32 tensors, rectangular: results in F32, against the checker on the bf16-rounded values
+    B, Sq, Skv, H, D = 1, 300, 520, 6, 128
+    scale = float(1.0 / np.sqrt(D))
+    gen = torch.Generator().manual_seed(11)
+    q, g = (_bf16_round(torch.randn((B, Sq, H, D), generator=gen).numpy()).float() for _ in range(2))
+    k, v = (_bf16_round(torch.randn((B, Skv, H, D), generator=gen).numpy()).float() for _ in range(2))
+    want = oracle.sdpa_bwd_f32(q.numpy(), k.numpy(), v.numpy(), g.numpy(), scale)
+    got = A.sdpa_backward_rect(q.cuda(), k.cuda(), v.cuda(), g.cuda(), scale)
+    torch.cuda.synchronize()
+    for name, a, b in zip(("dQ", "dK", "dV"), (got.d_q, got.d_k, got.d_v), want):
+        assert a.dtype == torch.float32 and tuple(a.shape) == b.shape
+        assert _cos(a.cpu().numpy(), b) >= 0.999, (name, _cos(a.cpu().numpy(), b))
+
+    # allocator-backed variants: same bits, allocators left as the reference leaves them
+    S = 384
+    qb, kb, vb, gb = (torch.randn((B, S, H, D), generator=gen).to(torch.bfloat16).cuda() for _ in range(4))
+    plain = A.sdpa_backward(qb, kb, vb, gb, scale)
+    ring = A.ScratchRingAllocator(16 << 20)
+    held = ring.alloc(1000)                       # something the caller already holds in the ring
+    before = ring.used_bytes()
+    via_ring = A.sdpa_backward_scratch(qb, kb, vb, gb, scale, ring)
+    assert ring.used_bytes() == before and held.numel() == 1000
+    slab = A.StepSlab(32 << 20)
+    via_slab = A.sdpa_backward_slab(qb, kb, vb, gb, scale, slab)
+    lo, hi = slab.buf.data_ptr(), slab.buf.data_ptr() + slab.buf.numel()
+    assert lo <= via_slab.d_q.data_ptr() < hi and lo <= via_slab.d_v.data_ptr() < hi and slab.used_bytes() > 0
+    via_rect_slab = A.sdpa_backward_rect_slab(qb, kb, vb, gb, scale, slab)
+    via_dispatch = A.sdpa_backward_dispatch(qb, kb, vb, gb, scale, B, S, H, D)
+    slab.reset()
+    via_dispatch_slab = A.sdpa_backward_dispatch_slab(qb, kb, vb, gb, scale, B, S, H, D, slab)
+    torch.cuda.synchronize()
+    for other in (via_ring, via_slab, via_rect_slab, via_dispatch, via_dispatch_slab):
+        for a, b in zip((plain.d_q, plain.d_k, plain.d_v), (other.d_q, other.d_k, other.d_v)):
+            assert torch.equal(a, b)
+    fwd = A.sdpa_flash_train_fwd(qb, kb, vb, scale)
+    raw = A.sdpa_flash_backward_dispatch(fwd.q_pad, fwd.k_pad, fwd.v_pad, fwd.o_pad, fwd.stats, gb, scale, B, S, H, D)
+    torch.cuda.synchronize()
+    assert torch.equal(raw.d_q, plain.d_q) and torch.equal(raw.d_k, plain.d_k) and torch.equal(raw.d_v, plain.d_v)
+
+    # errors, with the reference's messages
+    with pytest.raises(A.Error, match="sdpa_backward: q/k/v/d_out dtype mismatch"):
+        A.sdpa_backward(qb, kb.float(), vb, gb, scale)
+    with pytest.raises(A.Error, match=r"sdpa_backward_rect: k shape != \[B,Skv,H,Dh\]"):
+        A.sdpa_backward_rect(qb, kb[:, :, :3], vb, gb, scale)
+    with pytest.raises(A.Error, match=r"sdpa_backward_rect: d_out shape != \[B,Sq,H,Dh\]"):
+        A.sdpa_backward_rect(qb, kb, vb, gb[:, :100], scale)
+    with pytest.raises(A.Error, match="no comptime bucket"):
+        A.sdpa_backward_dispatch(qb, kb, vb, gb, scale, B, S + 1, H, D)
+    with pytest.raises(A.Error, match="sdpa_flash_backward_dispatch: no bucket"):
+        A.sdpa_flash_backward_dispatch(fwd.q_pad, fwd.k_pad, fwd.v_pad, fwd.o_pad, fwd.stats, gb, scale, B, S, H + 1, D)
+    with pytest.raises(A.Error, match="additive mask is not supported"):
+        A.sdpa_backward_masked(qb, kb, vb, torch.zeros((H * S, S), device="cuda"), gb, scale)
+    with pytest.raises(A.Error, match="exceeds the slab size"):
+        A.sdpa_backward_scratch(qb, kb, vb, gb, scale, A.ScratchRingAllocator(1 << 12))
