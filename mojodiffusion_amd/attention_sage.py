@@ -9,7 +9,8 @@ sdpa_nomask :1690-1718, sdpa_nomask_tiled :1762-1787, sdpa_qwen_keymask :1790-18
 sdpa_cross_nomask :1860-1894, sdpa_cross_masked :1897-1936, sdpa_nomask_slab
 :2144-2169), and the math-mode backward surface of serenitymojo/ops/attention_backward.mojo
 (sdpa_backward :435, _masked :566, _rect :928, _scratch :1099, _rect_slab :1477, _slab :1641) with
-its shape dispatchers (autograd_v2/ops_record.mojo:165, :463; attention_flash.mojo:610).  Tensors are [B, S, H, Dh]; torch is
+its shape dispatchers (autograd_v2/ops_record.mojo:165, :463; attention_flash.mojo:610) and the
+recorded attention node (autograd_v2/ops_record.mojo:329-352).  Tensors are [B, S, H, Dh]; torch is
 used only to own device memory and the stream.  What differs from the cuDNN path:
 no 128-padding copies are needed (ragged S is handled in the kernels), so the
 `*_pad` members of the result alias the caller's tensors.
@@ -454,6 +455,37 @@ def sdpa_backward_dispatch_slab(q, k, v, d_out, scale, B, S, H, Dh, slab, varian
     if tuple(q.shape) != (B, S, H, Dh):
         raise Error("sdpa_backward_dispatch: no comptime bucket for (B,S,H,Dh)=(%d,%d,%d,%d)" % (B, S, H, Dh))
     return sdpa_backward_slab(q, k, v, d_out, scale, slab, variant)
+
+
+class _SdpaNode(torch.autograd.Function):
+    """The OPK_SDPA node of the reference's autograd engine in its flash recording
+    (serenitymojo/autograd_v2/ops_record.mojo:329-352 records q, k, v and — with the flash arm —
+    the forward's saved set; autograd_v2/engine.mojo:236-252 feeds that set and the upstream
+    gradient, cast to BF16, to sdpa_flash_backward_dispatch and casts the three gradients back)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale, variant):
+        if q.dtype != k.dtype or q.dtype != v.dtype:
+            raise Error("sdpa_nomask: q/k/v dtype mismatch")
+        fwd = sdpa_flash_train_fwd(q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16), scale, variant)
+        ctx.save_for_backward(fwd.q_pad, fwd.k_pad, fwd.v_pad, fwd.o_pad, fwd.stats)
+        ctx.scale = float(scale)
+        return fwd.o.to(q.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        q, k, v, o, stats = ctx.saved_tensors
+        B, S, H, Dh = q.shape
+        g_bf = g.to(torch.bfloat16).contiguous()
+        fb = sdpa_flash_backward_dispatch(q, k, v, o, stats, g_bf, ctx.scale, B, S, H, Dh)
+        return fb.d_q.to(g.dtype), fb.d_k.to(g.dtype), fb.d_v.to(g.dtype), None, None
+
+
+def record_sdpa(q, k, v, scale, variant=PV_FP16):
+    """att = sdpa_nomask(q, k, v, scale) recorded for backpropagation
+    (serenitymojo/autograd_v2/ops_record.mojo:329-352): the result carries a node whose backward
+    yields d_q, d_k, d_v.  torch's autograd graph stands in for the reference's `Graph`."""
+    return _SdpaNode.apply(q, k, v, scale, variant)
 
 
 def sdpa_nomask(q, k, v, scale, variant=PV_FP16):

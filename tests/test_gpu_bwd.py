@@ -427,3 +427,34 @@ def test_math_mode_backward_surface(oracle):
         A.sdpa_backward_masked(qb, kb, vb, torch.zeros((H * S, S), device="cuda"), gb, scale)
     with pytest.raises(A.Error, match="exceeds the slab size"):
         A.sdpa_backward_scratch(qb, kb, vb, gb, scale, A.ScratchRingAllocator(1 << 12))
+
+
+def test_recorded_sdpa_node_backpropagates():
+    """record_sdpa (serenitymojo/autograd_v2/ops_record.mojo:329-352 with the engine's flash arm,
+    autograd_v2/engine.mojo:236-252): F32 activations in, gradients in F32 out of loss.backward(),
+    against torch's own fp32 attention on the bf16-rounded tensors (cosine >= 0.999, the gate of
+    ops/tests/sdpa_flash_parity.mojo:177); BF16 leaves get BF16 gradients."""
+    A = attention_sage
+    B, S, H, D = 1, 640, 10, 128
+    scale = float(1.0 / np.sqrt(D))
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    base = [torch.randn((B, S, H, D), device="cuda", generator=gen).to(torch.bfloat16).float() for _ in range(3)]
+    w = torch.randn((B, S, H, D), device="cuda", generator=gen)
+    q, k, v = (t.clone().requires_grad_(True) for t in base)
+    att = A.record_sdpa(q, k, v, scale)
+    assert att.dtype == torch.float32 and att.requires_grad
+    (att * w).sum().backward()
+    Q, K, V = (t.clone().permute(0, 2, 1, 3).requires_grad_(True) for t in base)
+    ref = torch.softmax(scale * Q @ K.transpose(-1, -2), dim=-1) @ V
+    (ref * w.permute(0, 2, 1, 3)).sum().backward()
+    torch.cuda.synchronize()
+    assert _cos(att.detach().cpu().numpy(), ref.detach().permute(0, 2, 1, 3).cpu().numpy()) >= 0.999
+    for name, got, want in (("dQ", q.grad, Q.grad), ("dK", k.grad, K.grad), ("dV", v.grad, V.grad)):
+        assert got.dtype == torch.float32
+        c = _cos(got.cpu().numpy(), want.permute(0, 2, 1, 3).cpu().numpy())
+        assert c >= 0.999, (name, c)
+    qb, kb, vb = (t.to(torch.bfloat16).requires_grad_(True) for t in base)
+    A.record_sdpa(qb, kb, vb, scale).float().sum().backward()
+    assert qb.grad.dtype == torch.bfloat16 and vb.grad.shape == vb.shape
+    with pytest.raises(A.Error, match="sdpa_nomask: q/k/v dtype mismatch"):
+        A.record_sdpa(qb, kb.float(), vb, scale)
