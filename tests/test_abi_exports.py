@@ -143,3 +143,42 @@ def test_host_mirror_error_strings():
         A.sdpa_qwen_keymask(qb, qb, qb, 129, 5, 0.1)
     with pytest.raises(A.Error, match="sdpa_qwen_keymask: k/v shape mismatch"):
         A.sdpa_qwen_keymask(qb, qb[:, :64], qb, 64, 5, 0.1)
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """include/mi355_sage.h is the boundary a Mojo / C / C++ caller binds: it has to compile as
+    strict C11 and as C++ with nothing but the standard headers, and a C program linked against
+    the library has to resolve its symbols (no torch, no Python in between)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None or shutil.which("g++") is None:
+        import pytest
+        pytest.skip("no host compiler")
+    inc = os.path.join(ROOT, "include")
+    src = tmp_path / "use.c"
+    src.write_text(
+        '#include "mi355_sage.h"\n'
+        '#include <stdio.h>\n'
+        '#include <string.h>\n'
+        'int main(void) {\n'
+        '    /* argument errors are reported before any device is touched */\n'
+        '    int rc = mi355_sage_sdpa_bf16(NULL, NULL, NULL, NULL, 1, 1, 1, 1, 128, 1.0f, NULL, NULL, NULL, NULL,\n'
+        '                                  0, 0, 0, 0, 0, NULL, MI355_SAGE_PV_FP16, NULL, 0);\n'
+        '    if (rc != MI355_SAGE_EINVAL) return 2;\n'
+        '    if (strncmp(mi355_sage_version(), "mi355_sage", 10) != 0) return 3;\n'
+        '    if (mi355_sage_pad_kv(32760) != 32768) return 4;\n'
+        '    if (mi355_sage_workspace_bytes(1, 24, 4608, 4608, 128, MI355_SAGE_PV_FP16) == 0) return 5;\n'
+        '    printf("ok\\n");\n'
+        '    return 0;\n'
+        '}\n')
+    subprocess.check_call(["gcc", "-std=c11", "-pedantic", "-Wall", "-Wextra", "-Wstrict-prototypes", "-Werror",
+                           "-I", inc, "-fsyntax-only", str(src)])
+    cpp = tmp_path / "use.cpp"
+    cpp.write_text('#include "mi355_sage.h"\nint main() { return mi355_sage_pad_q(1) > 0 ? 0 : 1; }\n')
+    subprocess.check_call(["g++", "-std=c++17", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", inc, "-fsyntax-only", str(cpp)])
+    exe = tmp_path / "use"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.check_call(["gcc", "-std=c11", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-lmi355_sage",
+                           "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", (out.returncode, out.stdout, out.stderr)
