@@ -182,3 +182,18 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
                            "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
     out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0 and out.stdout.strip() == "ok", (out.returncode, out.stdout, out.stderr)
+
+
+def test_cpp_host_header_compiles_with_the_host_compiler(tmp_path):
+    """include/mi355_sage_host.hpp (the call surface for compiled callers) needs nothing but the
+    C ABI header, the standard library and HIP's runtime API header."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None or not os.path.exists("/opt/rocm/include/hip/hip_runtime_api.h"):
+        import pytest
+        pytest.skip("no host compiler or no HIP headers")
+    src = tmp_path / "use.cpp"
+    src.write_text('#include "mi355_sage_host.hpp"\n'
+                   'int main() { mi355_sage_host::DeviceContext ctx; (void)ctx; return mi355_sage_host::PV_FP8 == 1 ? 0 : 1; }\n')
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"),
+                           "-isystem", "/opt/rocm/include", "-fsyntax-only", str(src)])
