@@ -187,6 +187,52 @@ def clock_probe(args, L, w, qd, kd, vd, o, st, stream):
     }))
 
 
+LOOP_PARTS = {1: "no exponentials", 2: "no LDS fragment reads", 3: "no workgroup barrier in the loop",
+              4: "no tile copies in the loop", 5: "no P.V matrix instructions", 6: "one score instruction per chain instead of four"}
+
+
+def loop_parts(args, L, w, qd, kd, vd, o, st, ws, stream, ms_first):
+    """What each part of the attention loop is worth in the real kernel: the same step through the
+    shipped library and through builds that leave one part out (their results are wrong by design),
+    in turn, several rounds, medians."""
+    import torch
+    from mojodiffusion_amd import _lib
+    libs = {0: L}
+    for n in LOOP_PARTS:
+        path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libmi355_sage_part%d.so" % n)
+        if not os.path.exists(path):
+            print("bench.py: %s is missing; run `make -C mojodiffusion_amd/csrc parts` first" % path, file=sys.stderr)
+            sys.exit(4)
+        P = ctypes.CDLL(path)
+        P.mi355_sage_sdpa_bf16_ex.restype, P.mi355_sage_sdpa_bf16_ex.argtypes = _lib.SIGNATURES["mi355_sage_sdpa_bf16_ex"]
+        libs[n] = P
+    B, S, H, D = w.B, w.S, w.H, w.D
+
+    def step(P):
+        rc = P.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), B, H, S, S, D, w.scale,
+                                       st, st, st, st, 0, 0, 0, 0, 0, stream, w.variant, w.blkq, w.blkk, K_FLAGS,
+                                       ws.data_ptr(), ws.numel())
+        if rc != 0:
+            raise RuntimeError("rc=%d" % rc)
+
+    times = {n: [] for n in libs}
+    for _ in range(7):
+        for n, P in libs.items():
+            for _ in range(20):
+                step(P)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                step(P)
+            torch.cuda.synchronize()
+            times[n].append((time.perf_counter() - t0) * 1e3 / args.steps)
+    med = {n: sorted(t)[len(t) // 2] for n, t in times.items()}
+    out = {"workload": w.name, "steps_per_round": args.steps, "rounds": 7, "shipped_ms_per_step": round(med[0], 5), "parts": {}}
+    for n, what in LOOP_PARTS.items():
+        out["parts"][what] = {"ms_per_step": round(med[n], 5), "vs_shipped_pct": round(100.0 * (med[n] / med[0] - 1.0), 1)}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,6 +246,9 @@ def main():
                     help="run the attention kernel of the measurement build (libmi355_sage_probe.so), which records "
                          "its own shader cycles and elapsed constant-rate time per workgroup, and print the clock "
                          "the chip sustained under it")
+    ap.add_argument("--loop-parts", action="store_true",
+                    help="time the step with the measurement builds that leave one part of the attention loop out "
+                         "(make -C mojodiffusion_amd/csrc parts), all in this process, in turn")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain device copy of 256 MiB (read 256 MiB, write 256 MiB) five times: "
                          "the known-size kernel the HBM traffic counters are scaled by")
@@ -273,6 +322,9 @@ def main():
 
     if args.clock_probe:
         clock_probe(args, L, w, qd, kd, vd, o, st, stream)
+        return
+    if args.loop_parts:
+        loop_parts(args, L, w, qd, kd, vd, o, st, ws, stream, ms_per_step)
         return
 
     # ---- the same step replayed from a HIP graph (launch gaps shrink to the graph's own) -----

@@ -32,7 +32,19 @@
 #include <atomic>
 #include <type_traits>
 
+// Measurement builds only (`make parts`, bench.py --loop-parts): SAGE_LOOP_PART = n leaves one part
+// of the main loop out, so that its worth in the real kernel can be timed.  Results are wrong by
+// design; every kernel still runs to its end (no address depends on what is left out).  Such a
+// build instantiates the plain D = 128 kernels only.
+//   1 no exponentials   2 no LDS fragment reads   3 no workgroup barrier in the loop
+//   4 no tile copies in the loop   5 no P.V matrix instructions   6 one score instruction per chain
+#ifndef SAGE_LOOP_PART
+#define SAGE_LOOP_PART 0
+#endif
+
 namespace sage {
+
+constexpr int kLoopPart = SAGE_LOOP_PART;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -336,17 +348,23 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     uint32_t p[2][PW];
 
     auto read_kf = [&](int slot, int kb) {
+        if (kLoopPart == 2 && slot >= 0) return;
 #pragma unroll
         for (int st = 0; st < KSTEPS; st++)
             kf[kb][st] = *reinterpret_cast<const v4i*>(&lds_k[slot][koff[st] + kb * 32 * D]);
     };
     auto read_vf = [&](int slot, int u) {               // unit u = (key step j, channel block d)
         const int j = u / DB, d = u % DB;
+        if (kLoopPart == 2 && slot >= 0) return;
 #pragma unroll
         for (int x = 0; x < FPU; x++)
             vf[u][x] = *reinterpret_cast<const v4i*>(&lds_v[slot][voff[j * FPU + x] + d * 32 * VROW]);
     };
     auto pv_unit = [&](int pb, int u) {
+        if (kLoopPart == 5 && pb >= 0) {
+            asm volatile("" ::"v"(p[pb][u % PW]), "v"(vf[u][0]));      // operands stay alive
+            return;
+        }
         const int j = u / DB, d = u % DB;
         if constexpr (VARIANT == 0) {
             const v4i pw = {(int)p[pb][j * 4], (int)p[pb][j * 4 + 1], (int)p[pb][j * 4 + 2], (int)p[pb][j * 4 + 3]};
@@ -395,8 +413,10 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int st = 0; st < KSTEPS; st++)
-                s[kb] = st == 0 ? mfma_i8_from_magic<D>(kf[kb][0], qf[0])
-                                : __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], s[kb], 0, 0, 0);
+                if (kLoopPart == 6 && st > 0) asm volatile("" ::"v"(kf[kb][st]));
+                else
+                    s[kb] = st == 0 ? mfma_i8_from_magic<D>(kf[kb][0], qf[0])
+                                    : __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], s[kb], 0, 0, 0);
 
         float f[2], c0[2];
 #pragma unroll
@@ -490,8 +510,13 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
                 p0 = __builtin_amdgcn_exp2f(xs[kb][i] - mref);
                 p1 = __builtin_amdgcn_exp2f(xs[kb][i + 1] - mref);
             } else {
-                p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
-                p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
+                if (kLoopPart == 1) {
+                    p0 = fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]);
+                    p1 = fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]);
+                } else {
+                    p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
+                    p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
+                }
             }
             if constexpr (VARIANT == 0) {
                 const v2h pr = {(_Float16)p0, (_Float16)p1};
@@ -525,9 +550,11 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
         // fetch the fragments of K(t+1).
         auto midpoint = [&]() {
             dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
-            __syncthreads();
-            dma_k(min(t + LEAD + 1, last), (t + LEAD + 1) % NSK);
-            dma_v(min(t + LEAD, last), (t + LEAD) % NSV);
+            if (kLoopPart != 3) __syncthreads();
+            if (kLoopPart != 4) {
+                dma_k(min(t + LEAD + 1, last), (t + LEAD + 1) % NSK);
+                dma_v(min(t + LEAD, last), (t + LEAD) % NSV);
+            }
             read_kf(slot_knext, 0);
         };
 
@@ -808,6 +835,10 @@ size_t attn_split_bytes(int workgroups, int D) {
 
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st) {
     if (a.nkv_pad / a.blkk > kMaxKScales) return hipErrorInvalidValue;      // K scales would not fit the LDS staging
+#if SAGE_LOOP_PART != 0
+    if (a.D != 128 || a.amask != nullptr || a.stats != nullptr) return hipErrorInvalidValue;
+    return a.variant == 0 ? launch_attn_dv<128, 0>(a, st) : launch_attn_dv<128, 1>(a, st);
+#endif
     if (a.D == 128) return a.variant == 0 ? launch_attn_dv<128, 0>(a, st) : launch_attn_dv<128, 1>(a, st);
     if (a.D == 64) return a.variant == 0 ? launch_attn_dv<64, 0>(a, st) : launch_attn_dv<64, 1>(a, st);
     if (a.D == 256) return a.variant == 0 ? launch_attn_dv<256, 0>(a, st) : launch_attn_dv<256, 1>(a, st);
