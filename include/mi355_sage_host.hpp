@@ -24,6 +24,7 @@
 
 #include <cstdint>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -116,13 +117,17 @@ inline void check_shapes(const char* name, const Tensor& q, const Tensor& k, con
     if (square && q.shape()[1] != k.shape()[1]) throw Error(n + ": k/v shape does not match q [B,S,H,Dh]");
 }
 
-// One growing workspace per stream, kept for the life of the process (the library's own policy for
+// One growing workspace per (device, stream), kept for the life of the process (the library's own policy for
 // a NULL workspace, spelled out on the caller's side so that steady-state calls allocate nothing).
 inline void* workspace(size_t nbytes, hipStream_t stream, size_t* have) {
-    struct Slot { hipStream_t stream; void* p; size_t bytes; };
+    struct Slot { int dev; hipStream_t stream; void* p; size_t bytes; };
     static std::vector<Slot> slots;
+    static std::mutex guard;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) throw Error("workspace: no current device");
+    std::lock_guard<std::mutex> lock(guard);
     for (Slot& s : slots)
-        if (s.stream == stream) {
+        if (s.dev == dev && s.stream == stream) {
             if (s.bytes < nbytes) {
                 void* p = nullptr;
                 const size_t want = nbytes > 2 * s.bytes ? nbytes : 2 * s.bytes;
@@ -135,7 +140,7 @@ inline void* workspace(size_t nbytes, hipStream_t stream, size_t* have) {
         }
     void* p = nullptr;
     if (hipMalloc(&p, nbytes) != hipSuccess) throw Error("workspace allocation failed");
-    slots.push_back(Slot{stream, p, nbytes});
+    slots.push_back(Slot{dev, stream, p, nbytes});
     *have = nbytes;
     return p;
 }
