@@ -404,11 +404,17 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     // max / compare / cross-lane chain from the common path.  A reference that has become too
     // low shows up as a large tile sum (every p is non-negative, so sum <= 2^12 bounds each
     // p, far inside fp16 range); then the tile is redone the careful way.
-    auto iteration = [&](int t, auto x_tag, auto first_tag) {
+    auto iteration = [&](int t, auto x_tag, auto first_tag, auto slot_tag) {
         constexpr int X = decltype(x_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
         constexpr bool OPT = VARIANT == 0 && !FIRST && !ADDMASK;
-        const int slot_vprev = (t + NSV - 1) % NSV, slot_knext = (t + 1) % NSK;
+        // ST >= 0: t mod 4 as a compile-time number (both rings have four slots then), so that every
+        // slot below is a constant and the LDS addresses are register + immediate
+        constexpr int ST = decltype(slot_tag)::value;
+        static_assert(ST < 0 || (NSK == 4 && NSV == 4 && (ST & 1) == X), "constant slots need four-slot rings");
+        const int slot_vprev = ST >= 0 ? (ST + 3) & 3 : (t + NSV - 1) % NSV, slot_knext = ST >= 0 ? (ST + 1) & 3 : (t + 1) % NSK;
+        const int slot_kcopy = ST >= 0 ? (ST + LEAD + 1) & 3 : (t + LEAD + 1) % NSK, slot_vcopy = ST >= 0 ? (ST + LEAD) & 3 : (t + LEAD) % NSV;
+        const int slot_vcur = ST >= 0 ? ST : t % NSV;
 
         // ---- S^T = K(t) . Q^T : two 32-key blocks
         v16i s[2];
@@ -555,8 +561,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
             dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
             if (kLoopPart != 3) __syncthreads();
             if (kLoopPart != 4) {
-                dma_k(min(t + LEAD + 1, last), (t + LEAD + 1) % NSK);
-                dma_v(min(t + LEAD, last), (t + LEAD) % NSV);
+                dma_k(min(t + LEAD + 1, last), slot_kcopy);
+                dma_v(min(t + LEAD, last), slot_vcopy);
             }
             read_kf(slot_knext, 0);
         };
@@ -595,7 +601,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
         }
         // first V^T fragments of tile t for the next iteration (published by this iteration's midpoint)
 #pragma unroll
-        for (int u = 0; u < PD; u++) read_vf(t % NSV, u);
+        for (int u = 0; u < PD; u++) read_vf(slot_vcur, u);
         read_kf(slot_knext, 1);
     };
 
@@ -603,14 +609,35 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     using F = std::false_type;
     using X0 = std::integral_constant<int, 0>;
     using X1 = std::integral_constant<int, 1>;
-    iteration(0, X0{}, T{});
-    {
+    using SR = std::integral_constant<int, -1>;         // slots from t at run time
+    // (the split instantiations sit at the register limit and keep their slots in registers)
+    if constexpr (NSK == 4 && NSV == 4 && !SPLIT) {
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        using S2 = std::integral_constant<int, 2>;
+        using S3 = std::integral_constant<int, 3>;
+        iteration(0, X0{}, T{}, S0{});
+        int t = 1;
+        for (; t + 3 <= last; t += 4) {
+            iteration(t, X1{}, F{}, S1{});
+            iteration(t + 1, X0{}, F{}, S2{});
+            iteration(t + 2, X1{}, F{}, S3{});
+            iteration(t + 3, X0{}, F{}, S0{});
+        }
+        // the last one to three tiles (t is 1 mod 4 here)
+        for (; t < last; t += 2) {
+            iteration(t, X1{}, F{}, SR{});
+            iteration(t + 1, X0{}, F{}, SR{});
+        }
+        if (t == last) iteration(t, X1{}, F{}, SR{});
+    } else {
+        iteration(0, X0{}, T{}, SR{});
         int t = 1;
         for (; t < last; t += 2) {
-            iteration(t, X1{}, F{});
-            iteration(t + 1, X0{}, F{});
+            iteration(t, X1{}, F{}, SR{});
+            iteration(t + 1, X0{}, F{}, SR{});
         }
-        if (t == last) iteration(t, X1{}, F{});
+        if (t == last) iteration(t, X1{}, F{}, SR{});
     }
     // ---- drain: P.V of the last tile ------------------------------------------------------
     auto drain = [&](auto x_tag) {
