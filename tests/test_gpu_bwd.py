@@ -412,6 +412,20 @@ def test_math_mode_backward_surface(oracle):
     torch.cuda.synchronize()
     assert torch.equal(raw.d_q, plain.d_q) and torch.equal(raw.d_k, plain.d_k) and torch.equal(raw.d_v, plain.d_v)
 
+    # F32 tensors through the allocator-backed variants (bf16 staging and results inside the allocators)
+    qf, kf, vf, gf = (t.float() for t in (qb, kb, vb, gb))
+    plain32 = A.sdpa_backward(qf, kf, vf, gf, scale)
+    ring32 = A.sdpa_backward_scratch(qf, kf, vf, gf, scale, ring)
+    assert ring.used_bytes() == before
+    slab.reset()
+    slab32 = A.sdpa_backward_slab(qf, kf, vf, gf, scale, slab)
+    torch.cuda.synchronize()
+    assert plain32.d_q.dtype == torch.float32 and lo <= slab32.d_k.data_ptr() < hi
+    for other in (ring32, slab32):
+        for a, b in zip((plain32.d_q, plain32.d_k, plain32.d_v), (other.d_q, other.d_k, other.d_v)):
+            assert torch.equal(a, b)
+    assert torch.equal(plain32.d_v, plain.d_v.float())
+
     # errors, with the reference's messages
     with pytest.raises(A.Error, match="sdpa_backward: q/k/v/d_out dtype mismatch"):
         A.sdpa_backward(qb, kb.float(), vb, gb, scale)
