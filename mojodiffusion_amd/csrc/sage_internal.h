@@ -13,7 +13,7 @@ constexpr int kTileKV = 64;    // keys per main-loop iteration
 constexpr int kPadKV  = 128;   // key tokens are padded to this (every scale-block size divides it)
 constexpr int kLeaf   = 16;    // tokens per leaf of the K-mean summation tree
 constexpr int kGroup  = 256;   // tokens per group (16 leaves)
-constexpr int kMaxKScales = 1024;   // K scale blocks per head the attention kernel stages in LDS
+constexpr int kMaxKScales = 4096;   // K scale blocks per head the attention kernel stages in LDS (16 KiB)
 
 inline int64_t pad_to(int64_t n, int64_t m) { return (n + m - 1) / m * m; }
 

@@ -151,6 +151,35 @@ def test_properties_constant_v_and_smoothing_invariance(oracle):
     assert cos >= 0.999, (cos, mx)
 
 
+def test_sequence_beyond_1024_key_scale_blocks():
+    """98 304 keys = 1536 K scale blocks of 64 tokens per head (the kernel stages a head's K scales in
+    LDS; up to 4096 of them), one head, e4m3 P.V: sampled rows against an fp32 softmax(QK^T)V, and the
+    length one block past the limit is refused."""
+    import torch
+    L = _lib.lib()
+    base = WORKLOADS[5]
+    w = base.scaled(B=1, H=1, S=98304)
+    q, k, v = _device_inputs(w, 99)
+    o = _one_shot_dev(q, k, v, w)
+    assert torch.isfinite(o.float()).all()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(8)
+    rows = torch.randint(0, w.S, (256,), generator=g, device="cuda")
+    rows[0], rows[1] = 0, w.S - 1
+    s = (q[0, rows, 0].float() @ k[0, :, 0].float().T) * w.scale
+    ref = torch.softmax(s, dim=-1) @ v[0, :, 0].float()
+    got = o[0, rows, 0].float()
+    cos = torch.nn.functional.cosine_similarity(got.flatten(), ref.flatten(), dim=0).item()
+    assert cos >= COS and (got - ref).abs().max().item() <= 4e-2, (cos, (got - ref).abs().max().item())
+    # 4097 scale blocks: refused before anything is launched
+    n = 4096 * 64 + 1
+    st = _lib.strides_bhnd(n, 1, 128)
+    rc = L.mi355_sage_sdpa_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), 1, 1, 256, n, 128, w.scale,
+                                _lib.strides_bhnd(256, 1, 128), st, st, _lib.strides_bhnd(256, 1, 128), 0, 0, 0, 0, 0,
+                                0, 0, None, 0)
+    assert rc == -2
+
+
 @pytest.mark.parametrize("variant", [0, 1])
 def test_reference_maximum_keeps_rising(oracle, variant):
     """Keys grow along the sequence, so the row maximum rises from tile to tile by far more
