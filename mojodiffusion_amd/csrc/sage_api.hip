@@ -62,9 +62,10 @@ View make_view(const void* p, const int64_t* s, int64_t off) {
 bool blk_ok(int blk) { return blk == 32 || blk == 64 || blk == 128; }
 
 // The attention kernel keeps one head's K scales in LDS.
-int check_kv_len(int N_kv, int blkk) {
-    if (pad_to(N_kv, kPadKV) / blkk > kMaxKScales) {
-        SAGE_LOG("N_kv=%d with %d-token K blocks exceeds %d scale blocks per head", N_kv, blkk, kMaxKScales);
+int check_kv_len(int N_kv, int blkk, int D) {
+    (void)blkk;
+    if (pad_to(N_kv, kPadKV) > max_keys(D)) {
+        SAGE_LOG("N_kv=%d exceeds the %d keys per head the attention kernel takes", N_kv, max_keys(D));
         return MI355_SAGE_EUNSUPPORTED;
     }
     return 0;
@@ -98,7 +99,7 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.rowinv_q = take((size_t)B * Nq * sizeof(float));        // whole-row RMSNorm statistic per token (optional pre-op)
     c.rowinv_k = take((size_t)B * Nkv * sizeof(float));
     // hand-over slots of the attention kernel's split scheduling (shapes that use it only)
-    c.split = take(attn_split_bytes(attn_split_workgroups(B, H, Nq, Nkv, D), D));
+    c.split = take(attn_split_bytes(attn_split_workgroups(B, H, Nq, Nkv, D, variant), D));
     c.total = off;
     return c;
 }
@@ -295,7 +296,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if (!blk_ok(blkq) || !blk_ok(blkk)) { SAGE_LOG("block sizes must be 32, 64 or 128"); return MI355_SAGE_EUNSUPPORTED; }
     if (k_flags & ~3) return MI355_SAGE_EUNSUPPORTED;
     int rc;
-    if ((rc = check_kv_len(N_kv, blkk))) return rc;
+    if ((rc = check_kv_len(N_kv, blkk, D))) return rc;
     if ((rc = check_view("Q", Q, qs, q_off)) || (rc = check_view("K", K, ks, k_off)) ||
         (rc = check_view("V", V, vs, v_off)) || (rc = check_view("O", O, os, o_off)))
         return rc;
@@ -654,7 +655,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
     if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk)) return MI355_SAGE_EUNSUPPORTED;
     int rc;
-    if ((rc = check_kv_len(N_kv, blkk))) return rc;
+    if ((rc = check_kv_len(N_kv, blkk, D))) return rc;
     if ((rc = check_view("O", O, o_strides, o_off))) return rc;
     AttnArgs a{};
     a.q8 = static_cast<const int8_t*>(q8); a.qscale = static_cast<const float*>(qscale); a.blkq = blkq;
@@ -668,7 +669,7 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     a.stats = static_cast<float*>(stats);
     // Same scheduling, hence the same bits, as the one-shot calls: shapes that are split over a
     // fixed number of workgroups need hand-over slots, kept per (device, stream) by the library.
-    const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid, D), D);
+    const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid, D, variant), D);
     if (split_bytes > 0 && (rc = internal_workspace(g_split_ws, split_bytes, static_cast<hipStream_t>(stream), &a.split))) return rc;
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;

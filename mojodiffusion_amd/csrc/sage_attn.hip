@@ -32,19 +32,11 @@
 #include <atomic>
 #include <type_traits>
 
-// Measurement builds only (`make parts`, bench.py --loop-parts): SAGE_LOOP_PART = n leaves one part
-// of the main loop out, so that its worth in the real kernel can be timed.  Results are wrong by
-// design; every kernel still runs to its end (no address depends on what is left out).  Such a
-// build instantiates the plain D = 128 kernels only.
-//   1 no exponentials   2 no LDS fragment reads   3 no workgroup barrier in the loop
-//   4 no tile copies in the loop   5 no P.V matrix instructions   6 one score instruction per chain
-#ifndef SAGE_LOOP_PART
-#define SAGE_LOOP_PART 0
+#ifndef SAGE_DBG
+#define SAGE_DBG 0
 #endif
-
 namespace sage {
-
-constexpr int kLoopPart = SAGE_LOOP_PART;
+constexpr int kDbg = SAGE_DBG;   // TEMPORARY measurement switches: 1 no copies, 2 no barrier, 4 no fragment reads, 8 no kscale read, 16 no OPT check, 32 no mask check, 64 no vmcnt wait
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -78,7 +70,9 @@ __device__ __forceinline__ void dma16(const void* gbase_uniform, uint32_t goff, 
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(lds_base_uniform), "v"(goff), "s"(gbase_uniform)
-                 : "memory");      // (m0 is a reserved register to the compiler: it never keeps a value in it across statements)
+                 : "memory");      // (m0 cannot be named as a clobber: to this compiler it is a reserved register — it
+                                   // warns that "clobbering them may lead to undefined behaviour" — which it never
+                                   // keeps a value in across statements; its own uses set m0 right before the use)
 }
 // Wait until at most N of this wave's copies are still in flight (they complete in order).
 template <int N> __device__ __forceinline__ void dma_wait() {
@@ -151,7 +145,10 @@ template <int VARIANT> struct Lazy {
 // global loads share the vector-memory counter with the tile copies, i.e. it waits for all of
 // them at the midpoint: it is bound by the N_q x N_kv bias it has to read, not by the copies.
 template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT>
-__global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_attn_kernel(
+#ifndef SAGE_NW
+#define SAGE_NW 8
+#endif
+__global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
@@ -161,6 +158,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     float* __restrict__ stats, int n_qtiles, int total_wg,
     const uint16_t* __restrict__ amask, int64_t amb, int64_t amh, int64_t amn,
     int split_groups, float* split_part, int* split_flags, int split_wait) {
+    constexpr int KS_OFF = VARIANT == 0 ? 3 : 2;        // see lds_ks
     constexpr int VB = (VARIANT == 0) ? 2 : 1;          // bytes per V element
     constexpr int KSTEPS = D / 32;                      // int8 MFMA steps over the head dim
     constexpr int DB = D / 32;                          // 32-channel output blocks
@@ -168,17 +166,17 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     constexpr int V_BYTES = D * kTileKV * VB;           // V^T tile
     // 256 channels: the output accumulators alone take 128 registers per lane, so a wave gets a SIMD
     // to itself (up to 512 registers) and a workgroup is 4 waves = 128 query rows.
-    constexpr int NW = D > 128 ? 4 : 8;                 // waves per workgroup
+    constexpr int NW = D > 128 ? 4 : SAGE_NW;                 // waves per workgroup
     constexpr int THREADS = NW * 64;
     constexpr int ROWS_WG = NW * 32;                    // query rows per workgroup
     constexpr int K_NCH = K_BYTES / 1024, V_NCH = V_BYTES / 1024;      // 1 KiB copies per tile
     constexpr int K_CH = (K_NCH + NW - 1) / NW;         // copies per wave (short tiles: some waves repeat a copy)
     constexpr int V_CH = (V_NCH + NW - 1) / NW;
     constexpr int LEAD = D > 128 ? 1 : 2;               // tile copies run this many iterations ahead (LDS: 160 KiB)
-    // ring depths.  K needs LEAD + 1 slots; up to 128 channels it gets a fourth, so that both rings'
-    // slot numbers are a mask away (with three, the remainder by 3 and what follows from it sit in
-    // front of every LDS address and copy of the loop: measured 0.8-1.0 % of the step)
-    constexpr int NSK = D > 128 ? LEAD + 1 : LEAD + 2, NSV = LEAD + 2;
+    // ring depths: the tile in use, LEAD tiles published or in flight, and the slot the next copy
+    // goes to — for K the tile whose scores are being computed is t+1, for V^T the tile in use is t-1.
+    // (Up to 128 channels that is four slots each, so slot numbers are a mask away.)
+    constexpr int NSK = LEAD + 2, NSV = LEAD + 2;
     constexpr int K_CPR = D / 16;                       // chunks per K row
     constexpr int V_CPR = kTileKV * VB / 16;            // chunks per V^T row
     constexpr int VROW = kTileKV * VB;                  // bytes per V^T row
@@ -192,7 +190,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
 
     __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NSK][K_BYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][V_BYTES];
-    __shared__ float lds_ks[kMaxKScales];
+    __shared__ __attribute__((aligned(16))) float lds_ks[max_keys(D) / 32 + 4];
 
     // Work items are (q tile, b*h) pairs, `total_wg` of them; an item takes `ntiles` steps (key
     // tiles).  Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; each XCD gets a
@@ -274,10 +272,11 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     // would make the compiler wait for ALL outstanding vector-memory operations, i.e. for the
     // tile copies that are meant to stay in flight.
     const float* ksc = kscale + bh * (nkv_pad / blkk);
-    const int nks = (int)(nkv_pad / blkk);
     const int ush = blkk == 32 ? 0 : (blkk == 64 ? 1 : 2);      // log2(32-key blocks per scale block)
-    for (int i = row_in_tile + half * ROWS_WG; i < nks; i += THREADS) lds_ks[i] = ksc[i];     // (each thread a distinct index below THREADS)
-    auto kscale_of = [&](int u32blk) -> float { return lds_ks[u32blk >> ush]; };
+    // (staged per 32-key block, KS_OFF entries in: the main loop fetches the eight entries of one trip
+    // with two 16-byte reads, and its first entry then sits on a 16-byte boundary)
+    for (int i = tid; i < (int)(nkv_pad / 32); i += THREADS) lds_ks[KS_OFF + i] = ksc[i >> ush];
+    auto kscale_of = [&](int u32blk) -> float { return lds_ks[KS_OFF + u32blk]; };
 
     // tile indices below are relative to the segment's first tile
     const uint8_t* kg = reinterpret_cast<const uint8_t*>(k8) + bh * nkv_pad * D + (int64_t)t_off * K_BYTES;
@@ -286,16 +285,26 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
 
     // Tile-relative LDS byte offsets of this lane's MFMA A-operand fragments.  Rows
     // 32 apart keep the same swizzle, so the 32-row blocks are plain constant offsets.
-    int koff[KSTEPS], voff[JS * FPU];
+    // (held as complete LDS addresses — ring base included — behind an empty statement: a ring slot,
+    // key block or channel block is then an immediate offset of the read instruction, at most 61 440,
+    // where the compiler, left to fold the bases itself, re-forms addresses past 65 535 in the loop)
+    uint32_t koff[KSTEPS], voff[JS * FPU];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; s++) koff[s] = swz(l32 * K_CPR + s * 2 + half);
+    for (int s = 0; s < KSTEPS; s++) koff[s] = lds_addr(&lds_k[0][0]) + swz(l32 * K_CPR + s * 2 + half);
     if constexpr (VARIANT == 0) {
 #pragma unroll
-        for (int j = 0; j < JS; j++) voff[j] = swz(l32 * V_CPR + j * 2 + half);
+        for (int j = 0; j < JS; j++) voff[j] = lds_addr(&lds_v[0][0]) + swz(l32 * V_CPR + j * 2 + half);
     } else {
-        voff[0] = swz(l32 * V_CPR + half * 2);
-        voff[1] = swz(l32 * V_CPR + half * 2 + 1);
+        voff[0] = lds_addr(&lds_v[0][0]) + swz(l32 * V_CPR + half * 2);
+        voff[1] = lds_addr(&lds_v[0][0]) + swz(l32 * V_CPR + half * 2 + 1);
     }
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++) asm volatile("" : "+v"(koff[s]));
+#pragma unroll
+    for (int j = 0; j < JS * FPU; j++) asm volatile("" : "+v"(voff[j]));
+    typedef const __attribute__((address_space(3))) v4i* lds_v4i_ptr;
+    auto k_frag = [&](int slot, int st, int kb) -> v4i { return *reinterpret_cast<lds_v4i_ptr>(koff[st] + (uint32_t)(slot * K_BYTES + kb * 32 * D)); };
+    auto v_frag = [&](int slot, int jx, int d) -> v4i { return *reinterpret_cast<lds_v4i_ptr>(voff[jx] + (uint32_t)(slot * V_BYTES + d * 32 * VROW)); };
 
     // Copy i of wave w fills the 1 KiB run c = (i*8 + w) mod (copies per tile) of a tile (short
     // tiles are covered twice with identical data, which keeps every wave's copy count equal);
@@ -315,16 +324,16 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
         vsrc[i] = swz(c * 64 + lane);
         vdst[i] = lds_addr(&lds_v[0][0]) + c * 1024;
     }
-    auto dma_k = [&](int t, int slot) {
-        const uint8_t* g = kg + (int64_t)t * K_BYTES;
+    auto dma_k_at = [&](const uint8_t* g, int slot) {
 #pragma unroll
         for (int i = 0; i < K_CH; i++) dma16(g, ksrc[i], __builtin_amdgcn_readfirstlane(kdst[i] + slot * K_BYTES));
     };
-    auto dma_v = [&](int t, int slot) {
-        const uint8_t* g = vg + (int64_t)t * V_BYTES;
+    auto dma_v_at = [&](const uint8_t* g, int slot) {
 #pragma unroll
         for (int i = 0; i < V_CH; i++) dma16(g, vsrc[i], __builtin_amdgcn_readfirstlane(vdst[i] + slot * V_BYTES));
     };
+    auto dma_k = [&](int t, int slot) { dma_k_at(kg + (int64_t)t * K_BYTES, slot); };
+    auto dma_v = [&](int t, int slot) { dma_v_at(vg + (int64_t)t * V_BYTES, slot); };
 
     v16f oacc[DB];
 #pragma unroll
@@ -344,111 +353,176 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
     for (int i = 0; i < 16; i++) lacc[i] = 0.0f;
     const v8i ones8 = {0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838, 0x38383838};
 
-    // Loop-carried fragments: K of the tile whose scores come next, the first PD units of
-    // V^T of the tile whose P.V comes next, and the packed probabilities of two tiles (parity).
-    v4i kf[2][KSTEPS];
-    v4i vf[NUNIT][FPU];
-    uint32_t p[2][PW];
+    // The main loop advances in STEPS of SK keys: 32 for the fp16 variant (one P.V matrix
+    // instruction covers 16 keys), 64 for the e4m3 variant (its matrix instruction covers 64).  A
+    // 64-key tile in LDS holds SPT = 64 / SK steps.  Step h is NM matrix-instruction slots: the
+    // P.V instructions of step h-1 and the score instructions of step h+1, dealt evenly (fp16:
+    // P.V, score, P.V, ...; e4m3: score, score, P.V, ...), each followed by its share of the vector
+    // work of step h's softmax.  Every matrix instruction then has independent vector instructions
+    // behind it in program order, and the vector ALU never meets a run of matrix instructions with
+    // nothing of its own to do (measured on the instruction mix alone, two waves per SIMD:
+    // 2060 clocks per 64 keys with the score instructions in a block of their own, 1680 dealt
+    // out like this).  Three steps are in flight per wave, yet the scores (two buffers of SK keys)
+    // and the packed probabilities (two buffers) take no more registers than one 64-key tile did.
+    constexpr int SK = VARIANT == 0 ? 32 : 64;          // keys per step
+    constexpr int SKB = SK / 32;                        // 32-key blocks per step
+    constexpr int SPT = kTileKV / SK;                   // steps per tile
+    constexpr int NQ = KSTEPS * SKB;                    // score matrix instructions per step
+    constexpr int NPV = NUNIT / SPT;                    // P.V matrix instructions per step
+    constexpr int NM = NQ + NPV;                        // slots per step
+    constexpr int OPP = VARIANT == 0 ? 7 : 5;           // vector operations per pair of scores (see vop)
+    constexpr int NP = 8 * SKB;                         // pairs of scores per lane and step
+    constexpr int NV = NP * OPP;                        // vector operations of a step's softmax
+    constexpr int PWS = PW / SPT;                       // dwords of packed P per step
+#ifndef SAGE_PDS
+#define SAGE_PDS 2
+#endif
+#ifndef SAGE_GRP
+#define SAGE_GRP 3
+#endif
+    constexpr int PDS = SAGE_PDS < NM / 2 ? SAGE_PDS : NM / 2;      // operand fragments are requested this many slots ahead
+    constexpr int KOFF = SPT == 1 ? 2 : 1;              // the barrier of tile t publishes K(t + KOFF) and V(t)
+    constexpr int PERIOD = 4 * SPT;                     // steps after which ring slots and parity repeat
+    // GRP == 3: the operands of three slots are requested together, three to five slots ahead and in
+    // reverse order, so that the first of the three matrix instructions waits for the request made
+    // last — LDS answers in order — and the other two need no wait instruction at all.
+    constexpr int GRP = VARIANT == 0 ? SAGE_GRP : 1;
+    constexpr int PF = GRP > 1 ? GRP : PDS;             // slots whose operands a step finds requested on entry
+    static_assert(NM % 3 == 0 && NM / 3 == KSTEPS && PDS <= NM / 2 && (GRP == 1 || GRP == 3), "slot pattern");
+    auto slot_is_qk = [](int m) { return VARIANT == 0 ? m % 3 == 1 : m % 3 != 2; };
+    // number of the score instruction or of the P.V unit (within the step) in slot m
+    auto slot_index = [](int m) {
+        if (VARIANT == 0) return m % 3 == 1 ? m / 3 : 2 * (m / 3) + (m % 3) / 2;
+        return m % 3 == 2 ? m / 3 : 2 * (m / 3) + m % 3;
+    };
 
-    auto read_kf = [&](int slot, int kb) {
-        if (kLoopPart == 2 && slot >= 0) return;
+    // Loop-carried: the operand fragments of the first PDS slots, the scores of two steps and the
+    // packed probabilities of two steps (by parity of the step).
+    v4i fr[NM][FPU];
+    v16i s[2][SKB];
+    uint32_t p[2][PWS];
+
+    // Operands of slot m of a step whose score instructions read key block `kbq` (fp16 variant; the
+    // e4m3 variant reads both blocks) of the K tile in `kslot` and whose P.V instructions read the
+    // steps `sub` of the V^T tile in `vslot`.
+    auto fetch = [&](int m, int kslot, int kbq, int vslot, int sub) {
+        if (kDbg & 4) { asm volatile("" : "+v"(fr[m][0])); return; }
+        if (slot_is_qk(m)) {
+            const int n = slot_index(m), st = SKB == 1 ? n : n >> 1, kb = SKB == 1 ? kbq : n & 1;
+            fr[m][0] = k_frag(kslot, st, kb);
+        } else {
+            const int u = slot_index(m), j = VARIANT == 0 ? 2 * sub + u / DB : 0, d = u % DB;
 #pragma unroll
-        for (int st = 0; st < KSTEPS; st++)
-            kf[kb][st] = *reinterpret_cast<const v4i*>(&lds_k[slot][koff[st] + kb * 32 * D]);
-    };
-    auto read_vf = [&](int slot, int u) {               // unit u = (key step j, channel block d)
-        const int j = u / DB, d = u % DB;
-        if (kLoopPart == 2 && slot >= 0) return;
-#pragma unroll
-        for (int x = 0; x < FPU; x++)
-            vf[u][x] = *reinterpret_cast<const v4i*>(&lds_v[slot][voff[j * FPU + x] + d * 32 * VROW]);
-    };
-    auto pv_unit = [&](int pb, int u) {
-        if (kLoopPart == 5 && pb >= 0) {
-            asm volatile("" ::"v"(p[pb][u % PW]), "v"(vf[u][0]));      // operands stay alive
-            return;
+            for (int x = 0; x < FPU; x++)
+                fr[m][x] = v_frag(vslot, j * FPU + x, d);
         }
-        const int j = u / DB, d = u % DB;
+    };
+    auto qk_step = [&](int sb, int n, const v4i& a) {
+        const int st = SKB == 1 ? n : n >> 1, kb = SKB == 1 ? 0 : n & 1;
+        s[sb][kb] = st == 0 ? mfma_i8_from_magic<D>(a, qf[0]) : __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[st], s[sb][kb], 0, 0, 0);
+    };
+    auto pv_unit = [&](int pb, int u, const v4i (&a)[FPU]) {
+        const int jj = u / DB, d = u % DB;
         if constexpr (VARIANT == 0) {
-            const v4i pw = {(int)p[pb][j * 4], (int)p[pb][j * 4 + 1], (int)p[pb][j * 4 + 2], (int)p[pb][j * 4 + 3]};
-            oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, vf[u][0]),
+            const v4i pw = {(int)p[pb][jj * 4], (int)p[pb][jj * 4 + 1], (int)p[pb][jj * 4 + 2], (int)p[pb][jj * 4 + 3]};
+            oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a[0]),
                                                              __builtin_bit_cast(v8h, pw), oacc[d], 0, 0, 0);
         } else {
-            const v8i a = {vf[u][0].x, vf[u][0].y, vf[u][0].z, vf[u][0].w, vf[u][1].x, vf[u][1].y, vf[u][1].z, vf[u][1].w};
+            const v8i a8 = {a[0].x, a[0].y, a[0].z, a[0].w, a[1].x, a[1].y, a[1].z, a[1].w};
             const v8i pw = {(int)p[pb][0], (int)p[pb][1], (int)p[pb][2], (int)p[pb][3],
                             (int)p[pb][4], (int)p[pb][5], (int)p[pb][6], (int)p[pb][7]};
-            oacc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pw, oacc[d], 0, 0, 0, 0, 0, 0);
-            if (u == NUNIT - 1) lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones8, pw, lacc, 0, 0, 0, 0, 0, 0);
+            oacc[d] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, pw, oacc[d], 0, 0, 0, 0, 0, 0);
+            if (u == NPV - 1) lacc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones8, pw, lacc, 0, 0, 0, 0, 0, 0);
         }
     };
 
-    // ---- prologue: K(0), V(0), K(1) into the rings --------------------------------------
+    // ---- prologue: K(0) (.. K(KOFF-1)), then K(x + KOFF), V(x) for x < LEAD into the rings; scores of step 0
     // (tile indices past the end are clamped: the extra copies are in bounds and unused)
-    dma_k(0, 0);
+#pragma unroll
+    for (int x = 0; x < KOFF; x++) dma_k(min(x, last), x % NSK);
 #pragma unroll
     for (int x = 0; x < LEAD; x++) {
-        dma_k(min(x + 1, last), (x + 1) % NSK);
+        dma_k(min(x + KOFF, last), (x + KOFF) % NSK);
         dma_v(min(x, last), x % NSV);
     }
-    dma_wait<0>();
+    dma_wait<LEAD*(K_CH + V_CH)>();
     __syncthreads();
-    read_kf(0, 0);
-    read_kf(0, 1);
+    {
+        v4i k0[NQ];
+#pragma unroll
+        for (int n = 0; n < NQ; n++) {
+            const int st = SKB == 1 ? n : n >> 1, kb = SKB == 1 ? 0 : n & 1;
+            k0[n] = k_frag(0, st, kb);
+        }
+#pragma unroll
+        for (int n = 0; n < NQ; n++) qk_step(0, n, k0[n]);
+    }
+    const int last_step = ntiles * SPT - 1;
+#pragma unroll
+    for (int m = PF - 1; m >= 0; m--)
+        if (slot_is_qk(m)) fetch(m, (1 / SPT) % NSK, 1 % SPT, 0, 0);
 
-    // Iteration t (X = t & 1).  On entry: kf = K(t) fragments; (t > 0) p[X^1] = P(t-1),
-    // vf[0..PD) = V(t-1) fragments; K(t+1) and V(t) are in flight, started at the midpoint of
-    // iteration t-1.
+    // Step h (X = h & 1, tile t = h / SPT).  On entry: s[X] = scores of step h; (h > 0) p[X^1] = P(h-1);
+    // fr[0..PDS) = the first slots' operands; the tiles the step reads are published.  The step
+    // computes the scores of step h+1 into s[X^1], adds P(h-1).V(h-1) to the output and turns s[X]
+    // into p[X].  The first step of a tile holds the tile's barrier.
     //
-    // OPT (fp16 variant, interior tiles): the exponentials are taken against the reference
-    // maximum as it stands, without looking for the tile maximum first — that removes the
+    // OPT (fp16 variant, interior steps): the exponentials are taken against the reference
+    // maximum as it stands, without looking for the step's maximum first — that removes the
     // max / compare / cross-lane chain from the common path.  A reference that has become too
-    // low shows up as a large tile sum (every p is non-negative, so sum <= 2^12 bounds each
-    // p, far inside fp16 range); then the tile is redone the careful way.
-    auto iteration = [&](int t, auto x_tag, auto first_tag, auto slot_tag) {
-        constexpr int X = decltype(x_tag)::value;
+    // low shows up as a large sum (every p is non-negative, so sum <= 2^12 bounds each
+    // p, far inside fp16 range); then the step is redone the careful way.
+    //
+    // HT >= 0: h modulo 4 * SPT as a compile-time number (both rings have four slots then), so that
+    // every ring slot and key block below is a constant and the LDS addresses are register + immediate.
+    // HT < 0: h is known at run time only, but for its position in the tile, -1 - HT.
+    float kst[8];       // K scales of the eight 32-key blocks of one trip of the main loop
+    const uint8_t *kg_trip = kg, *vg_trip = vg;          // K and V^T tile of the trip's first step
+    auto step = [&](int h, auto x_tag, auto h_tag, auto first_tag, auto qk_tag) {
+        constexpr int X = decltype(x_tag)::value;            // h & 1: selects the score / probability buffers
+        constexpr int HT = decltype(h_tag)::value;
         constexpr bool FIRST = decltype(first_tag)::value;
+        constexpr bool DOQK = decltype(qk_tag)::value;       // false in the last step
         constexpr bool OPT = VARIANT == 0 && !FIRST && !ADDMASK;
-        // ST >= 0: t mod 4 as a compile-time number (both rings have four slots then), so that every
-        // slot below is a constant and the LDS addresses are register + immediate
-        constexpr int ST = decltype(slot_tag)::value;
-        static_assert(ST < 0 || (NSK == 4 && NSV == 4 && (ST & 1) == X), "constant slots need four-slot rings");
-        const int slot_vprev = ST >= 0 ? (ST + 3) & 3 : (t + NSV - 1) % NSV, slot_knext = ST >= 0 ? (ST + 1) & 3 : (t + 1) % NSK;
-        const int slot_kcopy = ST >= 0 ? (ST + LEAD + 1) & 3 : (t + LEAD + 1) % NSK, slot_vcopy = ST >= 0 ? (ST + LEAD) & 3 : (t + LEAD) % NSV;
-        const int slot_vcur = ST >= 0 ? ST : t % NSV;
+        constexpr bool TRIP = HT >= 0 && !FIRST;             // a step of the main loop: no masked keys, scales in kst
+        static_assert(HT < 0 || (NSK == 4 && NSV == 4), "constant slots need four-slot rings");
+        constexpr int SUB = HT >= 0 ? HT % SPT : -1 - HT;    // step within its tile
+        static_assert(SUB >= 0 && SUB < SPT, "position in the tile");
+        static_assert((SPT == 1 || X == SUB) && (HT < 0 || X == (HT & 1)), "parity of the step");
+        const int t = SPT == 2 ? h >> 1 : h;
+        // tiles: score operands of step h+1, and of step h+2 (requested at the end of this step);
+        // V^T of step h-1, and of step h
+        const int tq = (h + 1) / SPT, tq2 = (h + 2) / SPT, tv = (h + SPT - 1) / SPT - 1, tv2 = h / SPT;
+        const int slot_kq = HT >= 0 ? ((HT + 1) / SPT) & 3 : tq % NSK, slot_kq2 = HT >= 0 ? ((HT + 2) / SPT) & 3 : tq2 % NSK;
+        const int slot_vp = HT >= 0 ? ((HT + 4 * SPT - 1) / SPT) & 3 : (tv + NSV) % NSV, slot_vp2 = HT >= 0 ? (HT / SPT) & 3 : tv2 % NSV;
+        constexpr int kbq = (SUB + 1) % SPT, kbq2 = SUB % SPT;            // key block of the scores (fp16 variant)
+        constexpr int subv = (SUB + SPT - 1) % SPT, subv2 = SUB;          // step of the V^T tile
+        const int slot_kcopy = HT >= 0 ? (HT / SPT + KOFF + LEAD) & 3 : (t + KOFF + LEAD) % NSK;
+        const int slot_vcopy = HT >= 0 ? (HT / SPT + LEAD) & 3 : (t + LEAD) % NSV;
 
-        // ---- S^T = K(t) . Q^T : two 32-key blocks
-        v16i s[2];
+        float f[SKB], c0[SKB];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int st = 0; st < KSTEPS; st++)
-                if (kLoopPart == 6 && st > 0) asm volatile("" ::"v"(kf[kb][st]));
-                else
-                    s[kb] = st == 0 ? mfma_i8_from_magic<D>(kf[kb][0], qf[0])
-                                    : __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[kb][st], qf[st], s[kb], 0, 0, 0);
-
-        float f[2], c0[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) f[kb] = sq * kscale_of((t + t_off) * 2 + kb);
-        // Tiles that hold masked keys (the ragged end, the masked range) are rare: a real branch.
+        for (int kb = 0; kb < SKB; kb++)
+            f[kb] = sq * (TRIP ? kst[((HT + PERIOD - 1) % PERIOD) * SKB + kb] : kscale_of(t_off * 2 + h * SKB + kb));
+        // Steps that hold masked keys (the ragged end, the masked range) are rare: a real branch.
         // A masked score becomes -inf (as an integer: below every real accumulator), which the
         // exponent path below turns into p = 0 without any further test.
-        const int key0 = (t + t_off) * kTileKV;
-        if (key0 + kTileKV > kv_valid || (key0 < mask_hi && key0 + kTileKV > mask_lo)) {
+        const int key0 = t_off * kTileKV + h * SK;
+        if (!TRIP && __builtin_expect(key0 + SK > kv_valid || (key0 < mask_hi && key0 + SK > mask_lo), 0)) {
             asm volatile("" ::: "memory");
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < SKB; kb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int key = key0 + kb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                    if (key >= kv_valid || (key >= mask_lo && key < mask_hi)) s[kb][i] = (int)0xFF800000;
+                    if (key >= kv_valid || (key >= mask_lo && key < mask_hi)) s[X][kb][i] = (int)0xFF800000;
                 }
         }
         // biased scores in the log2 domain, without the reference maximum (ADDMASK only)
-        float xs[2][ADDMASK ? 16 : 1];
+        float xs[SKB][ADDMASK ? 16 : 1];
         if constexpr (ADDMASK) {
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < SKB; kb++) {
                 const float base = -(Magic<D>::F * f[kb]);
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
@@ -466,7 +540,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
                                          __uint_as_float(w1 << 16), __uint_as_float(w1 & 0xFFFF0000u)};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float sdq = fmaf(__int_as_float(s[kb][g * 4 + e]), f[kb], base);
+                        const float sdq = fmaf(__int_as_float(s[X][kb][g * 4 + e]), f[kb], base);
                         xs[kb][g * 4 + e] = fmaf(mv[e], 1.4426950408889634f, sdq);
                     }
                 }
@@ -474,25 +548,25 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
         }
         float corr = 1.0f;
         bool refresh = false;
-        // tile maximum on the raw accumulators (monotone in the score since f > 0), refresh decision
+        // the step's maximum on the raw accumulators (monotone in the score since f > 0), refresh decision
         auto decide = [&](float tau) {
             float mt = -INFINITY;
             if constexpr (ADDMASK) {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < SKB; kb++)
 #pragma unroll
                     for (int i = 0; i < 16; i++) mt = fmaxf(mt, xs[kb][i]);
             } else
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
-                int ma = max(max(s[kb][0], s[kb][1]), s[kb][2]);
-                int mb = max(max(s[kb][3], s[kb][4]), s[kb][5]);
+            for (int kb = 0; kb < SKB; kb++) {
+                int ma = max(max(s[X][kb][0], s[X][kb][1]), s[X][kb][2]);
+                int mb = max(max(s[X][kb][3], s[X][kb][4]), s[X][kb][5]);
 #pragma unroll
                 for (int i = 6; i < 14; i += 4) {
-                    ma = max(max(ma, s[kb][i]), s[kb][i + 1]);
-                    mb = max(max(mb, s[kb][i + 2]), s[kb][i + 3]);
+                    ma = max(max(ma, s[X][kb][i]), s[X][kb][i + 1]);
+                    mb = max(max(mb, s[X][kb][i + 2]), s[X][kb][i + 3]);
                 }
-                const int mi = max(max(ma, mb), max(s[kb][14], s[kb][15]));
+                const int mi = max(max(ma, mb), max(s[X][kb][14], s[X][kb][15]));
                 const float mk = mi < 0 ? -INFINITY : (float)(mi - Magic<D>::I) * (f[kb] * (1.0f / kMagicUnit));
                 mt = fmaxf(mt, mk);
             }
@@ -503,94 +577,119 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
             if (refresh) m_new = Lazy<VARIANT>::integer_ref ? ceilf(fmaxf(m_used, mt)) : fmaxf(m_used, mt);
             corr = __builtin_amdgcn_exp2f(m_used - m_new);           // 1 when nothing changed
             m_used = m_new;
-            l_run *= corr;             // already includes tile t-1's probabilities
+            l_run *= corr;             // already includes step h-1's probabilities
         };
         if (!OPT) decide(Lazy<VARIANT>::tau);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
+        for (int kb = 0; kb < SKB; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
         const float l_before = l_run;
 
-        // Exponentials of scores n, n+1 of this lane (n counts through kb, then i).
-        auto exp_pair = [&](int n) {
-            const int kb = n >> 4, i = n & 15;
-            float p0, p1;
-            if constexpr (ADDMASK) {
-                const float mref = m_used - Lazy<VARIANT>::log2_pscale;
-                p0 = __builtin_amdgcn_exp2f(xs[kb][i] - mref);
-                p1 = __builtin_amdgcn_exp2f(xs[kb][i + 1] - mref);
-            } else {
-                if (kLoopPart == 1) {
-                    p0 = fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]);
-                    p1 = fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]);
+        // The softmax of the step as NV single vector operations, so that they can be dealt out over
+        // the slots.  Pair k = scores 2k, 2k+1 of this lane (k counts through the key block, then the
+        // accumulator element); its operations: exponent argument of either score, the two exponentials,
+        // the packing and (fp16 variant) the two additions to the lane's share of the row sum.  The sum
+        // is taken over the unrounded probabilities with plain fp32 additions: v_dot2c_f32_f16 on the
+        // packed pair would do it in one instruction, but that instruction does not start while a
+        // matrix instruction is executing (measured: matrix instruction + two of them = 57 clocks,
+        // + two of any other vector instruction = 33), so each one would cost the matrix pipe a bubble.
+        float ea[NP][2];
+        // Order: the two exponent arguments of pair 0; then per pair k its two exponentials, the
+        // exponent arguments of pair k+1, its packing and its additions — an exponential's result is
+        // first read two instructions later (read right away it costs a wait state and the latency).
+        auto vop = [&](int n) {
+            int k, r;
+            if (n < 2) { k = 0; r = n; }
+            else {
+                const int mm = n - 2, kblk = mm / OPP < NP - 1 ? mm / OPP : NP - 1, q = mm - kblk * OPP;
+                if (q < 2) { k = kblk; r = 2 + q; }
+                else if (kblk < NP - 1) {
+                    if (q < 4) { k = kblk + 1; r = q - 2; }
+                    else { k = kblk; r = q; }
+                } else { k = kblk; r = q + 2; }
+            }
+            const int kb = k >> 3, i = (2 * k) & 15;
+            if (r < 2) {
+                if constexpr (ADDMASK) ea[k][r] = xs[kb][i + r] - (m_used - Lazy<VARIANT>::log2_pscale);
+                else ea[k][r] = fmaf(__int_as_float(s[X][kb][i + r]), f[kb], c0[kb]);
+            } else if (r < 4) {
+                ea[k][r - 2] = __builtin_amdgcn_exp2f(ea[k][r - 2]);
+            } else if (r == 4) {
+                if constexpr (VARIANT == 0) {
+                    const v2h pr = {(_Float16)ea[k][0], (_Float16)ea[k][1]};
+                    p[X][k] = __builtin_bit_cast(uint32_t, pr);
+                    // (pinned: left alone, the compiler moves every conversion of the step behind the
+                    // check at its end and keeps all the exponentials in registers until then)
+                    asm volatile("" : "+v"(p[X][k]));
                 } else {
-                    p0 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i]), f[kb], c0[kb]));
-                    p1 = __builtin_amdgcn_exp2f(fmaf(__int_as_float(s[kb][i + 1]), f[kb], c0[kb]));
+                    const int w = k >> 1;
+                    if (k & 1) p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(ea[k][0], ea[k][1], (int)p[X][w], true);
+                    else p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(ea[k][0], ea[k][1], 0, false);
+                    asm volatile("" : "+v"(p[X][w]));
                 }
-            }
-            if constexpr (VARIANT == 0) {
-                const v2h pr = {(_Float16)p0, (_Float16)p1};
-                const v2h ones = {(_Float16)1.0f, (_Float16)1.0f};
-                // the normaliser sums the rounded probabilities the product actually uses
-                l_run = __builtin_amdgcn_fdot2(pr, ones, l_run, false);
-                p[X][n >> 1] = __builtin_bit_cast(uint32_t, pr);
             } else {
-                const int w = n >> 2;
-                if (n & 2) p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, (int)p[X][w], true);
-                else p[X][w] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
+                l_run += ea[k][r - 5];
             }
-        };
-        auto exp_group = [&](int g) {                  // the EPU scores that go with PV unit g
-            if constexpr (EPU == 1) {                  // one score per unit: a pair with every second unit
-                if (g & 1) return;
-                exp_pair(g);
-            } else {
-#pragma unroll
-                for (int e = 0; e < EPU; e += 2) exp_pair(g * EPU + e);
-            }
-            // Pin the group here: an empty volatile statement that consumes the results keeps the
-            // compiler from sinking the exponentials below the matrix instructions they are meant
-            // to overlap with.
-            if constexpr (VARIANT == 0) asm volatile("" : "+v"(l_run), "+v"(p[X][(g * EPU) >> 1]));
-            else asm volatile("" : "+v"(p[X][(g * EPU) >> 2]));
         };
 
-        // At the midpoint every wave has finished iteration t-1 completely, so the ring slots
-        // it read are free: publish K(t+1)/V(t), start the copies of K(t+2) and V(t+1), and
-        // fetch the fragments of K(t+1).
+        // At the barrier every wave has finished the previous tile's steps completely, so the ring
+        // slots they read are free: publish K(t + KOFF) / V(t), start the copies of K(t + KOFF + LEAD)
+        // and V(t + LEAD).
         auto midpoint = [&]() {
-            dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
-            if (kLoopPart != 3) __syncthreads();
-            if (kLoopPart != 4) {
-                dma_k(min(t + LEAD + 1, last), slot_kcopy);
+            if (!(kDbg & 64)) dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
+            if (!(kDbg & 2)) __syncthreads();
+            if (!(kDbg & 1)) {
+            if constexpr (TRIP) {
+                // (the main loop stops early enough that these tiles exist; their addresses are the
+                // trip's base plus a constant)
+                constexpr int dt = ((HT + PERIOD - 1) % PERIOD + 1 % SPT) / SPT;       // tiles since the trip's first step
+                dma_k_at(kg_trip + (dt + KOFF + LEAD) * K_BYTES, slot_kcopy);
+                dma_v_at(vg_trip + (dt + LEAD) * V_BYTES, slot_vcopy);
+            } else {
+                dma_k(min(t + KOFF + LEAD, last), slot_kcopy);
                 dma_v(min(t + LEAD, last), slot_vcopy);
             }
-            read_kf(slot_knext, 0);
+            }
         };
 
-        // ---- softmax(t) interleaved with O^T += V^T(t-1) . P^T(t-1)
 #pragma unroll
-        for (int u = 0; u < NUNIT; u++) {
-            if (!FIRST) {
-                if (u + PD < NUNIT) read_vf(slot_vprev, u + PD);
-                pv_unit(X ^ 1, u);
+        for (int m = 0; m < NM; m++) {
+            // operands of the slots ahead (past the end: of the next step's first slots)
+            auto fetch_slot = [&](int mf) {
+                if (mf < NM) {
+                    if (slot_is_qk(mf) ? DOQK : !FIRST) fetch(mf, slot_kq, kbq, slot_vp, subv);
+                } else {
+                    if (!slot_is_qk(mf - NM) || DOQK) fetch(mf - NM, slot_kq2, kbq2, slot_vp2, subv2);
+                }
+            };
+            if constexpr (GRP == 1) {
+                fetch_slot(m + PDS);
+            } else if (m % GRP == 0) {
+#pragma unroll
+                for (int g = GRP - 1; g >= 0; g--) fetch_slot(m + GRP + g);
             }
-            exp_group(u);
-            if (u == NUNIT / 2 - 1) midpoint();
+            if (slot_is_qk(m)) {
+                if (DOQK) qk_step(X ^ 1, slot_index(m), fr[m][0]);
+            } else if (!FIRST) {
+                pv_unit(X ^ 1, slot_index(m), fr[m]);
+            }
+#pragma unroll
+            for (int n = m * NV / NM; n < (m + 1) * NV / NM; n++) vop(n);
+            if (SUB == 0 && m == NM / 2 - 1) midpoint();
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (OPT) {
+        if (OPT && !(kDbg & 16)) {
             // !(x <= bound) also catches an infinite or NaN sum
-            if (__any(!(l_run - l_before <= 4096.0f))) {
+            if (__builtin_expect(__any(!(l_run - l_before <= 4096.0f)), 0)) {
                 l_run = l_before;
                 decide(0.0f);
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
+                for (int kb = 0; kb < SKB; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
 #pragma unroll
-                for (int n = 0; n < 32; n += 2) exp_pair(n);
+                for (int n = 0; n < NV; n++) vop(n);
             }
         }
-        if (!FIRST && refresh) {
-            // the accumulators include tile t-1 at the old reference; move them to the new one
+        if (!FIRST && __builtin_expect(refresh, 0)) {
+            // the accumulators include step h-1 at the old reference; move them to the new one
             // (the empty volatile statement keeps this rare block a real branch)
             asm volatile("" ::: "memory");
 #pragma unroll
@@ -599,56 +698,82 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512, D > 128 ? 1 : 2) void sage_att
                 for (int i = 0; i < 16; i++) oacc[d][i] *= corr;
             lacc[0] *= corr;
         }
-        // first V^T fragments of tile t for the next iteration (published by this iteration's midpoint)
-#pragma unroll
-        for (int u = 0; u < PD; u++) read_vf(slot_vcur, u);
-        read_kf(slot_knext, 1);
     };
 
     using T = std::true_type;
     using F = std::false_type;
     using X0 = std::integral_constant<int, 0>;
     using X1 = std::integral_constant<int, 1>;
-    using SR = std::integral_constant<int, -1>;         // slots from t at run time
-    // (the split instantiations sit at the register limit and keep their slots in registers)
-    if constexpr (NSK == 4 && NSV == 4 && !SPLIT) {
-        using S0 = std::integral_constant<int, 0>;
-        using S1 = std::integral_constant<int, 1>;
-        using S2 = std::integral_constant<int, 2>;
-        using S3 = std::integral_constant<int, 3>;
-        iteration(0, X0{}, T{}, S0{});
-        int t = 1;
-        for (; t + 3 <= last; t += 4) {
-            iteration(t, X1{}, F{}, S1{});
-            iteration(t + 1, X0{}, F{}, S2{});
-            iteration(t + 2, X1{}, F{}, S3{});
-            iteration(t + 3, X0{}, F{}, S0{});
+    using R0 = std::integral_constant<int, -1>;                         // ring slots from h at run time; first step of a tile
+    using R1 = std::integral_constant<int, SPT == 2 ? -2 : -1>;         // ... the step of odd h
+    // The last step computes no further scores.  (With a single step the first one is also the last;
+    // it computes the scores of the clamped copy and nobody reads them.)
+    int hs = 1;
+    // (the split instantiations sit at the register limit and keep their slots in registers; so do the
+    // ones with an additive mask, whose time goes into reading the mask anyway)
+    if constexpr (NSK == 4 && NSV == 4 && !SPLIT && !ADDMASK) {
+        step(0, X0{}, std::integral_constant<int, 0>{}, T{}, T{});
+        // The main loop takes the steps in front of the first masked key (the ragged end, the masked
+        // range) without looking for masked keys; the steps after that go through the loop below.
+        int clean = (kv_valid - t_off * kTileKV) / SK;
+        if (mask_hi > mask_lo && t_off * kTileKV < mask_hi) clean = min(clean, max(mask_lo - t_off * kTileKV, 0) / SK);
+        // (... and in front of the last tiles, so that the copies a trip starts need no clamping)
+        const int trip_end = min(last_step - SPT * (KOFF + LEAD) + (SPT - 1), clean);
+        for (; hs + PERIOD <= trip_end; hs += PERIOD) {
+            kg_trip = kg + (int64_t)(hs / SPT) * K_BYTES;
+            vg_trip = vg + (int64_t)(hs / SPT) * V_BYTES;
+            {
+                const v4f* kp = reinterpret_cast<const v4f*>(&lds_ks[KS_OFF + t_off * 2 + hs * SKB]);
+                const v4f k0 = kp[0], k1 = kp[1];
+                kst[0] = k0.x; kst[1] = k0.y; kst[2] = k0.z; kst[3] = k0.w;
+                kst[4] = k1.x; kst[5] = k1.y; kst[6] = k1.z; kst[7] = k1.w;
+            }
+            step(hs, X1{}, std::integral_constant<int, 1 % PERIOD>{}, F{}, T{});
+            step(hs + 1, X0{}, std::integral_constant<int, 2 % PERIOD>{}, F{}, T{});
+            step(hs + 2, X1{}, std::integral_constant<int, 3 % PERIOD>{}, F{}, T{});
+            step(hs + 3, X0{}, std::integral_constant<int, 4 % PERIOD>{}, F{}, T{});
+            if constexpr (PERIOD == 8) {
+                step(hs + 4, X1{}, std::integral_constant<int, 5>{}, F{}, T{});
+                step(hs + 5, X0{}, std::integral_constant<int, 6>{}, F{}, T{});
+                step(hs + 6, X1{}, std::integral_constant<int, 7>{}, F{}, T{});
+                step(hs + 7, X0{}, std::integral_constant<int, 0>{}, F{}, T{});
+            }
         }
-        // the last one to three tiles (t is 1 mod 4 here)
-        for (; t < last; t += 2) {
-            iteration(t, X1{}, F{}, SR{});
-            iteration(t + 1, X0{}, F{}, SR{});
-        }
-        if (t == last) iteration(t, X1{}, F{}, SR{});
     } else {
-        iteration(0, X0{}, T{}, SR{});
-        int t = 1;
-        for (; t < last; t += 2) {
-            iteration(t, X1{}, F{}, SR{});
-            iteration(t + 1, X0{}, F{}, SR{});
-        }
-        if (t == last) iteration(t, X1{}, F{}, SR{});
+        step(0, X0{}, R0{}, T{}, T{});
     }
-    // ---- drain: P.V of the last tile ------------------------------------------------------
+    // the remaining steps, ring slots from the step number (hs is odd here)
+    for (; hs + 1 < last_step; hs += 2) {
+        step(hs, X1{}, R1{}, F{}, T{});
+        step(hs + 1, X0{}, R0{}, F{}, T{});
+    }
+    if (hs == last_step) {
+        step(hs, X1{}, R1{}, F{}, F{});
+    } else if constexpr (SPT == 1) {                    // (with two steps per tile the last step is an odd one)
+        if (hs + 1 == last_step) {
+            step(hs, X1{}, R1{}, F{}, T{});
+            step(hs + 1, X0{}, R0{}, F{}, F{});
+        }
+    }
+    // ---- drain: P.V of the last step ------------------------------------------------------
     auto drain = [&](auto x_tag) {
         constexpr int X = decltype(x_tag)::value;
+        v4i vd[NPV][FPU];
+        auto read_vd = [&](int u) {
+            const int j = VARIANT == 0 ? 2 * (SPT - 1) + u / DB : 0, d = u % DB;
 #pragma unroll
-        for (int u = 0; u < NUNIT; u++) {
-            if (u + PD < NUNIT) read_vf(last % NSV, u + PD);
-            pv_unit(X, u);
+            for (int x = 0; x < FPU; x++)
+                vd[u][x] = v_frag(last % NSV, j * FPU + x, d);
+        };
+#pragma unroll
+        for (int u = 0; u < PD && u < NPV; u++) read_vd(u);
+#pragma unroll
+        for (int u = 0; u < NPV; u++) {
+            if (u + PD < NPV) read_vd(u + PD);
+            pv_unit(X, u, vd[u]);
         }
     };
-    if (last & 1) drain(X1{});
+    if (SPT == 2 || (last_step & 1)) drain(X1{});
     else drain(X0{});
 
     // Hand-over between workgroups of ONE XCD goes through that XCD's L2, which every compute unit
@@ -780,11 +905,11 @@ __global__ void split_clear_kernel(int* flags, int n) {
 
 template <int D, int VARIANT>
 static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
-    constexpr int kThreads = D > 128 ? 256 : 512;             // 32 query rows per wave
+    constexpr int kThreads = D > 128 ? 256 : SAGE_NW * 64;             // 32 query rows per wave
     const int n_qtiles = (int)(a.nq_pad / (kThreads / 2));
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    const int split = D > 128 ? 0 : attn_split_workgroups(a.B, a.H, a.Nq, a.kv_valid, D);
+    const int split = attn_split_workgroups(a.B, a.H, a.Nq, a.kv_valid, D, VARIANT);
     int* flags = nullptr;
     float* part = nullptr;
     if (split > 0) {
@@ -802,7 +927,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
                        (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags, g_split_wait.load())
 #define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                                  \
     do {                                                                  \
-        if constexpr (D <= 128) {                                         \
+        if constexpr (D <= 128 && VARIANT == 0) {                         \
             if (split > 0) SAGE_LAUNCH_ATTN2(STATS, ADDMASK, true);       \
             else SAGE_LAUNCH_ATTN2(STATS, ADDMASK, false);                \
         } else {                                                          \
@@ -836,11 +961,12 @@ static std::atomic<int> g_split_mode{0};       // 0: by shape; -1: never; n > 0:
 
 void attn_split_override(int mode) { g_split_mode.store(mode); }
 
-int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D) {
+int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D, int variant) {
 #ifdef SAGE_CLOCK_PROBE
     return 0;                                  // the measurement build reports per-item clocks
 #else
     if (D > 128) return 0;                     // four-wave workgroups: one per item
+    if (variant != 0) return 0;                // the e4m3 loop has no registers left for the hand-over
     const int64_t items = pad_to(Nq, kTileQ) / kTileQ * B * H;
     const int64_t ntiles = (kv_valid + kTileKV - 1) / kTileKV;
     const int mode = g_split_mode.load();
@@ -864,11 +990,7 @@ size_t attn_split_bytes(int workgroups, int D) {
 }
 
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st) {
-    if (a.nkv_pad / a.blkk > kMaxKScales) return hipErrorInvalidValue;      // K scales would not fit the LDS staging
-#if SAGE_LOOP_PART != 0
-    if (a.D != 128 || a.amask != nullptr || a.stats != nullptr) return hipErrorInvalidValue;
-    return a.variant == 0 ? launch_attn_dv<128, 0>(a, st) : launch_attn_dv<128, 1>(a, st);
-#endif
+    if (a.nkv_pad > max_keys(a.D)) return hipErrorInvalidValue;      // K scales would not fit the LDS staging
     if (a.D == 128) return a.variant == 0 ? launch_attn_dv<128, 0>(a, st) : launch_attn_dv<128, 1>(a, st);
     if (a.D == 64) return a.variant == 0 ? launch_attn_dv<64, 0>(a, st) : launch_attn_dv<64, 1>(a, st);
     if (a.D == 256) return a.variant == 0 ? launch_attn_dv<256, 0>(a, st) : launch_attn_dv<256, 1>(a, st);

@@ -13,7 +13,9 @@ constexpr int kTileKV = 64;    // keys per main-loop iteration
 constexpr int kPadKV  = 128;   // key tokens are padded to this (every scale-block size divides it)
 constexpr int kLeaf   = 16;    // tokens per leaf of the K-mean summation tree
 constexpr int kGroup  = 256;   // tokens per group (16 leaves)
-constexpr int kMaxKScales = 4096;   // K scale blocks per head the attention kernel stages in LDS (16 KiB)
+// The attention kernel stages one head's K scales in LDS, one entry per 32 keys: keys per head it takes
+// (256 channels: the tile rings leave room for a quarter as many entries).
+__host__ __device__ constexpr int max_keys(int D) { return (D > 128 ? 2048 : 8192) * 32; }
 
 inline int64_t pad_to(int64_t n, int64_t m) { return (n + m - 1) / m * m; }
 
@@ -118,7 +120,7 @@ hipError_t launch_attn(const AttnArgs& a, hipStream_t st);
 // Shapes whose items do not fill whole rounds of workgroups are spread evenly over a fixed number
 // of workgroups that hand partial results to each other through `split`.  Number of workgroups
 // (a multiple of 8), or 0 for one workgroup per item; depends on the shape only.
-int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D);
+int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D, int variant);
 size_t attn_split_bytes(int workgroups, int D);
 constexpr size_t kSplitFlagBytes = 4096;     // one int per workgroup in front of the state slots
 constexpr int kSplitMaxWorkgroups = 1024;
