@@ -136,7 +136,7 @@ def clock_probe(args, L, w, qd, kd, vd, o, st, stream):
     import numpy as np
     import torch
     from mojodiffusion_amd import _lib
-    P = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libmi355_sage_probe.so"))
+    P = ctypes.CDLL(args.probe_lib or os.path.join(os.path.dirname(_lib.LIB_PATH), "libmi355_sage_probe.so"))
     for name in ("mi355_sage_quant_qk_bf16", "mi355_sage_quant_v_f16", "mi355_sage_quant_v_fp8", "mi355_sage_attn_fwd"):
         getattr(P, name).restype, getattr(P, name).argtypes = _lib.SIGNATURES[name]
     B, S, H, D = w.B, w.S, w.H, w.D
@@ -187,50 +187,82 @@ def clock_probe(args, L, w, qd, kd, vd, o, st, stream):
     }))
 
 
-LOOP_PARTS = {1: "no exponentials", 2: "no LDS fragment reads", 3: "no workgroup barrier in the loop",
-              4: "no tile copies in the loop", 5: "no P.V matrix instructions", 6: "one score instruction per chain instead of four"}
-
-
-def loop_parts(args, L, w, qd, kd, vd, o, st, ws, stream, ms_first):
-    """What each part of the attention loop is worth in the real kernel: the same step through the
-    shipped library and through builds that leave one part out (their results are wrong by design),
-    in turn, several rounds, medians."""
-    import torch
+def run_workload(L, torch, w, qd, kd, vd, steps, warmup, n_events):
+    """One workload through the one-shot call (wall clock over back-to-back steps) and through the
+    stage entry points with HIP events on the launch stream: the quantize stage as the one-shot call
+    runs it (three launches, mi355_sage_quant_qkv_bf16) and the attention kernel."""
     from mojodiffusion_amd import _lib
-    libs = {0: L}
-    for n in LOOP_PARTS:
-        path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libmi355_sage_part%d.so" % n)
-        if not os.path.exists(path):
-            print("bench.py: %s is missing; run `make -C mojodiffusion_amd/csrc parts` first" % path, file=sys.stderr)
-            sys.exit(4)
-        P = ctypes.CDLL(path)
-        P.mi355_sage_sdpa_bf16_ex.restype, P.mi355_sage_sdpa_bf16_ex.argtypes = _lib.SIGNATURES["mi355_sage_sdpa_bf16_ex"]
-        libs[n] = P
+    dev = qd.device
     B, S, H, D = w.B, w.S, w.H, w.D
+    o = torch.empty_like(qd)
+    st = _lib.strides_bhnd(S, H, D)
+    nws = L.mi355_sage_workspace_bytes(B, H, S, S, D, w.variant)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
 
-    def step(P):
-        rc = P.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), B, H, S, S, D, w.scale,
-                                       st, st, st, st, 0, 0, 0, 0, 0, stream, w.variant, w.blkq, w.blkk, K_FLAGS,
-                                       ws.data_ptr(), ws.numel())
+    def step(on_stream=stream):
+        rc = L.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
+                                       B, H, S, S, D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, on_stream,
+                                       w.variant, w.blkq, w.blkk, K_FLAGS, ws.data_ptr(), nws)
         if rc != 0:
-            raise RuntimeError("rc=%d" % rc)
+            raise RuntimeError("mi355_sage_sdpa_bf16_ex rc=%d" % rc)
 
-    times = {n: [] for n in libs}
-    for _ in range(7):
-        for n, P in libs.items():
-            for _ in range(20):
-                step(P)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                step(P)
-            torch.cuda.synchronize()
-            times[n].append((time.perf_counter() - t0) * 1e3 / args.steps)
-    med = {n: sorted(t)[len(t) // 2] for n, t in times.items()}
-    out = {"workload": w.name, "steps_per_round": args.steps, "rounds": 7, "shipped_ms_per_step": round(med[0], 5), "parts": {}}
-    for n, what in LOOP_PARTS.items():
-        out["parts"][what] = {"ms_per_step": round(med[n], 5), "vs_shipped_pct": round(100.0 * (med[n] / med[0] - 1.0), 1)}
-    print(json.dumps(out))
+    # The chip takes some milliseconds of load to leave its idle clocks (a 50-step run right after
+    # start-up reads 12 % slower than a 1000-step one): run the same step, untimed, for 0.15 s
+    # before the warm-up proper, whatever --warmup says.
+    ramp_steps = 0
+    r0 = time.perf_counter()
+    while time.perf_counter() - r0 < 0.15:
+        for _ in range(4):
+            step()
+        torch.cuda.synchronize()
+        ramp_steps += 4
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
+    q8 = torch.empty((B, H, nqp, D), dtype=torch.int8, device=dev)
+    k8 = torch.empty((B, H, nkp, D), dtype=torch.int8, device=dev)
+    qs = torch.empty((B, H, nqp // w.blkq), dtype=torch.float32, device=dev)
+    ks = torch.empty((B, H, nkp // w.blkk), dtype=torch.float32, device=dev)
+    km, qm, kmu, vsc = (torch.empty((B, H, D), dtype=torch.float32, device=dev) for _ in range(4))
+    vq = torch.empty((B, H, nkp // 64, D, 64), dtype=torch.int16 if w.variant == 0 else torch.uint8, device=dev)
+    scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, H, S, D), 8), dtype=torch.uint8, device=dev)
+
+    def stage_quant():
+        return L.mi355_sage_quant_qkv_bf16(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), B, H, S, S, D, w.scale, st, st, st,
+                                           0, 0, 0, w.variant, w.blkq, w.blkk, K_FLAGS, 0, 0, q8.data_ptr(), qs.data_ptr(),
+                                           k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
+                                           vq.data_ptr(), vsc.data_ptr(), scr.data_ptr(), scr.numel(), stream)
+
+    def stage_attn():
+        return L.mi355_sage_attn_fwd(q8.data_ptr(), qs.data_ptr(), w.blkq, k8.data_ptr(), ks.data_ptr(), w.blkk,
+                                     vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, 0, 0, D,
+                                     o.data_ptr(), st, 0, None, None, stream)
+
+    def time_stage(fn, n):
+        for _ in range(3):
+            assert fn() == 0
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for a, b in evs:
+            a.record()
+            assert fn() == 0
+            b.record()
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
+
+    qt_avg, qt_med, qt_min = time_stage(stage_quant, n_events)
+    at_avg, at_med, at_min = time_stage(stage_attn, n_events)
+    return dict(step=step, ms_per_step=ms_per_step, ramp_steps=ramp_steps, quant=(qt_avg, qt_med, qt_min),
+                attn=(at_avg, at_med, at_min), keep=(o, ws, q8, k8, qs, ks, km, qm, kmu, vsc, vq, scr))
 
 
 def main():
@@ -240,15 +272,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-other-workloads", action="store_true",
+                    help="leave out config.other_workloads (the other DiT shapes, a few steps each)")
     ap.add_argument("--summarize-traffic", nargs=4, metavar="DIR",
                     help="print the traffic summary from four rocprofv3 --pmc output directories (no GPU needed)")
     ap.add_argument("--clock-probe", action="store_true",
-                    help="run the attention kernel of the measurement build (libmi355_sage_probe.so), which records "
+                    help="run the attention kernel of a measurement build (default libmi355_sage_probe.so), which records "
                          "its own shader cycles and elapsed constant-rate time per workgroup, and print the clock "
-                         "the chip sustained under it")
-    ap.add_argument("--loop-parts", action="store_true",
-                    help="time the step with the measurement builds that leave one part of the attention loop out "
-                         "(make -C mojodiffusion_amd/csrc parts), all in this process, in turn")
+                         "the chip sustained under it and the shader clocks a 64-key tile took")
+    ap.add_argument("--probe-lib", default=None, help="measurement build --clock-probe loads (a path)")
+    ap.add_argument("--probe-heads", type=int, default=None,
+                    help="--clock-probe with this many heads instead of the workload's (few heads: a cool, idle chip)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain device copy of 256 MiB (read 256 MiB, write 256 MiB) five times: "
                          "the known-size kernel the HBM traffic counters are scaled by")
@@ -265,7 +299,7 @@ def main():
     import torch
 
     from mojodiffusion_amd import _lib
-    from mojodiffusion_amd.workloads import WORKLOADS, make_inputs
+    from mojodiffusion_amd.workloads import WORKLOADS, make_inputs, device_inputs
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the library has no CPU path", file=sys.stderr)
@@ -282,52 +316,26 @@ def main():
         return
     L = _lib.lib()
     w = WORKLOADS[args.workload]
+    if args.clock_probe and args.probe_heads:
+        w = w.scaled(H=args.probe_heads)
     q, k, v = make_inputs(w)
     up = lambda x: torch.from_numpy(x.view(np.int16)).to(dev).view(torch.bfloat16)
     qd, kd, vd = up(q), up(k), up(v)
-    o = torch.empty_like(qd)
     B, S, H, D = w.B, w.S, w.H, w.D
     st = _lib.strides_bhnd(S, H, D)
-    nws = L.mi355_sage_workspace_bytes(B, H, S, S, D, w.variant)
-    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
 
-    def step():
-        rc = L.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
-                                       B, H, S, S, D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, stream,
-                                       w.variant, w.blkq, w.blkk, K_FLAGS, ws.data_ptr(), nws)
-        if rc != 0:
-            raise RuntimeError("mi355_sage_sdpa_bf16_ex rc=%d" % rc)
+    if args.clock_probe:
+        clock_probe(args, L, w, qd, kd, vd, torch.empty_like(qd), st, stream)
+        return
 
-    # The chip takes some milliseconds of load to leave its idle clocks (a 50-step run right after
-    # start-up reads 12 % slower than a 1000-step one): run the same step, untimed, for 0.15 s
-    # before the warm-up proper, whatever --warmup says.
-    ramp_steps = 0
-    r0 = time.perf_counter()
-    while time.perf_counter() - r0 < 0.15:
-        for _ in range(20):
-            step()
-        torch.cuda.synchronize()
-        ramp_steps += 20
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    n_ev = max(args.steps, 20)
+    r = run_workload(L, torch, w, qd, kd, vd, args.steps, args.warmup, n_ev)
+    ms_per_step = r["ms_per_step"]
     tops = w.ops / (ms_per_step * 1e-3) / 1e12
 
-    if args.clock_probe:
-        clock_probe(args, L, w, qd, kd, vd, o, st, stream)
-        return
-    if args.loop_parts:
-        loop_parts(args, L, w, qd, kd, vd, o, st, ws, stream, ms_per_step)
-        return
-
-    # ---- the same step replayed from a HIP graph (launch gaps shrink to the graph's own) -----
+    # ---- the same step replayed from a HIP graph: what a caller that captures its layer loop sees.
+    # 200 replays after 50, whatever --steps says (a handful of replays mostly measures the ramp).
     graph_ms = None
     try:
         side = torch.cuda.Stream()
@@ -336,77 +344,27 @@ def main():
         with torch.cuda.stream(side):
             cap_stream = torch.cuda.current_stream().cuda_stream
             with torch.cuda.graph(g, stream=side):
-                rc = L.mi355_sage_sdpa_bf16_ex(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(),
-                                               B, H, S, S, D, w.scale, st, st, st, st, 0, 0, 0, 0, 0, cap_stream,
-                                               w.variant, w.blkq, w.blkk, K_FLAGS, ws.data_ptr(), nws)
-            if rc != 0:
-                raise RuntimeError("capture rc=%d" % rc)
-            for _ in range(args.warmup):
+                r["step"](cap_stream)
+            for _ in range(50):
                 g.replay()
             torch.cuda.synchronize()
             g0 = time.perf_counter()
-            for _ in range(args.steps):
+            for _ in range(200):
                 g.replay()
             torch.cuda.synchronize()
-            graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
+            graph_ms = (time.perf_counter() - g0) * 1e3 / 200
     except Exception as e:                                  # reported, never fatal for the headline number
         print("bench.py: graph replay timing skipped: %r" % (e,), file=sys.stderr)
     torch.cuda.synchronize()
 
-    # ---- stage timings with HIP events on the launch stream -------------------------
-    nqp, nkp = L.mi355_sage_pad_q(S), L.mi355_sage_pad_kv(S)
-    q8 = torch.empty((B, H, nqp, D), dtype=torch.int8, device=dev)
-    k8 = torch.empty((B, H, nkp, D), dtype=torch.int8, device=dev)
-    qs = torch.empty((B, H, nqp // w.blkq), dtype=torch.float32, device=dev)
-    ks = torch.empty((B, H, nkp // w.blkk), dtype=torch.float32, device=dev)
-    km, qm, kmu = (torch.empty((B, H, D), dtype=torch.float32, device=dev) for _ in range(3))
-    vsc = torch.empty((B, H, D), dtype=torch.float32, device=dev)
-    vq = torch.empty((B, H, nkp // 64, D, 64), dtype=torch.int16 if w.variant == 0 else torch.uint8, device=dev)
-    scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, H, S, D), 8), dtype=torch.uint8, device=dev)
-
-    def stage_quant_qk():
-        return L.mi355_sage_quant_qk_bf16(qd.data_ptr(), kd.data_ptr(), B, H, S, S, D, w.scale, st, st, 0, 0,
-                                          w.blkq, w.blkk, K_FLAGS, 0, 0, q8.data_ptr(), qs.data_ptr(), k8.data_ptr(),
-                                          ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
-                                          scr.data_ptr(), scr.numel(), stream)
-
-    def stage_quant_v():
-        if w.variant == 0:
-            return L.mi355_sage_quant_v_f16(vd.data_ptr(), B, H, S, D, st, 0, 0, 0, vq.data_ptr(), stream)
-        return L.mi355_sage_quant_v_fp8(vd.data_ptr(), B, H, S, D, st, 0, 0, 0, vq.data_ptr(), vsc.data_ptr(),
-                                        scr.data_ptr(), scr.numel(), stream)
-
-    def stage_attn():
-        return L.mi355_sage_attn_fwd(q8.data_ptr(), qs.data_ptr(), w.blkq, k8.data_ptr(), ks.data_ptr(), w.blkk,
-                                     vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, 0, 0, D,
-                                     o.data_ptr(), st, 0, None, None, stream)
-
-    def time_stage(fn, n):
-        assert fn() == 0
-        torch.cuda.synchronize()
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-        for a, b in evs:
-            a.record()
-            assert fn() == 0
-            b.record()
-        torch.cuda.synchronize()
-        ts = sorted(a.elapsed_time(b) for a, b in evs)
-        return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
-
-    n_ev = max(args.steps, 20)
-    qk_avg, qk_med, _ = time_stage(stage_quant_qk, n_ev)
-    v_avg, v_med, _ = time_stage(stage_quant_v, n_ev)
-    at_avg, at_med, at_min = time_stage(stage_attn, n_ev)
+    qt_avg, qt_med, qt_min = r["quant"]
+    at_avg, at_med, at_min = r["attn"]
     attn_tops = w.ops / (at_avg * 1e-3) / 1e12
     peak = PEAK_INT8_TOPS if w.variant == 0 else PEAK_FP8_TOPS
     # algorithmic HBM bytes of the quantize stage: Q,K,V read once as bf16; int8 Q/K and fp16/e4m3 V written
     elems = B * H * S * D
     quant_bytes = 3 * elems * 2 + 2 * elems + elems * (2 if w.variant == 0 else 1)
-    quant_gbs = quant_bytes / ((qk_avg + v_avg) * 1e-3) / 1e9
-    # the timed step runs the one-shot call, whose quantizers share launches (V repack with the K
-    # statistics, Q with K encode): its quantize share is the step minus the attention launch
-    one_shot_quant_ms = ms_per_step - at_avg
-    one_shot_gbs = quant_bytes / (one_shot_quant_ms * 1e-3) / 1e9 if one_shot_quant_ms > 0 else None
+    quant_gbs = quant_bytes / (qt_avg * 1e-3) / 1e9
 
     out = {
         "metric": METRIC,
@@ -429,18 +387,12 @@ def main():
             "ops_per_step": w.ops,
             "pct_of_peak": round(100.0 * tops / peak, 2),
             "peak_tops_used": peak,
-            # the stage entry points, each timed on its own (the one-shot call fuses the quantizers
-            # into two launches, so its quantize share is about ms_per_step - attn)
-            "stage_ms": {"quant_qk": round(qk_avg, 5), "quant_v": round(v_avg, 5), "attn": round(at_avg, 5)},
-            "one_shot_quant_ms": round(one_shot_quant_ms, 5),
+            # HIP-event pairs on the launch stream around the quantize stage as the step runs it (three
+            # launches through mi355_sage_quant_qkv_bf16) and around the attention launch
+            "stage_ms": {"quant_qkv": round(qt_avg, 5), "attn": round(at_avg, 5)},
             "graph_replay_ms": None if graph_ms is None else round(graph_ms, 5),
-            "clock_ramp_steps": ramp_steps,      # untimed steps run before the warm-up, see above
-            # "GB/s": the stage entry points called one after the other (Q/K, then V: five launches);
-            # "one_shot_GB/s": the three launches the timed step really runs
-            "quant_stage_hbm": {"algorithmic_bytes": quant_bytes, "GB/s": round(quant_gbs, 1),
-                                "frac_of_8TB/s": round(quant_gbs / PEAK_HBM_GBS, 4),
-                                "one_shot_GB/s": None if one_shot_gbs is None else round(one_shot_gbs, 1),
-                                "one_shot_frac_of_8TB/s": None if one_shot_gbs is None else round(one_shot_gbs / PEAK_HBM_GBS, 4)},
+            "graph_replays": 200,
+            "clock_ramp_steps": r["ramp_steps"],      # untimed steps run before the warm-up, see run_workload
             "device": torch.cuda.get_device_name(0),
         },
         "roofline": {
@@ -456,11 +408,41 @@ def main():
             "avg_ms": round(at_avg, 5), "median_ms": round(at_med, 5), "min_ms": round(at_min, 5),
             "algorithmic_ops_per_launch": w.ops,
         },
+        # the HBM-bound part of the step: prep_kernel, stats_final_kernel, quant_kernel together
+        "roofline_quantize": {
+            "kernels": "prep_kernel + stats_final_kernel + quant_kernel (one event pair around the three launches)",
+            "bound": "hbm",
+            "achieved": round(quant_gbs, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(quant_gbs / PEAK_HBM_GBS, 4),
+            "algorithmic_bytes": quant_bytes,
+            "avg_ms": round(qt_avg, 5), "median_ms": round(qt_med, 5), "min_ms": round(qt_min, 5),
+        },
     }
+    del r
+
+    if not args.skip_other_workloads and args.workload == 2:
+        # The other DiT shapes at full size with inputs drawn on the device: a few timed steps each.
+        others = {}
+        plan = {3: (40, 10), 4: (12, 4), 5: (5, 2)}
+        for wid, (n_steps, n_warm) in plan.items():
+            ww = WORKLOADS[wid]
+            qq, kk, vv = device_inputs(ww, 7000 + wid)
+            rr = run_workload(L, torch, ww, qq, kk, vv, n_steps, n_warm, max(n_steps // 2, 5))
+            pk = PEAK_INT8_TOPS if ww.variant == 0 else PEAK_FP8_TOPS
+            t_ = ww.ops / (rr["ms_per_step"] * 1e-3) / 1e12
+            a_ = ww.ops / (rr["attn"][0] * 1e-3) / 1e12
+            others[ww.name] = {"steps": n_steps, "warmup": n_warm, "ms_per_step": round(rr["ms_per_step"], 4),
+                               "TOPS": round(t_, 1), "pct_of_peak": round(100.0 * t_ / pk, 2),
+                               "attn_kernel_avg_ms": round(rr["attn"][0], 4), "attn_kernel_frac_of_peak": round(a_ / pk, 4),
+                               "quant_qkv_avg_ms": round(rr["quant"][0], 4), "dtype": "int8/f16" if ww.variant == 0 else "int8/f8e4m3"}
+            del rr, qq, kk, vv
+            torch.cuda.empty_cache()
+        out["config"]["other_workloads"] = others
 
     if not args.skip_cpu_baseline:
         from oracle import sage_oracle
-        # bounded sample: a subset of heads at the full sequence length
         # bounded sample: whole passes over a subset of heads at the full sequence length, repeated
         # until about ten seconds of CPU work have been timed
         heads = min(H, 8)

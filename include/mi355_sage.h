@@ -295,6 +295,21 @@ int mi355_sage_quant_qk_norm_rope_bf16(
     void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
     void* scratch, size_t scratch_bytes, void* stream);
 
+/* Q, K and V in the three launches the one-shot calls use (V repack or V channel maxima ride
+ * with the K statistics, the e4m3 V encode with the Q / K encoders): same outputs, bit for bit, as
+ * mi355_sage_quant_qk_bf16 followed by mi355_sage_quant_v_f16 / _fp8, which take five.  vq is v16
+ * or v8 by `variant`; vscale is written for MI355_SAGE_PV_FP8 only (may be NULL otherwise).
+ * scratch as for mi355_sage_quant_qk_bf16. */
+int mi355_sage_quant_qkv_bf16(
+    const void* Q, const void* K, const void* V,
+    int B, int H, int N_q, int N_kv, int D, float scale,
+    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+    int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+    int variant, int blkq, int blkk, int k_flags, int mask_lo, int mask_hi,
+    void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
+    void* vq, void* vscale,
+    void* scratch, size_t scratch_bytes, void* stream);
+
 /* V -> fp16 (round-to-nearest-even, finite overflow saturates), tiled layout. */
 int mi355_sage_quant_v_f16(
     const void* V, int B, int H, int N_kv, int D,

@@ -36,6 +36,8 @@ SIGNATURES = {
     "mi355_sage_quant_scratch_bytes": (ctypes.c_size_t, [_int] * 4),
     "mi355_sage_quant_qk_bf16": (_int, [_vp, _vp] + [_int] * 5 + [ctypes.c_float, _i64p, _i64p, _i64, _i64]
                                  + [_int] * 5 + [_vp] * 8 + [ctypes.c_size_t, _vp]),
+    "mi355_sage_quant_qkv_bf16": (_int, [_vp] * 3 + [_int] * 5 + [ctypes.c_float, _i64p, _i64p, _i64p, _i64, _i64, _i64]
+                                  + [_int] * 6 + [_vp] * 10 + [ctypes.c_size_t, _vp]),
     "mi355_sage_quant_qk_norm_rope_bf16": (_int, [_vp, _vp] + [_int] * 5 + [ctypes.c_float, _i64p, _i64p, _i64, _i64]
                                            + [_vp, _vp, ctypes.c_float, _vp, _vp, _i64, _int]
                                            + [_int] * 3 + [_vp] * 8 + [ctypes.c_size_t, _vp]),

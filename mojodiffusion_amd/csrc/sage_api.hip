@@ -601,6 +601,42 @@ int mi355_sage_sdpa_bf16_norm_rope_train_fwd(const void* Q, const void* K, const
                      default_blkq(variant), 64, kDefaultFlags, workspace, workspace_bytes, pre);
 }
 
+int mi355_sage_quant_qkv_bf16(const void* Q, const void* K, const void* V, int B, int H, int N_q, int N_kv, int D,
+                              float scale, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                              int64_t q_off, int64_t k_off, int64_t v_off,
+                              int variant, int blkq, int blkk, int k_flags, int mask_lo, int mask_hi,
+                              void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
+                              void* vq, void* vscale, void* scratch, size_t scratch_bytes, void* stream) {
+    if (!Q || !K || !V || !q8 || !qscale || !k8 || !kscale || !kmean || !qmul || !kmul || !vq || !scratch) return MI355_SAGE_EINVAL;
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
+    if (!q_strides || !k_strides || !v_strides) return MI355_SAGE_EINVAL;
+    if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
+    if (variant == MI355_SAGE_PV_FP8 && !vscale) return MI355_SAGE_EINVAL;
+    if (!dims_ok(D) || !blk_ok(blkq) || !blk_ok(blkk) || (k_flags & ~3)) return MI355_SAGE_EUNSUPPORTED;
+    const ScratchCarve sc = scratch_carve(B, H, N_kv, D);
+    if (scratch_bytes < sc.total) return MI355_SAGE_EWORKSPACE;
+    int rc;
+    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("K", K, k_strides, k_off)) ||
+        (rc = check_view("V", V, v_strides, v_off)))
+        return rc;
+    KeyMask km;
+    const int kept = clip_mask(N_kv, mask_lo, mask_hi, &km);
+    if (kept <= 0) return MI355_SAGE_EINVAL;
+    uint8_t* scr = static_cast<uint8_t*>(scratch);
+    QuantOut o{};
+    o.q8 = static_cast<int8_t*>(q8); o.qscale = static_cast<float*>(qscale);
+    o.k8 = static_cast<int8_t*>(k8); o.kscale = static_cast<float*>(kscale);
+    o.kmean = static_cast<float*>(kmean); o.qmul = static_cast<float*>(qmul); o.kmul = static_cast<float*>(kmul);
+    o.kpart_sum = reinterpret_cast<double*>(scr + sc.kpart_sum);
+    o.kpart_mm = reinterpret_cast<float*>(scr + sc.kpart_mm);
+    o.rowinv_q = reinterpret_cast<float*>(scr + sc.rowinv_q);
+    o.rowinv_k = reinterpret_cast<float*>(scr + sc.rowinv_k);
+    const View v = make_view(V, v_strides, v_off);
+    return quantize(make_view(Q, q_strides, q_off), make_view(K, k_strides, k_off), &v, B, H, N_q, N_kv, D, scale,
+                    blkq, blkk, k_flags, km, kept, o, variant, vq, static_cast<float*>(vscale),
+                    reinterpret_cast<float*>(scr + sc.vpart), Pre{}, static_cast<hipStream_t>(stream));
+}
+
 int mi355_sage_quant_v_f16(const void* V, int B, int H, int N_kv, int D, const int64_t* v_strides,
                            int64_t v_off, int mask_lo, int mask_hi, void* v16, void* stream) {
     if (!V || !v16 || !v_strides) return MI355_SAGE_EINVAL;

@@ -32,11 +32,16 @@
 #include <atomic>
 #include <type_traits>
 
-#ifndef SAGE_DBG
-#define SAGE_DBG 0
+// Measurement builds only (`make parts`, never part of the library): SAGE_LOOP_PART is a mask of
+// parts of the main loop to leave out, so that what each is worth can be read off the kernel's own
+// clock stamps (bench.py --clock-probe --probe-lib ...).  Results are wrong by design; every kernel
+// still runs to its end (no address and no trip count depends on what is left out).
+//   1 no tile copies in the loop   2 no workgroup barrier in the loop   4 no LDS fragment reads
+#ifndef SAGE_LOOP_PART
+#define SAGE_LOOP_PART 0
 #endif
 namespace sage {
-constexpr int kDbg = SAGE_DBG;   // TEMPORARY measurement switches: 1 no copies, 2 no barrier, 4 no fragment reads, 8 no kscale read, 16 no OPT check, 32 no mask check, 64 no vmcnt wait
+constexpr int kLoopPart = SAGE_LOOP_PART;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -406,7 +411,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
     // e4m3 variant reads both blocks) of the K tile in `kslot` and whose P.V instructions read the
     // steps `sub` of the V^T tile in `vslot`.
     auto fetch = [&](int m, int kslot, int kbq, int vslot, int sub) {
-        if (kDbg & 4) { asm volatile("" : "+v"(fr[m][0])); return; }
+        if (kLoopPart & 4) { asm volatile("" : "+v"(fr[m][0])); return; }
         if (slot_is_qk(m)) {
             const int n = slot_index(m), st = SKB == 1 ? n : n >> 1, kb = SKB == 1 ? kbq : n & 1;
             fr[m][0] = k_frag(kslot, st, kb);
@@ -635,9 +640,9 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
         // slots they read are free: publish K(t + KOFF) / V(t), start the copies of K(t + KOFF + LEAD)
         // and V(t + LEAD).
         auto midpoint = [&]() {
-            if (!(kDbg & 64)) dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
-            if (!(kDbg & 2)) __syncthreads();
-            if (!(kDbg & 1)) {
+            dma_wait<ADDMASK ? 0 : (LEAD - 1) * (K_CH + V_CH)>();
+            if (!(kLoopPart & 2)) __syncthreads();
+            if (!(kLoopPart & 1)) {
             if constexpr (TRIP) {
                 // (the main loop stops early enough that these tiles exist; their addresses are the
                 // trip's base plus a constant)
@@ -677,7 +682,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
             if (SUB == 0 && m == NM / 2 - 1) midpoint();
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (OPT && !(kDbg & 16)) {
+        if (OPT) {
             // !(x <= bound) also catches an infinite or NaN sum
             if (__builtin_expect(__any(!(l_run - l_before <= 4096.0f)), 0)) {
                 l_run = l_before;

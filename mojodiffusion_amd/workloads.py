@@ -89,3 +89,28 @@ def make_inputs(w):
         out.append(np.ascontiguousarray(f32_to_bf16_bits(x).transpose(0, 2, 1, 3)))
         del x
     return tuple(out)
+
+
+def device_inputs(w, seed):
+    """(q, k, v) bf16 torch tensors [B, S, H, D] on the GPU with the workload's statistics, drawn by
+    torch's device generator: for full-size runs that need no bit-reproducible host copy (the
+    largest workload takes minutes to draw on the host)."""
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    shape = (w.B, w.S, w.H, w.D)
+    q = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    k = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32)
+    if w.k_offset_std > 0:
+        k += w.k_offset_std * torch.randn((w.B, 1, w.H, w.D), generator=g, device="cuda", dtype=torch.float32)
+    if w.k_outlier_frac > 0:
+        n = int(np.ceil(w.k_outlier_frac * w.D))
+        gain = torch.ones((w.B, 1, w.H, w.D), device="cuda")
+        for b in range(w.B):
+            for h in range(w.H):
+                idx = torch.randperm(w.D, generator=g, device="cuda")[:n]
+                gain[b, 0, h, idx] = w.k_outlier_gain
+        k *= gain
+    k = k.to(torch.bfloat16)
+    v = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    return q, k, v

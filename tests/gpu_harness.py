@@ -115,6 +115,33 @@ def quant_v(v_bits, variant, mask=(0, 0), strides=None, v_off=0, shape=None):
     return dict(vq=out.cpu().numpy(), vscale=vs.cpu().numpy(), dev=dict(vq=out, vscale=vs))
 
 
+def quant_qkv(q_bits, k_bits, v_bits, scale, variant, blkq, blkk, mask=(0, 0)):
+    """mi355_sage_quant_qkv_bf16: the three launches of the one-shot calls.  Same dict as quant_qk plus vq, vscale."""
+    L = _lib.lib()
+    B, Sq, H, D = q_bits.shape
+    Skv = k_bits.shape[1]
+    sq, sk = _lib.strides_bhnd(Sq, H, D), _lib.strides_bhnd(Skv, H, D)
+    qd, kd, vd = dev_bf16(q_bits), dev_bf16(k_bits), dev_bf16(v_bits)
+    nqp, nkp = L.mi355_sage_pad_q(Sq), L.mi355_sage_pad_kv(Skv)
+    q8 = torch.full((B, H, nqp, D), 77, dtype=torch.int8, device="cuda")
+    k8 = torch.full((B, H, nkp, D), 77, dtype=torch.int8, device="cuda")
+    qs = torch.full((B, H, nqp // blkq), -1.0, dtype=torch.float32, device="cuda")
+    ks = torch.full((B, H, nkp // blkk), -1.0, dtype=torch.float32, device="cuda")
+    km, qm, kmu, vs = (torch.full((B, H, D), -1.0, dtype=torch.float32, device="cuda") for _ in range(4))
+    vq = torch.full((B, H, nkp // 64, D, 64), 0x7E, dtype=torch.int16 if variant == 0 else torch.uint8, device="cuda")
+    scr = torch.full((max(L.mi355_sage_quant_scratch_bytes(B, H, Skv, D), 8),), 0xAB, dtype=torch.uint8, device="cuda")
+    rc = L.mi355_sage_quant_qkv_bf16(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), B, H, Sq, Skv, D, scale, sq, sk, sk, 0, 0, 0,
+                                     variant, blkq, blkk, _lib.K_SMOOTH | _lib.K_BALANCE, mask[0], mask[1],
+                                     q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(),
+                                     kmu.data_ptr(), vq.data_ptr(), vs.data_ptr(), scr.data_ptr(), scr.numel(), stream())
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    vq_np = vq.cpu().numpy()
+    return dict(q8=q8.cpu().numpy(), qscale=qs.cpu().numpy(), k8=k8.cpu().numpy(), kscale=ks.cpu().numpy(),
+                kmean=km.cpu().numpy(), qmul=qm.cpu().numpy(), kmul=kmu.cpu().numpy(),
+                vq=vq_np.view(np.uint16) if variant == 0 else vq_np, vscale=vs.cpu().numpy() if variant == 1 else None)
+
+
 def attn_fwd(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv, kv_valid=None, want_stats=False,
              mask=(0, 0), qshift=None):
     """Device tensors in the device layouts.  Returns (o bits uint16 [B,Sq,H,D], stats or None)."""

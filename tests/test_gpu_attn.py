@@ -555,27 +555,8 @@ def test_workload2_full_size(oracle):
 
 
 def _device_inputs(w, seed):
-    """Inputs of a workload's statistics generated on the GPU (the full-size property tests do not
-    need the seeded host generator, and the largest workload would take minutes on the host)."""
-    import torch
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    shape = (w.B, w.S, w.H, w.D)
-    q = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
-    k = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32)
-    if w.k_offset_std > 0:
-        k += w.k_offset_std * torch.randn((w.B, 1, w.H, w.D), generator=g, device="cuda", dtype=torch.float32)
-    if w.k_outlier_frac > 0:
-        n = int(np.ceil(w.k_outlier_frac * w.D))
-        gain = torch.ones((w.B, 1, w.H, w.D), device="cuda")
-        for b in range(w.B):
-            for h in range(w.H):
-                idx = torch.randperm(w.D, generator=g, device="cuda")[:n]
-                gain[b, 0, h, idx] = w.k_outlier_gain
-        k *= gain
-    k = k.to(torch.bfloat16)
-    v = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
-    return q, k, v
+    from mojodiffusion_amd.workloads import device_inputs
+    return device_inputs(w, seed)
 
 
 def _one_shot_dev(q, k, v, w):

@@ -162,6 +162,28 @@ def test_quant_v_bit_exact(oracle, D, S):
     np.testing.assert_array_equal(H.untile_v(g1["vq"], 1), v8)
 
 
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("wid,S,mask", [(2, 1100, (0, 0)), (1, 520, (0, 0)), (4, 700, (130, 260))])
+def test_three_launch_stage_equals_the_separate_stages(wid, S, mask, variant):
+    """mi355_sage_quant_qkv_bf16 runs the quantizers the way the one-shot calls do (three launches with
+    shared roles); its outputs are those of the Q/K and V stage entry points, which the tests above
+    hold to the CPU checker, bit for bit."""
+    import gpu_harness as H
+    w = WORKLOADS[wid].scaled(B=2, H=3, S=S)
+    q, k, v = make_inputs(w)
+    blkq = 128 if variant == 0 else 32
+    got = H.quant_qkv(q, k, v, w.scale, variant, blkq, 64, mask=mask)
+    qk = H.quant_qk(q, k, w.scale, blkq, 64, True, mask=mask)
+    vv = H.quant_v(v, variant, mask=mask)
+    for name in ("q8", "k8"):
+        np.testing.assert_array_equal(got[name], qk[name], err_msg=name)
+    for name in ("qscale", "kscale", "kmean", "qmul", "kmul"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), qk[name].view(np.uint32), err_msg=name)
+    np.testing.assert_array_equal(got["vq"], vv["vq"])
+    if variant == 1:
+        np.testing.assert_array_equal(got["vscale"].view(np.uint32), vv["vscale"].view(np.uint32))
+
+
 def test_quant_full_size_properties():
     """Workload 2 at full size: size-independent properties of the device output
     (no CPU pass over 14 M elements per tensor needed)."""
