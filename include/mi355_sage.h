@@ -334,27 +334,29 @@ int mi355_sage_attn_fwd(
     void* O, const int64_t* o_strides, int64_t o_offset_elems,
     const void* qshift, void* stats, void* stream);
 
-/* Scheduling of the attention kernel (no counterpart in the reference; for tests and tuning).
- * One workgroup computes 256 query rows of one head against all keys; a shape whose row tiles
+/* Scheduling of the attention kernel (no counterpart in the reference).
+ * One workgroup computes 256 query rows of one head against all keys.  A shape whose row tiles
  * leave the last round of the 256 compute units at most half full (more than 256 tiles, 16 % or
- * more of the launch idle) is instead cut into equal shares of (row tile, key tile) steps for
- * exactly 256 workgroups, which hand unnormalised partial results to each other inside the launch.  The choice depends on the
- * shape only, so all entry points give the same bits for the same problem; outputs of the two
- * schedules differ by rounding (the probabilities of a row are rounded against a different
- * running maximum).  mode 0: by shape (default); -1: never split; n > 0 (multiple of 8, <= 1024):
- * always split over n workgroups.  Process-wide; affects workspace sizes (the hand-over slots are
- * part of mi355_sage_workspace_bytes), so set it before sizing workspaces.  mi355_sage_attn_fwd,
- * which takes no workspace, keeps its slots in a library-owned per-stream buffer (allocated on
- * the first such call of a stream, never while that stream is being captured). */
-int mi355_sage_set_attn_split(int mode);
-
-/* How long a workgroup of the split schedule polls for another workgroup's partial result before
- * it gives up and writes NaN into its rows (the launch never hangs; no counterpart in the
- * reference).  polls > 0: that many polls of about a microsecond (default 262144; the longest
- * wait that can legitimately occur is one row tile's worth of work, a few milliseconds); 0: back
- * to the default; polls < 0: test mode — no workgroup announces its result and every waiting one
- * gives up after -polls polls, which is how the give-up path is exercised without a hang. */
-int mi355_sage_set_attn_split_wait(int polls);
+ * more of the launch idle; fp16 variant, head dim up to 128) is instead cut into equal shares of
+ * (row tile, key tile) steps for exactly 256 workgroups, which hand unnormalised partial results to
+ * each other inside the launch.  The choice depends on the shape only, so all entry points give the
+ * same bits for the same problem; outputs of the two schedules differ by rounding (the probabilities
+ * of a row are rounded against a different running maximum).  The hand-over relies on workgroup ids
+ * being dealt round-robin to 8 XCDs of 32 compute units, so the schedule is used only on a device
+ * that reports exactly that (hipDeviceAttributeNumberOfXccs == 8, 256 compute units); on any other
+ * partitioning every shape takes one workgroup per row tile.  Its hand-over slots are part of
+ * mi355_sage_workspace_bytes for the shapes that qualify (whatever the device); mi355_sage_attn_fwd,
+ * which takes no workspace, keeps its slots in a library-owned per-stream buffer (allocated on the
+ * first such call of a stream, never while that stream is being captured).
+ *
+ * A workgroup that does not find a partial result it waits for (a bounded wait: the launch never
+ * hangs), or finds it written on another XCD, writes NaN into its rows AND counts a fault on the
+ * device.  mi355_sage_attn_split_faults returns the number of such workgroups on the current device
+ * since the last reset (0 in a healthy run; negative: a HIP error), and clears the count when
+ * `reset` is non-zero.  It copies one word from the device with the blocking HIP call: synchronise
+ * the streams whose launches are to be covered first.  No attention call checks the count itself,
+ * so none of them synchronises. */
+int mi355_sage_attn_split_faults(int reset);
 
 /* Backward.  Replaces flame_cudnn_sdpa_bwd_bf16 (serenitymojo/ops/cshim/cudnn_sdpa_bwd.cpp:325-347;
  * Mojo callers ops/attention_flash.mojo:345-433, :478-535, :538-607): identical parameter list up

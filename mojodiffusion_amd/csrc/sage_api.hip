@@ -1,6 +1,7 @@
 // sage_api.hip — the C ABI of libmi355_sage.so (declared in include/mi355_sage.h).
 // Host-side only: argument checks, workspace carving, kernel sequencing.
 #include "../../include/mi355_sage.h"
+#include "../../include/mi355_sage_test.h"
 #include "sage_internal.h"
 
 #include <cstdio>
@@ -98,8 +99,8 @@ Carve carve(int B, int H, int Nq, int Nkv, int D, int variant) {
     c.qshift = take(bh * nqp * sizeof(float));
     c.rowinv_q = take((size_t)B * Nq * sizeof(float));        // whole-row RMSNorm statistic per token (optional pre-op)
     c.rowinv_k = take((size_t)B * Nkv * sizeof(float));
-    // hand-over slots of the attention kernel's split scheduling (shapes that use it only)
-    c.split = take(attn_split_bytes(attn_split_workgroups(B, H, Nq, Nkv, D, variant), D));
+    // hand-over slots of the attention kernel's split scheduling, for the shapes that qualify
+    c.split = take(attn_split_bytes(attn_split_rule(B, H, Nq, Nkv, D, variant), D));
     c.total = off;
     return c;
 }
@@ -372,7 +373,13 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         a.amask = static_cast<const uint16_t*>(mask.add) + mask.add_off;
         a.amb = mask.add_strides[0]; a.amh = mask.add_strides[1]; a.amn = mask.add_strides[2];
     }
-    a.split = ws + c.split;
+    // (one decision for carving and launching; slots the caller's workspace was not sized for — a
+    // forced schedule of the test switch — come from the library's per-stream buffer)
+    a.split_wgs = attn_split_workgroups(B, H, N_q, kv, D, variant);
+    if (a.split_wgs > 0) {
+        if (attn_split_bytes(a.split_wgs, D) <= attn_split_bytes(attn_split_rule(B, H, N_q, kv, D, variant), D)) a.split = ws + c.split;
+        else if ((rc = internal_workspace(g_split_ws, attn_split_bytes(a.split_wgs, D), st, &a.split))) return rc;
+    }
     SAGE_HIP(launch_attn(a, st));
     return MI355_SAGE_OK;
 }
@@ -705,10 +712,19 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     a.stats = static_cast<float*>(stats);
     // Same scheduling, hence the same bits, as the one-shot calls: shapes that are split over a
     // fixed number of workgroups need hand-over slots, kept per (device, stream) by the library.
-    const size_t split_bytes = attn_split_bytes(attn_split_workgroups(B, H, N_q, kv_valid, D, variant), D);
+    a.split_wgs = attn_split_workgroups(B, H, N_q, kv_valid, D, variant);
+    const size_t split_bytes = attn_split_bytes(a.split_wgs, D);
     if (split_bytes > 0 && (rc = internal_workspace(g_split_ws, split_bytes, static_cast<hipStream_t>(stream), &a.split))) return rc;
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
+}
+
+int mi355_sage_attn_split_faults(int reset) { return attn_split_faults(reset); }
+
+// (declared in include/mi355_sage_test.h: switches for the library's own tests)
+int mi355_sage_attn_split_rule(int B, int H, int N_q, int N_kv, int D, int variant) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0) return 0;
+    return attn_split_rule(B, H, N_q, N_kv, D, variant);
 }
 
 int mi355_sage_set_attn_split(int mode) {

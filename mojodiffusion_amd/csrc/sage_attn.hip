@@ -149,6 +149,9 @@ template <int VARIANT> struct Lazy {
 // for every tile's maximum on the biased scores (no optimistic tiles) and lets its ordinary
 // global loads share the vector-memory counter with the tile copies, i.e. it waits for all of
 // them at the midpoint: it is bound by the N_q x N_kv bias it has to read, not by the copies.
+// Workgroups of the split schedule that gave up on a hand-over (see the kernel's fold-in part).
+static __device__ unsigned int g_split_faults;
+
 template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT>
 #ifndef SAGE_NW
 #define SAGE_NW 8
@@ -829,7 +832,10 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
                 __builtin_amdgcn_s_sleep(16);
             }
             asm volatile("" ::: "memory");
-            if (flag != 1 + my_xcd) poison = __builtin_nanf("");
+            if (flag != 1 + my_xcd) {
+                poison = __builtin_nanf("");
+                if (tid == 0) atomicAdd(&g_split_faults, 1u);       // what mi355_sage_attn_split_faults reports
+            }
             const float* part = split_part + (int64_t)pb * PART_FLOATS;
             auto peer = [&](int idx) { return __hip_atomic_load(part + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
             const float m_p = peer(DB * 16 * THREADS + lane_off), l_p = peer(DB * 16 * THREADS + THREADS + lane_off);
@@ -914,7 +920,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     const int n_qtiles = (int)(a.nq_pad / (kThreads / 2));
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    const int split = attn_split_workgroups(a.B, a.H, a.Nq, a.kv_valid, D, VARIANT);
+    const int split = (D <= 128 && VARIANT == 0) ? a.split_wgs : 0;
     int* flags = nullptr;
     float* part = nullptr;
     if (split > 0) {
@@ -962,22 +968,25 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
 // each way.  Twice as many workgroups (two per compute unit, one after the other) were slower
 // everywhere but at 1584 items.  The decision depends on the shape only, so every entry point
 // produces the same bits for the same problem.
-static std::atomic<int> g_split_mode{0};       // 0: by shape; -1: never; n > 0: always, over n workgroups
+static std::atomic<int> g_split_mode{0};       // 0: by shape and device; -1: never; n > 0: always, over n workgroups
 
 void attn_split_override(int mode) { g_split_mode.store(mode); }
 
-int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D, int variant) {
+static bool split_fits(int B, int H, int Nq, int kv_valid, int D, int variant) {
+    if (D > 128) return false;                 // four-wave workgroups: one per item
+    if (variant != 0) return false;            // the e4m3 loop has no registers left for the hand-over
+    const int64_t items = pad_to(Nq, kTileQ) / kTileQ * B * H;
+    const int64_t ntiles = (kv_valid + kTileKV - 1) / kTileKV;
+    return (items / 8 + 1) * ntiles * kSplitMaxWorkgroups < (int64_t)1 << 31;       // 32-bit step arithmetic in the kernel
+}
+
+int attn_split_rule(int B, int H, int Nq, int kv_valid, int D, int variant) {
 #ifdef SAGE_CLOCK_PROBE
     return 0;                                  // the measurement build reports per-item clocks
 #else
-    if (D > 128) return 0;                     // four-wave workgroups: one per item
-    if (variant != 0) return 0;                // the e4m3 loop has no registers left for the hand-over
+    if (!split_fits(B, H, Nq, kv_valid, D, variant)) return 0;
     const int64_t items = pad_to(Nq, kTileQ) / kTileQ * B * H;
     const int64_t ntiles = (kv_valid + kTileKV - 1) / kTileKV;
-    const int mode = g_split_mode.load();
-    if (mode < 0) return 0;
-    if ((items / 8 + 1) * ntiles * kSplitMaxWorkgroups >= (int64_t)1 << 31) return 0;    // 32-bit step arithmetic in the kernel
-    if (mode > 0) return mode;
     constexpr int64_t kUnits = 256;
     if (items <= kUnits) return 0;
     const int64_t rounds = (items + kUnits - 1) / kUnits;
@@ -987,6 +996,47 @@ int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D, int variant
     if (items * ntiles < kUnits * 16) return 0;                // spans too short to be worth the hand-over
     return (int)kUnits;
 #endif
+}
+
+// The hand-over goes through one XCD's L2 and relies on workgroup ids being dealt round-robin to 8
+// XCDs of 32 compute units: asked of the device once, and the schedule stays off anywhere else.
+static bool split_topology_ok() {
+    static std::atomic<int> known[64];         // 0: not asked yet, 1: yes, 2: no
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    int k = known[dev].load();
+    if (k == 0) {
+        int xccs = 0, cus = 0;
+        const bool ok = hipDeviceGetAttribute(&xccs, hipDeviceAttributeNumberOfXccs, dev) == hipSuccess &&
+                        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+                        xccs == 8 && cus == 256;
+        k = ok ? 1 : 2;
+        known[dev].store(k);
+    }
+    return k == 1;
+}
+
+int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D, int variant) {
+#ifdef SAGE_CLOCK_PROBE
+    return 0;
+#else
+    const int mode = g_split_mode.load();
+    if (mode < 0) return 0;
+    if (mode > 0) return split_fits(B, H, Nq, kv_valid, D, variant) ? mode : 0;    // (tests force it whatever the device)
+    const int n = attn_split_rule(B, H, Nq, kv_valid, D, variant);
+    return n > 0 && split_topology_ok() ? n : 0;
+#endif
+}
+
+int attn_split_faults(int reset) {
+    unsigned n = 0;
+    hipError_t e = hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_split_faults), sizeof(n));
+    if (e == hipSuccess && reset) {
+        const unsigned zero = 0;
+        e = hipMemcpyToSymbol(HIP_SYMBOL(g_split_faults), &zero, sizeof(zero));
+    }
+    if (e != hipSuccess) return -(int)e;
+    return n > 0x7FFFFFFFu ? 0x7FFFFFFF : (int)n;
 }
 
 size_t attn_split_bytes(int workgroups, int D) {

@@ -114,18 +114,24 @@ struct AttnArgs {
     float* stats;            // [B,H,Nq] or null
     const uint16_t* amask;   // additive bias, bf16, base + offset; null = none
     int64_t amb, amh, amn;   // its element strides for batch, head, query (key stride 1)
-    void* split;             // attn_split_bytes(attn_split_workgroups(...), D) bytes, 256-byte aligned (null when 0)
+    int split_wgs;           // workgroups of the split schedule (attn_split_workgroups), 0: one workgroup per item
+    void* split;             // attn_split_bytes(split_wgs, D) bytes, 256-byte aligned (null when 0)
 };
 hipError_t launch_attn(const AttnArgs& a, hipStream_t st);
 // Shapes whose items do not fill whole rounds of workgroups are spread evenly over a fixed number
-// of workgroups that hand partial results to each other through `split`.  Number of workgroups
-// (a multiple of 8), or 0 for one workgroup per item; depends on the shape only.
+// of workgroups that hand partial results to each other through `split`.
+// attn_split_rule: the number of workgroups (a multiple of 8) the shape alone asks for, or 0 for one
+// workgroup per item — what workspaces are sized by.
+// attn_split_workgroups: what a launch on the current device uses: the rule where the device deals
+// workgroup ids round-robin to 8 XCDs of 32 compute units (else 0), or what the test switch forces.
+int attn_split_rule(int B, int H, int Nq, int kv_valid, int D, int variant);
 int attn_split_workgroups(int B, int H, int Nq, int kv_valid, int D, int variant);
 size_t attn_split_bytes(int workgroups, int D);
 constexpr size_t kSplitFlagBytes = 4096;     // one int per workgroup in front of the state slots
 constexpr int kSplitMaxWorkgroups = 1024;
-void attn_split_override(int mode);          // 0: by shape (default); -1: never; n > 0 (multiple of 8): always n
+void attn_split_override(int mode);          // 0: by shape and device (default); -1: never; n > 0 (multiple of 8): always n
 void attn_split_wait(int polls);             // bound of the hand-over wait; 0: default; < 0: test mode (no flag is raised)
+int attn_split_faults(int reset);            // workgroups that gave up on the current device since the last reset; < 0: -hipError_t
 
 // ---- backward (sage_bwd.hip) -------------------------------------------------
 // bf16 flash backward: Q, K, V, O, dO and the forward's log-sum-exp in, dQ, dK, dV out.

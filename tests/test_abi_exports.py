@@ -10,8 +10,8 @@ from mojodiffusion_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_functions():
-    text = open(os.path.join(ROOT, "include", "mi355_sage.h")).read()
+def _declared_functions(header="mi355_sage.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mi355_sage_\w+)\s*\(", text)))
 
@@ -19,10 +19,12 @@ def _declared_functions():
 def test_every_declared_symbol_is_exported_and_bound():
     names = _declared_functions()
     assert len(names) >= 12
+    test_names = _declared_functions("mi355_sage_test.h")         # the library's own test switches
+    assert test_names and not set(test_names) & set(names)
     L = ctypes.CDLL(_lib.LIB_PATH)
-    for n in names:
+    for n in names + test_names:
         assert hasattr(L, n), "library does not export %s" % n
-    assert sorted(_lib.SIGNATURES) == names        # the Python binding covers the whole header
+    assert sorted(_lib.SIGNATURES) == sorted(names + test_names)  # the Python binding covers both headers
 
 
 def test_no_gpu_helpers():
@@ -41,31 +43,30 @@ def test_no_gpu_helpers():
 
 def test_split_schedule_is_a_function_of_the_shape():
     """Hand-over slots (256 workgroups x (D/32*16 + 2) x 512 floats + 4 KiB of flags) are part of the
-    workspace exactly for the shapes that split: more than 256 row tiles, last round of 256 at most
-    half full, 16 % or more of the launch idle, spans of 16 steps or more."""
+    workspace exactly for the shapes that split: fp16 variant, more than 256 row tiles, last round of
+    256 at most half full, 16 % or more of the launch idle, spans of 16 steps or more.  The size is a
+    function of the shape alone: the test switch that forces a schedule does not move it."""
     L = _lib.lib()
+    rule = lambda B, H, S, D, variant=0: L.mi355_sage_attn_split_rule(B, H, S, S, D, variant)
+    assert rule(1, 33, 2048, 64) == 256          # 264 tiles: 1.03 rounds
+    assert rule(1, 19, 4352, 128) == 256         # 323 tiles
+    assert rule(1, 32, 4608, 128) == 256         # 576 tiles: 2.25 rounds
+    assert rule(1, 24, 4608, 128) == 0           # 432 tiles: last round 69 % full
+    assert rule(2, 30, 4352, 128) == 0           # 1020 tiles: 3.98 rounds
+    assert rule(1, 24, 16896, 128) == 0          # 1584 tiles: idle share 12 %
+    assert rule(1, 32, 1536, 128) == 0           # 192 tiles: fewer than compute units
+    assert rule(1, 8, 1024, 64) == 0
+    assert rule(1, 32, 4608, 128, 1) == 0        # the e4m3 variant keeps one workgroup per row tile
+    assert rule(1, 32, 4608, 256) == 0           # so do 256 channels
     slots = lambda D: 4096 + 256 * ((D // 32) * 16 + 2) * 512 * 4
-
-    def extra(B, H, S, D):
-        assert L.mi355_sage_set_attn_split(0) == 0
-        with_split = L.mi355_sage_workspace_bytes(B, H, S, S, D, 0)
-        assert L.mi355_sage_set_attn_split(-1) == 0
-        try:
-            return with_split - L.mi355_sage_workspace_bytes(B, H, S, S, D, 0)
-        finally:
-            L.mi355_sage_set_attn_split(0)
-    assert extra(1, 33, 2048, 64) == slots(64)          # 264 tiles: 1.03 rounds
-    assert extra(1, 19, 4352, 128) == slots(128)        # 323 tiles
-    assert extra(1, 32, 4608, 128) == slots(128)        # 576 tiles: 2.25 rounds
-    assert extra(1, 24, 4608, 128) == 0                 # 432 tiles: last round 69 % full
-    assert extra(2, 30, 4352, 128) == 0                 # 1020 tiles: 3.98 rounds
-    assert extra(1, 24, 16896, 128) == 0                # 1584 tiles: idle share 12 %
-    assert extra(1, 32, 1536, 128) == 0                 # 192 tiles: fewer than compute units
-    assert extra(1, 8, 1024, 64) == 0
-    # forced modes
+    # same tensors, one shape that splits and one that does not: the difference is the slots
+    # (items and key tiles decide; 2 x 16 heads of 4608 rows are 576 row tiles like 1 x 32 heads)
+    assert L.mi355_sage_workspace_bytes(1, 32, 4608, 4608, 128, 0) - L.mi355_sage_workspace_bytes(1, 32, 4608, 4608, 128, 1) \
+        == slots(128) + (L.mi355_sage_workspace_bytes(1, 24, 4608, 4608, 128, 0) - L.mi355_sage_workspace_bytes(1, 24, 4608, 4608, 128, 1)) * 32 // 24
+    before = L.mi355_sage_workspace_bytes(1, 2, 512, 512, 64, 0)
     assert L.mi355_sage_set_attn_split(64) == 0
     try:
-        assert L.mi355_sage_workspace_bytes(1, 2, 512, 512, 64, 0) > 64 * 34 * 512 * 4
+        assert L.mi355_sage_workspace_bytes(1, 2, 512, 512, 64, 0) == before
     finally:
         L.mi355_sage_set_attn_split(0)
     for bad in (-2, 12, 1032):

@@ -36,9 +36,9 @@ def _close_to_plain(got_bits, plain_bits):
     assert (got_bits == plain_bits).mean() > 0.5          # most values round to the same bf16 anyway
 
 
-@pytest.mark.parametrize("wid,variant,S,groups", [(2, 0, 1100, 24), (2, 0, 1100, 64), (2, 0, 1100, 8), (2, 1, 1100, 24),
-                                                  (4, 1, 700, 64), (3, 0, 333, 1024), (1, 0, 1024, 40), (1, 1, 520, 16),
-                                                  (2, 0, 50, 16), (1, 1, 64, 24), (2, 0, 2000, 8), (1, 0, 2000, 200)])
+@pytest.mark.parametrize("wid,variant,S,groups", [(2, 0, 1100, 24), (2, 0, 1100, 64), (2, 0, 1100, 8), (2, 0, 700, 64),
+                                                  (3, 0, 333, 1024), (1, 0, 1024, 40), (1, 0, 520, 16),
+                                                  (2, 0, 50, 16), (1, 0, 64, 24), (2, 0, 2000, 8), (1, 0, 2000, 200)])
 def test_forced_split_against_checker_and_plain_schedule(oracle, split, wid, variant, S, groups):
     import gpu_harness as H
     from test_gpu_attn import _one_shot
@@ -129,8 +129,9 @@ def test_split_call_in_a_hip_graph(split):
     import torch
     import gpu_harness as H
     L = _lib.lib()
-    split(24)
-    w = WORKLOADS[2].scaled(B=1, H=3, S=1100)
+    split(0)
+    w = WORKLOADS[1].scaled(B=1, H=33, S=2048)             # 264 row tiles: splits by itself, slots in the caller's workspace
+    assert L.mi355_sage_attn_split_rule(w.B, w.H, w.S, w.S, w.D, 0) == 256
     q0, k0, v0 = (H.dev_bf16(x) for x in make_inputs(w))
     q, k, v = q0.clone(), k0.clone(), v0.clone()
     o = torch.empty_like(q)
@@ -165,6 +166,18 @@ def test_split_call_in_a_hip_graph(split):
         np.testing.assert_array_equal(H.to_bits(o), H.to_bits(eager))
 
 
+def test_the_e4m3_variant_keeps_one_workgroup_per_row_tile(split):
+    """Its loop has no registers to spare for the hand-over: a forced split leaves its schedule, hence
+    its bits, alone."""
+    from test_gpu_attn import _one_shot
+    w = WORKLOADS[4].scaled(B=2, H=3, S=700)
+    q, k, v = make_inputs(w)
+    split(-1)
+    plain = _one_shot(q, k, v, w.scale, 1)
+    split(64)
+    np.testing.assert_array_equal(_one_shot(q, k, v, w.scale, 1), plain)
+
+
 def test_split_mode_argument():
     L = _lib.lib()
     for bad in (-2, 12, 1032):
@@ -184,7 +197,9 @@ def test_a_partial_result_that_never_arrives_poisons_rows_and_nothing_hangs(spli
     w = WORKLOADS[2].scaled(B=2, H=3, S=1100)               # 30 items of 18 steps; 24 workgroups: spans of 24 steps
     q, k, v = make_inputs(w)
     split(24)
+    assert L.mi355_sage_attn_split_faults(1) >= 0           # (clears the device's count)
     good = bf16_bits_to_f32(_one_shot(q, k, v, w.scale, 0))
+    assert L.mi355_sage_attn_split_faults(0) == 0           # a healthy run counts nothing
     assert L.mi355_sage_set_attn_split_wait(-64) == 0
     try:
         bad = bf16_bits_to_f32(_one_shot(q, k, v, w.scale, 0))
@@ -192,10 +207,15 @@ def test_a_partial_result_that_never_arrives_poisons_rows_and_nothing_hangs(spli
         assert L.mi355_sage_set_attn_split_wait(0) == 0
     nan_rows = np.isnan(bad).any(axis=-1)                   # [B,S,H]
     assert nan_rows.any() and not nan_rows.all()
+    # the device kept count of the workgroups that gave up: one per poisoned row tile of a head
+    tiles = {(b, h, s // 256) for b, s, h in zip(*np.nonzero(nan_rows))}
+    assert L.mi355_sage_attn_split_faults(0) == len(tiles)
+    assert L.mi355_sage_attn_split_faults(1) == len(tiles) and L.mi355_sage_attn_split_faults(0) == 0
     # poisoned rows come as whole row tiles of a head; everything else is bit-identical
     np.testing.assert_array_equal(bad[~nan_rows], good[~nan_rows])
     assert np.isnan(bad[nan_rows]).all()
     again = bf16_bits_to_f32(_one_shot(q, k, v, w.scale, 0))
     np.testing.assert_array_equal(again, good)
+    assert L.mi355_sage_attn_split_faults(0) == 0
     for bad_arg in (-(1 << 25), 1 << 25):
         assert L.mi355_sage_set_attn_split_wait(bad_arg) == -1
