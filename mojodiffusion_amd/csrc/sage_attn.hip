@@ -94,39 +94,34 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 // |dot| < 2292099 (the largest possible |dot| is 128*127*127 = 2064512) changes only the
 // mantissa: a finished accumulator, read as fp32, IS the float 1/(2*pi) + dot * 2^-26.  No
 // int->float conversion is needed and dequantisation, max subtraction and the exponent
-// argument collapse into one FMA per score (the scale carries the factor 2^26).  This
-// particular constant is one the matrix instruction takes as an inline operand, so it costs
-// neither registers nor moves.
+// argument collapse into one FMA per score (the scale carries the factor 2^26).
 constexpr int kMagicI = 0x3E22F983;
 constexpr float kMagicF = 0.15915494309189532f;        // the same 32 bits
 constexpr float kMagicUnit = 67108864.0f;               // 2^26: accumulator-as-float steps per integer
 // With 256 channels |dot| can reach 256*127*127 = 4129024, more than the mantissa of 1/(2*pi) has
 // room for below it.  0.1875 = 2^-3 * (1 + 2^22 * 2^-23) leaves 2^22 = 4194304 either way at the
-// same step of 2^-26; it is no inline operand, so that instantiation keeps it in registers.
+// same step of 2^-26.
 constexpr int kMagicWideI = 0x3E400000;
 constexpr float kMagicWideF = 0.1875f;
+// e4m3 variant: a wave whose bias * f can exceed this takes the bias off its accumulators (see exact_bias).
+constexpr float kExactBias = 4096.0f;
 template <int D> struct Magic {
     static constexpr int I = D > 128 ? kMagicWideI : kMagicI;
     static constexpr float F = D > 128 ? kMagicWideF : kMagicF;
 };
 
-// First matrix instruction of a score chain: accumulator input = the inline constant above.
-// (The compiler keeps a splat constant in 16 registers and copies them into the accumulator
-// for every chain; the instruction itself can take this constant as an immediate.)  The
-// following instructions of the chain are compiler-visible builtins that accumulate in place,
-// so everything that reads the finished scores is ordered against a matrix instruction the
-// compiler knows about.
+// First matrix instruction of a score chain: accumulator input = the constant above, held in 16
+// registers for the whole kernel (behind an empty statement, or the compiler re-creates the 16
+// copies for every chain).  The instruction could take 1/(2*pi) as an inline operand, but only
+// written as assembly, and then the compiler does not know that a matrix instruction is writing
+// those registers: it neither keeps the wait states before the first other instruction that
+// touches them — a spill store two instructions later wrote the old contents — nor can it be told.
 template <int D>
-__device__ __forceinline__ v16i mfma_i8_from_magic(const v4i& a, const v4i& b) {
-    if constexpr (D > 128) {
-        constexpr int M = kMagicWideI;
-        const v16i c = {M, M, M, M, M, M, M, M, M, M, M, M, M, M, M, M};
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-    } else {
-        v16i d;
-        asm("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0.15915494" : "=&v"(d) : "v"(a), "v"(b));
-        return d;
-    }
+__device__ __forceinline__ v16i magic_splat() {
+    constexpr int M = Magic<D>::I;
+    v16i c = {M, M, M, M, M, M, M, M, M, M, M, M, M, M, M, M};
+    asm volatile("" : "+v"(c));
+    return c;
 }
 
 // A row's reference maximum is only refreshed (and the accumulators rescaled) when a tile
@@ -408,6 +403,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
     // packed probabilities of two steps (by parity of the step).
     v4i fr[NM][FPU];
     v16i s[2][SKB];
+    const v16i smagic = magic_splat<D>();
     uint32_t p[2][PWS];
 
     // Operands of slot m of a step whose score instructions read key block `kbq` (fp16 variant; the
@@ -427,7 +423,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
     };
     auto qk_step = [&](int sb, int n, const v4i& a) {
         const int st = SKB == 1 ? n : n >> 1, kb = SKB == 1 ? 0 : n & 1;
-        s[sb][kb] = st == 0 ? mfma_i8_from_magic<D>(a, qf[0]) : __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[st], s[sb][kb], 0, 0, 0);
+        s[sb][kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, qf[st], st == 0 ? smagic : s[sb][kb], 0, 0, 0);
     };
     auto pv_unit = [&](int pb, int u, const v4i (&a)[FPU]) {
         const int jj = u / DB, d = u % DB;
@@ -455,6 +451,19 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
     }
     dma_wait<LEAD*(K_CH + V_CH)>();
     __syncthreads();
+    // The exponent argument is score * f + c0 with c0 = -(bias * f + reference): the constant carries
+    // the accumulators' bias times f, and its rounding (half an ulp at that magnitude) shifts every
+    // exponent argument of a key block by the same small amount.  An e4m3 probability next to a
+    // rounding boundary then lands on the other side of it.  On the workloads' statistics the shift
+    // is ~1e-5 and harmless; a wave whose largest bias * f (its rows' Q scale times the largest K
+    // scale) would bring it to 1e-4 takes the bias off its accumulators first, in every step (exact:
+    // both are multiples of 2^-26 below 2^-2), and its constant is the reference alone.
+    bool exact_bias = false;
+    if constexpr (VARIANT == 1 && !ADDMASK) {
+        float ks_max = 0.0f;
+        for (int i = lane; i < (int)(nkv_pad / 32); i += 64) ks_max = fmaxf(ks_max, lds_ks[KS_OFF + i]);
+        exact_bias = __any(Magic<D>::F * sq * ks_max > kExactBias);
+    }
     {
         v4i k0[NQ];
 #pragma unroll
@@ -531,7 +540,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
         if constexpr (ADDMASK) {
 #pragma unroll
             for (int kb = 0; kb < SKB; kb++) {
-                const float base = -(Magic<D>::F * f[kb]);
+                // (the bias of the accumulators is taken off before the multiplication: exact, where
+                // folding it into the multiply-add's constant would cost the constant's rounding)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const int key = key0 + kb * 32 + g * 8 + half * 4;
@@ -548,7 +558,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
                                          __uint_as_float(w1 << 16), __uint_as_float(w1 & 0xFFFF0000u)};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float sdq = fmaf(__int_as_float(s[X][kb][g * 4 + e]), f[kb], base);
+                        const float sdq = (__int_as_float(s[X][kb][g * 4 + e]) - Magic<D>::F) * f[kb];
                         xs[kb][g * 4 + e] = fmaf(mv[e], 1.4426950408889634f, sdq);
                     }
                 }
@@ -589,7 +599,22 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
         };
         if (!OPT) decide(Lazy<VARIANT>::tau);
 #pragma unroll
-        for (int kb = 0; kb < SKB; kb++) c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
+        for (int kb = 0; kb < SKB; kb++) {
+            c0[kb] = Lazy<VARIANT>::log2_pscale - fmaf(Magic<D>::F, f[kb], m_used);
+        }
+        // (e4m3 variant, score scales beyond anything the workloads show: see `exact_bias`; such a wave
+        // takes none of its steps through the main loop)
+        if constexpr (VARIANT == 1 && !ADDMASK && !TRIP) {
+            if (__builtin_expect(exact_bias, 0)) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int kb = 0; kb < SKB; kb++) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) s[X][kb][i] = __float_as_int(__int_as_float(s[X][kb][i]) - Magic<D>::F);
+                    c0[kb] = Lazy<VARIANT>::log2_pscale - m_used;
+                }
+            }
+        }
         const float l_before = l_run;
 
         // The softmax of the step as NV single vector operations, so that they can be dealt out over
@@ -725,6 +750,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
         // range) without looking for masked keys; the steps after that go through the loop below.
         int clean = (kv_valid - t_off * kTileKV) / SK;
         if (mask_hi > mask_lo && t_off * kTileKV < mask_hi) clean = min(clean, max(mask_lo - t_off * kTileKV, 0) / SK);
+        if (exact_bias) clean = 0;
         // (... and in front of the last tiles, so that the copies a trip starts need no clamping)
         const int trip_end = min(last_step - SPT * (KOFF + LEAD) + (SPT - 1), clean);
         for (; hs + PERIOD <= trip_end; hs += PERIOD) {

@@ -187,15 +187,12 @@ def test_reference_maximum_keeps_rising(oracle, variant):
     maximum (refresh + accumulator rescale, redo of an optimistic tile) is exercised, in
     interior tiles, repeatedly.  The second case puts one huge key in the middle.
 
-    Nearly every row here is dominated by one or two keys.  The fp16 variant stays inside the
-    2e-2 bar everywhere.  For the e4m3 variant kernel and checker follow the same rule (whole-
-    number reference, normaliser over the rounded probabilities), but they evaluate exp2 with
-    different last bits, so a probability within ~1e-4 (relative) of an e4m3 rounding boundary
-    is rounded the other way by one of them: one weight moves by one e4m3 step (2^-3 .. 2^-4
-    relative), which in a row carried by two keys a and b shows as up to 2^-4 |v_a - v_b|.  (The
-    scores here are ~25 times larger than on real inputs and the last bits of the exponent
-    argument scale with them, so such flips are ~100 times more frequent than usual.)  The
-    test therefore holds 99 % of the elements to the 2e-2 bar and all of them to that bound."""
+    Nearly every row here is dominated by one or two keys, and the scores are ~25 times larger
+    than on real inputs.  Both variants stay inside the 2e-2 bar on every element: for the e4m3
+    variant kernel and checker follow the same rule (whole-number reference, normaliser over the
+    rounded probabilities), and with scores this large the kernel forms its exponent arguments
+    without the rounding of a large constant, so that a probability next to an e4m3 rounding
+    boundary is rounded the way the checker rounds it."""
     import gpu_harness as H
     w = WORKLOADS[2].scaled(B=1, H=2, S=1024, k_offset_std=0.0)
     q, k, v = make_inputs(w)
@@ -210,14 +207,36 @@ def test_reference_maximum_keeps_rising(oracle, variant):
         _, want32 = oracle.sdpa_bf16(q, kk, v, w.scale, variant=variant, blkq=128, blkk=64, smooth_k=False)
         cos, mx = H.cos_maxabs(bf16_bits_to_f32(got), want32)
         assert cos >= 0.9999, (cos, mx)
-        if variant == 0:
-            assert mx <= MAX_ABS, (cos, mx)
-        else:
-            diff = np.abs(bf16_bits_to_f32(got).astype(np.float64) - want32)
-            vf = bf16_bits_to_f32(v)
-            assert np.quantile(diff, 0.99) <= MAX_ABS, np.quantile(diff, 0.99)
-            assert mx <= 2.0 ** -4 * (vf.max() - vf.min()), (mx, vf.max() - vf.min())
+        assert mx <= MAX_ABS, (cos, mx)
         assert np.isfinite(bf16_bits_to_f32(got)).all()
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_result_does_not_depend_on_what_ran_before(oracle, variant):
+    """Short sequences with an odd and an even number of 64-key tiles (they end in different code of the
+    kernel), each computed three times with other work on the device in between that leaves
+    different bit patterns in registers, LDS and the library's workspace: the results are the same
+    bits every time, and inside the bar against the checker.  (A matrix instruction whose result
+    the next instructions did not wait for is the kind of mistake that passes every parity test
+    in a fresh process, where the stale contents happen to be the right ones.)"""
+    import torch
+    import gpu_harness as H
+    other = torch.empty(1 << 24, dtype=torch.uint8, device="cuda")
+    for S in (192, 256, 320, 448):
+        w = WORKLOADS[2].scaled(B=2, H=2, S=S)
+        q, k, v = make_inputs(w)
+        first = _one_shot(q, k, v, w.scale, variant, w.blkq, w.blkk)
+        _, want32 = oracle.sdpa_bf16(q, k, v, w.scale, variant=variant, blkq=w.blkq, blkk=w.blkk)
+        cos, mx = H.cos_maxabs(bf16_bits_to_f32(first), want32)
+        assert mx <= MAX_ABS and cos >= 0.9999, (S, cos, mx)
+        for fill in (0xFF, 0x3C):
+            other.fill_(fill)
+            big = WORKLOADS[2].scaled(B=1, H=2, S=1024)
+            _one_shot(*make_inputs(big), big.scale, 1 - variant)
+            other.fill_(fill ^ 0x55)
+            torch.cuda.synchronize()
+            again = _one_shot(q, k, v, w.scale, variant, w.blkq, w.blkk)
+            assert np.array_equal(first, again), (S, fill)
 
 
 def test_train_fwd_stats_and_padmask(oracle):
