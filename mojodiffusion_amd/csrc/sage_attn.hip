@@ -148,10 +148,7 @@ template <int VARIANT> struct Lazy {
 static __device__ unsigned int g_split_faults;
 
 template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT>
-#ifndef SAGE_NW
-#define SAGE_NW 8
-#endif
-__global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel(
+__global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
@@ -169,7 +166,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
     constexpr int V_BYTES = D * kTileKV * VB;           // V^T tile
     // 256 channels: the output accumulators alone take 128 registers per lane, so a wave gets a SIMD
     // to itself (up to 512 registers) and a workgroup is 4 waves = 128 query rows.
-    constexpr int NW = D > 128 ? 4 : SAGE_NW;                 // waves per workgroup
+    constexpr int NW = D > 128 ? 4 : 8;                 // waves per workgroup
     constexpr int THREADS = NW * 64;
     constexpr int ROWS_WG = NW * 32;                    // query rows per workgroup
     constexpr int K_NCH = K_BYTES / 1024, V_NCH = V_BYTES / 1024;      // 1 KiB copies per tile
@@ -377,19 +374,13 @@ __global__ __launch_bounds__(D > 128 ? 256 : SAGE_NW * 64) void sage_attn_kernel
     constexpr int NP = 8 * SKB;                         // pairs of scores per lane and step
     constexpr int NV = NP * OPP;                        // vector operations of a step's softmax
     constexpr int PWS = PW / SPT;                       // dwords of packed P per step
-#ifndef SAGE_PDS
-#define SAGE_PDS 2
-#endif
-#ifndef SAGE_GRP
-#define SAGE_GRP 3
-#endif
-    constexpr int PDS = SAGE_PDS < NM / 2 ? SAGE_PDS : NM / 2;      // operand fragments are requested this many slots ahead
+    constexpr int PDS = 2;      // operand fragments are requested this many slots ahead
     constexpr int KOFF = SPT == 1 ? 2 : 1;              // the barrier of tile t publishes K(t + KOFF) and V(t)
     constexpr int PERIOD = 4 * SPT;                     // steps after which ring slots and parity repeat
     // GRP == 3: the operands of three slots are requested together, three to five slots ahead and in
     // reverse order, so that the first of the three matrix instructions waits for the request made
     // last — LDS answers in order — and the other two need no wait instruction at all.
-    constexpr int GRP = VARIANT == 0 ? SAGE_GRP : 1;
+    constexpr int GRP = VARIANT == 0 ? 3 : 1;
     constexpr int PF = GRP > 1 ? GRP : PDS;             // slots whose operands a step finds requested on entry
     static_assert(NM % 3 == 0 && NM / 3 == KSTEPS && PDS <= NM / 2 && (GRP == 1 || GRP == 3), "slot pattern");
     auto slot_is_qk = [](int m) { return VARIANT == 0 ? m % 3 == 1 : m % 3 != 2; };
@@ -942,7 +933,7 @@ __global__ void split_clear_kernel(int* flags, int n) {
 
 template <int D, int VARIANT>
 static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
-    constexpr int kThreads = D > 128 ? 256 : SAGE_NW * 64;             // 32 query rows per wave
+    constexpr int kThreads = D > 128 ? 256 : 512;             // 32 query rows per wave
     const int n_qtiles = (int)(a.nq_pad / (kThreads / 2));
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;

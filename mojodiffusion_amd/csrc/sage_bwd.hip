@@ -231,7 +231,6 @@ __device__ __forceinline__ void bwd_pass_body(const BwdArgs& a, PassLds<D, PASS>
 
     const int Nx = PASS == 0 ? a.Nq : a.Nkv;
     const int valid_x = PASS == 0 ? a.valid_q : a.valid_kv;
-    const int Ny = PASS == 0 ? a.Nkv : a.Nq;
     const int valid_y = PASS == 0 ? a.valid_kv : a.valid_q;
     const int x_tiles = (Nx + XROWS - 1) / XROWS;
     const int xt = block % x_tiles;
@@ -241,7 +240,9 @@ __device__ __forceinline__ void bwd_pass_body(const BwdArgs& a, PassLds<D, PASS>
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
     const int x = xt * XROWS + wave * 32 + l32;
-    const int xc = min(x, Nx - 1);
+    // (rows past the valid length are never read: what the caller keeps there — NaNs included — must
+    // not reach a valid row's gradient through a product with a zero probability)
+    const int xc = min(x, max(valid_x, 1) - 1);
 
     // owner side: two resident row blocks (B operands: column = owner row, k = head channel)
     const View& xv1 = PASS == 0 ? a.q : a.k;
@@ -303,7 +304,7 @@ __device__ __forceinline__ void bwd_pass_body(const BwdArgs& a, PassLds<D, PASS>
     auto copy_tile = [&](int t, int stage) {
 #pragma unroll
         for (int i = 0; i < RPW; i++) {
-            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], Ny - 1);
+            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], valid_y - 1);      // padding repeats the last valid row
             const uint32_t dst = (uint32_t)((i * NW + wave) * 1024);
             dma16(y1, row * ys1 + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 0) * TILE_BYTES + dst));
             dma16(y2, row * ys2 + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 1) * TILE_BYTES + dst));
@@ -527,7 +528,7 @@ __device__ __forceinline__ void dkdv_role(const BwdArgs& a, DkDvLds<D>& L, int b
     const int pair = wave & 3;
     const int l32 = lane & 31, half = lane >> 5;
     const int x = xt * 128 + pair * 32 + l32;
-    const int xc = min(x, a.Nkv - 1);
+    const int xc = min(x, max(a.valid_kv, 1) - 1);
 
     // owner side: the P wave keeps K rows, the S wave V rows (B operands: column = key, k = head channel)
     const View& xv = ROLE == 0 ? a.k : a.v;
@@ -566,7 +567,7 @@ __device__ __forceinline__ void dkdv_role(const BwdArgs& a, DkDvLds<D>& L, int b
     auto copy_for_p = [&](int t, int stage) {
 #pragma unroll
         for (int i = 0; i < RPW; i++) {
-            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], a.Nq - 1);
+            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], a.valid_q - 1);
             const uint32_t dst = (uint32_t)((i * NW + wave) * 1024);
             dma16(yq, row * sq + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 0) * TILE_BYTES + dst));
             dma16(tg + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * 2 + 1) * TILE_BYTES + dst));
@@ -577,7 +578,7 @@ __device__ __forceinline__ void dkdv_role(const BwdArgs& a, DkDvLds<D>& L, int b
     auto copy_for_s = [&](int t, int stage) {
 #pragma unroll
         for (int i = 0; i < RPW; i++) {
-            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], a.Nq - 1);
+            const uint32_t row = (uint32_t)min(t * 64 + nat_row[i], a.valid_q - 1);
             const uint32_t dst = (uint32_t)((i * NW + wave) * 1024);
             dma16(yg, row * sg + nat_col[i], __builtin_amdgcn_readfirstlane(nat_base + (stage * 2 + 1) * TILE_BYTES + dst));
             dma16(tq + (int64_t)t * TILE_BYTES, tr_src[i], __builtin_amdgcn_readfirstlane(tr_base + (stage * 2 + 0) * TILE_BYTES + dst));

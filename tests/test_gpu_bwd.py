@@ -40,7 +40,7 @@ def _check(name, got, want, abs_frac=1e-2, cos_bar=0.9999):
     assert _cos(got, want) >= cos_bar, "%s: cosine %.6f" % (name, _cos(got, want))
 
 
-def _run_case(oracle, B, Sq, Skv, H, D, scale, seed, real_q=0, real_kv=0, spread=1.0):
+def _run_case(oracle, B, Sq, Skv, H, D, scale, seed, real_q=0, real_kv=0, spread=1.0, nan_padding=False):
     rng = np.random.default_rng(seed)
     q, k, v, g = (_bf16_round(rng.standard_normal(s) * spread) for s in
                   ((B, Sq, H, D), (B, Skv, H, D), (B, Skv, H, D), (B, Sq, H, D)))
@@ -50,6 +50,14 @@ def _run_case(oracle, B, Sq, Skv, H, D, scale, seed, real_q=0, real_kv=0, spread
     o = _bf16_round(o32)
     want = oracle.sdpa_bwd_f32(qf, kf, vf, gf, scale, o=o.float().numpy(), stats=stats, real_nq=real_q, real_nkv=real_kv)
     L = _lib.lib()
+    if nan_padding:            # what the caller keeps in the rows past the valid lengths is none of the call's business
+        nq = real_q if 0 < real_q < Sq else Sq
+        for t in (q, o, g):
+            t[:, nq:] = float("nan")
+        for t in (k, v):
+            t[:, nk:] = float("nan")
+        stats = stats.copy()
+        stats.reshape(B, H, Sq)[:, :, nq:] = np.nan
     dev = [t.cuda() for t in (q, k, v, o, g)]
     st = torch.from_numpy(stats).cuda()
     outs = [torch.full_like(dev[0], 7.0), torch.full_like(dev[1], 7.0), torch.full_like(dev[2], 7.0)]
@@ -91,6 +99,23 @@ def test_bwd_valid_lengths(oracle):
         _check(name, got, ref)
     assert not outs[0][:, rq:].float().abs().max().item()
     assert not outs[1][:, rk:].float().abs().max().item() and not outs[2][:, rk:].float().abs().max().item()
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_bwd_ignores_what_the_padding_rows_hold(oracle, D):
+    """NaNs in every row past real_N_q / real_N_kv of Q, K, V, O, dO and Stats: the gradients are
+    the same bits as with finite padding, and the padding rows of the gradients are zeros.  (The
+    reference's padding mask, cudnn_sdpa_bwd.cpp:344-363, makes cuDNN ignore those rows' contents.)"""
+    B, Sq, Skv, H = 1, 256, 320, 2
+    rq, rk = 201, 167
+    clean, _ = _run_case(oracle, B, Sq, Skv, H, D, 0.09, seed=9, real_q=rq, real_kv=rk)
+    dirty, want = _run_case(oracle, B, Sq, Skv, H, D, 0.09, seed=9, real_q=rq, real_kv=rk, nan_padding=True)
+    for name, a, b, ref in zip(("dQ", "dK", "dV"), clean, dirty, want):
+        assert torch.isfinite(b.float()).all(), name
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)), name
+        _check(name, b, ref)
+    assert not dirty[0][:, rq:].float().abs().max().item()
+    assert not dirty[1][:, rk:].float().abs().max().item() and not dirty[2][:, rk:].float().abs().max().item()
 
 
 def test_bwd_golden_shapes(oracle):
