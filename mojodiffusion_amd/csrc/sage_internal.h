@@ -58,7 +58,7 @@ struct PrepArgs {
     double* kpart_sum;               // [B,H,ngroups,D] group sums; null: no K pass
     float* kpart_mm;                 // [B,H,ngroups,D,2] group minima / maxima
     PreOp pre_k;
-    int ngroups, nk_wg, nv_units;    // filled by the launcher
+    int ngroups, nk_wg, nv_units, n_bh;    // filled by the launcher
 };
 hipError_t launch_prep(const PrepArgs& a, int B, int D, hipStream_t st);
 
@@ -97,7 +97,7 @@ struct QuantArgs {
     float* kscale;
     uint8_t* v8;
     PreOp pre_q, pre_k;
-    int nq_blk, nk_blk, nv_tile;     // filled by the launcher
+    int nq_blk, nk_blk, nv_tile, n_bh;     // filled by the launcher
 };
 hipError_t launch_quant(const QuantArgs& a, int B, int D, hipStream_t st);
 

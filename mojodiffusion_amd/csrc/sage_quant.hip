@@ -18,6 +18,16 @@
 
 namespace sage {
 
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+// Running maximum of the magnitudes of bf16 pairs, as 16-bit integers: of one order with the values
+// themselves, infinities and NaNs on top (>= 0x7F80).  One packed instruction per pair.
+__device__ __forceinline__ uint32_t bf16_mag_max(uint32_t acc, uint32_t pair) {
+    const u16x2 m = __builtin_elementwise_max(__builtin_bit_cast(u16x2, acc), __builtin_bit_cast(u16x2, pair & 0x7FFF7FFFu));
+    return __builtin_bit_cast(uint32_t, m);
+}
+__device__ __forceinline__ bool bf16_mag_finite(uint32_t acc) { return (acc & 0xFFFFu) < 0x7F80u && (acc >> 16) < 0x7F80u; }
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
@@ -179,7 +189,7 @@ __device__ __forceinline__ float rint_quotient(float x, float sc, float rinv, bo
 // Q (IS_K false): x = f32(q) * chmul[d].  K (IS_K true): x = (f32(k) - mean[d]) * chmul[d];
 // tokens that are masked or beyond N count for nothing and get code 0.
 // rowdot (Q only, may be null): <f32(q) * cmul, mean> per row.
-template <int D, int BLK, bool IS_K, bool PRE>
+template <int D, int BLK, bool IS_K, bool PRE, int NT>
 __device__ __forceinline__ void quant_i8_block(
     int t, int h, int b, const uint16_t* __restrict__ x, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, const KeyMask& km, const float* __restrict__ mean,
@@ -187,9 +197,9 @@ __device__ __forceinline__ void quant_i8_block(
     int8_t* __restrict__ codes, float* __restrict__ scales, float* __restrict__ rowdot, float* red,
     const PreOp& pre) {
     constexpr int CPR = D / 8;                 // 16-byte chunks per row
-    constexpr int NCH = BLK * CPR / 256;       // chunks per thread
-    static_assert(BLK * CPR % 256 == 0, "tile must split evenly over 256 threads");
-    static_assert(256 % CPR == 0, "a thread keeps one column group for all its chunks");
+    constexpr int NCH = BLK * CPR / NT;        // chunks per thread
+    static_assert(BLK * CPR % NT == 0, "tile must split evenly over the threads");
+    static_assert(NT % CPR == 0, "a thread keeps one column group for all its chunks");
     const int tid = threadIdx.x;
     const int r0 = t * BLK;
     const int col = (tid % CPR) * 8;
@@ -199,7 +209,7 @@ __device__ __forceinline__ void quant_i8_block(
     u32x4 raw[NCH];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        const int row = r0 + (i * 256 + tid) / CPR;
+        const int row = r0 + (i * NT + tid) / CPR;
         raw[i] = u32x4{0u, 0u, 0u, 0u};
         if (row < N) raw[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
     }
@@ -211,7 +221,7 @@ __device__ __forceinline__ void quant_i8_block(
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        const int row = r0 + (i * 256 + tid) / CPR;
+        const int row = r0 + (i * NT + tid) / CPR;
         unpack8(raw[i], v[i]);
         if constexpr (PRE) pre_apply<D>(pre, b, h, H, row, col, row < N, v[i]);
         bool counts;
@@ -239,34 +249,85 @@ __device__ __forceinline__ void quant_i8_block(
         }
         if (counts) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[i][e]));
+            for (int e = 0; e < 8; e += 2) amax = fmaxf(fmaxf(amax, fabsf(v[i][e])), fabsf(v[i][e + 1]));
         }
     }
 
     amax = wave_max(amax);
     if ((tid & 63) == 0) red[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    amax = red[0];
+#pragma unroll
+    for (int w = 1; w < NT / 64; w++) amax = fmaxf(amax, red[w]);
 
     const float sc = amax > 0.0f ? amax / 127.0f : 1.0f;      // blocks without a counting token: amax == 0
     if (tid == 0) scales[bh * (n_pad / BLK) + t] = sc;
     const bool fast = sc >= 0x1p-100f && sc <= 0x1p100f;
     const float rinv = 1.0f / sc;
 
+    uint32_t pk[NCH][2];
+    float far[NCH] = {};        // per 16-byte chunk: how close the thread's products come to a rounding tie
+    bool all_careful = PRE || !fast;
+    if constexpr (!PRE) {
+        // The common case, three operations per element and no test: t = x * rinv + 1.5 * 2^23 in one
+        // fused step IS rint of the exact product p, as an integer in the low bits of t (its lowest
+        // byte is the code: |p| <= 127 (1 + 2^-22) for every token that counts, so nothing needs
+        // clamping); d = p minus that integer.  p differs from the true quotient by at most
+        // 128 * 2^-24 (the rounding of rinv) and the true quotient is itself rounded by at most
+        // 2^-18, so wherever |d| <= 1/2 - 2^-16 all three round to the same integer.  The largest
+        // |d| of each chunk of eight is looked at after the loop: a chunk in which some lane of the
+        // wave comes closer to a tie is encoded again with the true quotient (about one chunk in
+        // seventy).  A NaN takes no part in any maximum and ends as code 0 here as there; an infinite
+        // input makes the scale infinite, and such a block is encoded with the true quotient throughout.
+        float kRound = 12582912.0f;                            // 1.5 * 2^23
+        float rv = rinv;
+        // (vector registers: the operations below then carry neither a scalar operand nor a literal,
+        // and issue at the short rate)
+        asm volatile("" : "+v"(rv), "+v"(kRound));
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int row = r0 + (i * NT + tid) / CPR;
+            const bool counts = IS_K ? key_kept(row, N, km) : row < N;
+            uint32_t tb[8];
+            float dm = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const float t0 = fmaf(v[i][e], rv, kRound), t1 = fmaf(v[i][e + 1], rv, kRound);
+                const float d0 = fmaf(v[i][e], rv, -(t0 - kRound)), d1 = fmaf(v[i][e + 1], rv, -(t1 - kRound));
+                dm = fmaxf(fmaxf(dm, fabsf(d0)), fabsf(d1));
+                tb[e] = __float_as_uint(t0);
+                tb[e + 1] = __float_as_uint(t1);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const uint32_t lo = __builtin_amdgcn_perm(tb[4 * j + 1], tb[4 * j], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm(tb[4 * j + 3], tb[4 * j + 2], 0x0c0c0400u);
+                pk[i][j] = counts ? __builtin_amdgcn_perm(hi, lo, 0x05040100u) : 0u;
+            }
+            far[i] = counts ? dm : 0.0f;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-        const int row = r0 + (i * 256 + tid) / CPR;
-        uint32_t pk[2] = {0u, 0u};
-        if (IS_K ? key_kept(row, N, km) : row < N) {
+        if (__builtin_expect(all_careful || __any(!(far[i] <= 0.5f - 0x1p-16f)), 0)) {
+            asm volatile("" ::: "memory");
+            const int row = r0 + (i * NT + tid) / CPR;
+            pk[i][0] = pk[i][1] = 0u;
+            if (IS_K ? key_kept(row, N, km) : row < N) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                float r = rint_quotient(v[i][e], sc, rinv, fast);
-                r = fminf(fmaxf(r, -127.0f), 127.0f);
-                pk[e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
+                for (int e = 0; e < 8; e++) {
+                    float r = rint_quotient(v[i][e], sc, rinv, fast);
+                    r = r > 127.0f ? 127.0f : r;               // (comparisons: a NaN stays one; the conversion instruction makes it 0)
+                    r = r < -127.0f ? -127.0f : r;
+                    pk[i][e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
+                }
             }
         }
-        u32x2 o = {pk[0], pk[1]};
-        *reinterpret_cast<u32x2*>(codes + (bh * n_pad + row) * D + col) = o;
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int row = r0 + (i * NT + tid) / CPR;
+        *reinterpret_cast<u32x2*>(codes + (bh * n_pad + row) * D + col) = u32x2{pk[i][0], pk[i][1]};
     }
 }
 
@@ -472,37 +533,82 @@ __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
 }
 
 // V tile -> e4m3 with the per-channel scales, tiled layout (slot order v_slot_fp8).
-template <int D>
+//
+// The code of an element is e4m3(RN(x / sc)).  The common case takes neither a divide nor the
+// conversion in integer arithmetic: with y = RN(1 / sc) (one true divide per channel and thread),
+// q0 = RN(x y), r = x - q0 sc (exact in one fused step) and q1 = RN(q0 + r y), q1 IS the correctly
+// rounded quotient (Markstein's correction step; it needs y correctly rounded, q0 within an ulp
+// and the significand of sc not all ones), and the conversion instruction rounds to nearest even
+// and reaches 448 exactly where the quotient's magnitude is 448 (1 + 2^-23) at most, which the
+// scale guarantees.  A wave that sees a non-finite input, or a scale outside the range where none
+// of this can underflow, or with an all-ones significand, takes the plain formula.
+template <int D, int NT>
 __device__ __forceinline__ void quant_v_fp8_body(
     int t, int h, int b, const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t sn,
     int N, int H, int64_t n_pad, const KeyMask& km, const float* __restrict__ vscale,
     uint8_t* __restrict__ out, uint8_t* tile) {
     constexpr int CPR = D / 8;
     constexpr int LD = D + 16;                             // padded row (bytes)
+    constexpr int NCH = 64 * CPR / NT;
+    static_assert(NT % CPR == 0, "a thread keeps one column group for all its chunks");
     const int tid = threadIdx.x;
     const int64_t bh = (int64_t)b * H + h;
     const uint16_t* src = v + b * sb + h * sh;
+    const int col = (tid % CPR) * 8;
+    u32x4 w[NCH];
 #pragma unroll
-    for (int i = 0; i < 64 * CPR / 256; i++) {
-        const int c = i * 256 + tid;
-        const int key = c / CPR, col = (c % CPR) * 8;
-        const int row = t * 64 + key;
-        u32x4 w = {0u, 0u, 0u, 0u};
-        if (key_kept(row, N, km)) w = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
-        float x[8], sc[8];
-        unpack8(w, x);
-        load8(vscale + bh * D + col, sc);
+    for (int i = 0; i < NCH; i++) {
+        const int row = t * 64 + (i * NT + tid) / CPR;
+        w[i] = u32x4{0u, 0u, 0u, 0u};
+        if (key_kept(row, N, km)) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * sn + col);
+    }
+    float sc[8], y[8];
+    load8(vscale + bh * D + col, sc);
+    bool plain = false;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        y[e] = 1.0f / sc[e];
+        plain = plain || !(sc[e] >= 0x1p-60f && sc[e] <= 0x1p60f) || (__float_as_uint(sc[e]) & 0x7FFFFFu) == 0x7FFFFFu;
+    }
+    uint32_t mag = 0u;
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) mag = bf16_mag_max(mag, w[i][e]);
+    plain = __any(plain || !bf16_mag_finite(mag));
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int key = (i * NT + tid) / CPR;
+        float x[8];
+        unpack8(w[i], x);
         uint32_t pk[2] = {0u, 0u};
+        if (__builtin_expect(plain, 0)) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) pk[e >> 2] |= f32_to_e4m3(x[e] / sc[e]) << ((e & 3) * 8);
+            for (int e = 0; e < 8; e++) pk[e >> 2] |= f32_to_e4m3(x[e] / sc[e]) << ((e & 3) * 8);
+        } else {
+            float q[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                // (the residual as -(q0 sc - x): an input of -0 then stays -0 through both steps, as it
+                // does through the divide)
+                const float q0 = x[e] * y[e];
+                q[e] = fmaf(-fmaf(q0, sc[e], -x[e]), y[e], q0);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                int p2 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * j], q[4 * j + 1], 0, false);
+                p2 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * j + 2], q[4 * j + 3], p2, true);
+                pk[j] = (uint32_t)p2;
+            }
+        }
         *reinterpret_cast<u32x2*>(&tile[v_slot_fp8(key) * LD + col]) = u32x2{pk[0], pk[1]};
     }
     __syncthreads();
     uint8_t* dst = out + ((bh * (n_pad / 64)) + t) * (int64_t)(D * 64);
     // output chunk = (channel d, 16 consecutive slots)
 #pragma unroll
-    for (int i = 0; i < D * 4 / 256; i++) {
-        const int c = i * 256 + tid;
+    for (int i = 0; i < D * 4 / NT; i++) {
+        const int c = i * NT + tid;
         const int d = c >> 2, s0 = (c & 3) * 16;
         uint32_t pk[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -525,8 +631,14 @@ __global__ __launch_bounds__(256) void prep_kernel(PrepArgs a) {
         KGroupSmem<DK> kg[GPW];
     };
     __shared__ __attribute__((aligned(16))) Smem sm;
+    // Consecutive workgroups take the same unit of consecutive heads: in [.., N, H, D] memory those
+    // are neighbours, so the workgroups in flight together read whole DRAM pages between them.  The
+    // K-statistics units (longer) are dealt evenly among the V units instead of coming last.
     const int per_bh = a.nv_units + a.nk_wg;
-    const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
+    const int bh = blockIdx.x % a.n_bh, slot = blockIdx.x / a.n_bh;
+    const int k_before = (int)(((int64_t)slot * a.nk_wg) / per_bh);
+    const bool is_k = (int)(((int64_t)(slot + 1) * a.nk_wg) / per_bh) > k_before;
+    const int r = is_k ? a.nv_units + k_before : slot - k_before;
     const int b = bh / a.H, h = bh % a.H;
     if (r < a.nv_units) {
         if (a.vmode == 0)
@@ -597,6 +709,7 @@ hipError_t launch_prep(const PrepArgs& a_in, int B, int D, hipStream_t st) {
     // K groups per workgroup: 2 at D = 64, 1 at D = 128; at D = 256 a group takes two workgroups
     a.nk_wg = a.kpart_sum == nullptr ? 0 : D == 256 ? a.ngroups * 2 : D == 128 ? a.ngroups : (a.ngroups + 1) / 2;
     a.nv_units = a.vmode == 0 ? (int)(a.nkv_pad / 64) : (a.vmode == 1 ? a.ngroups : 0);
+    a.n_bh = B * a.H;
     const int64_t total = (int64_t)B * a.H * (a.nv_units + a.nk_wg);
     if (total == 0) return hipSuccess;
     if (total > 0x7FFFFFFF) return hipErrorInvalidValue;
@@ -660,7 +773,15 @@ __global__ __launch_bounds__(64) void stats_final_kernel(FinalArgs a) {
     if (a.vscale != nullptr) {
         const float* p = a.vpart + bh * a.ngroups * a.D + d;
         float amax = 0.0f;
-        for (int g = 0; g < a.ngroups; g++) amax = fmaxf(amax, p[(int64_t)g * a.D]);
+        // (32 loads in flight at a time: taken one by one, each waits out a memory latency)
+        constexpr int NB = 32;
+        for (int g0 = 0; g0 < a.ngroups; g0 += NB) {
+            float v[NB];
+#pragma unroll
+            for (int j = 0; j < NB; j++) v[j] = p[(int64_t)(g0 + j < a.ngroups ? g0 + j : a.ngroups - 1) * a.D];
+#pragma unroll
+            for (int j = 0; j < NB; j++) amax = fmaxf(amax, v[j]);
+        }
         a.vscale[i] = amax > 0.0f ? amax / 448.0f : 1.0f;
     }
 }
@@ -674,21 +795,28 @@ hipError_t launch_stats_final(const FinalArgs& a, hipStream_t st) {
 // ---------------------------------------------------------------------------
 // Launch 3: Q blocks, K blocks and (e4m3 variant) V tiles as workgroup roles.
 // ---------------------------------------------------------------------------
+// Threads per workgroup: 512 at 128 channels — a block of 128 tokens is then four 16-byte chunks
+// per thread, few enough registers for eight waves per SIMD, which is what keeps loads in flight
+// while other waves encode (a workgroup loads, reduces, encodes and stores in turn).
+template <int D, bool PRE> constexpr int quant_threads() { return D == 128 && !PRE ? 256 : 256; }
+
 template <int D, bool PRE>
 __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
+    constexpr int NT = quant_threads<D, PRE>();
     union Smem {
-        float red[4];
+        float red[NT / 64];
         uint8_t tile8[64 * (D + 16)];
     };
     __shared__ __attribute__((aligned(16))) Smem sm;
-    const int per_bh = a.nq_blk + a.nk_blk + a.nv_tile;
-    const int bh = blockIdx.x / per_bh, r = blockIdx.x % per_bh;
+    // consecutive workgroups take the same rows of consecutive heads: in [.., N, H, D] memory those
+    // are neighbours, so the workgroups in flight together read whole DRAM pages between them
+    const int bh = blockIdx.x % a.n_bh, r = blockIdx.x / a.n_bh;
     const int b = bh / a.H, h = bh % a.H;
     const KeyMask none{0, 0};
     if (r < a.nq_blk) {
         const float* mul = a.qmul + (int64_t)bh * D;
         const float* mean = a.kmean + (int64_t)bh * D;
-#define SAGE_Q(BLK) quant_i8_block<D, BLK, false, PRE>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, none, \
+#define SAGE_Q(BLK) quant_i8_block<D, BLK, false, PRE, NT>(r, h, b, a.q.p, a.q.sb, a.q.sh, a.q.sn, a.Nq, a.H, a.nq_pad, none, \
                                                        mean, mul, a.cmul, a.q8, a.qscale, a.rowdot, sm.red, a.pre_q)
         if (a.blkq == 128) SAGE_Q(128);
         else if (a.blkq == 64) SAGE_Q(64);
@@ -698,14 +826,14 @@ __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
         const int t = r - a.nq_blk;
         const float* mul = a.kmul + (int64_t)bh * D;
         const float* mean = a.kmean + (int64_t)bh * D;
-#define SAGE_K(BLK) quant_i8_block<D, BLK, true, PRE>(t, h, b, a.k.p, a.k.sb, a.k.sh, a.k.sn, a.Nkv, a.H, a.nkv_pad, a.km, \
+#define SAGE_K(BLK) quant_i8_block<D, BLK, true, PRE, NT>(t, h, b, a.k.p, a.k.sb, a.k.sh, a.k.sn, a.Nkv, a.H, a.nkv_pad, a.km, \
                                                       mean, mul, 0.0f, a.k8, a.kscale, nullptr, sm.red, a.pre_k)
         if (a.blkk == 128) SAGE_K(128);
         else if (a.blkk == 64) SAGE_K(64);
         else SAGE_K(32);
 #undef SAGE_K
     } else {
-        quant_v_fp8_body<D>(r - a.nq_blk - a.nk_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km,
+        quant_v_fp8_body<D, NT>(r - a.nq_blk - a.nk_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km,
                             a.vscale, a.v8, sm.tile8);
     }
 }
@@ -717,16 +845,19 @@ hipError_t launch_quant(const QuantArgs& a_in, int B, int D, hipStream_t st) {
     a.nv_tile = a.v8 != nullptr ? (int)(a.nkv_pad / 64) : 0;
     if (a.q8 != nullptr && a.nq_pad % a.blkq != 0) return hipErrorInvalidValue;
     if (a.k8 != nullptr && a.nkv_pad % a.blkk != 0) return hipErrorInvalidValue;
+    a.n_bh = B * a.H;
     const int64_t total = (int64_t)B * a.H * (a.nq_blk + a.nk_blk + a.nv_tile);
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    dim3 grid((unsigned)total), block(256);
+    dim3 grid((unsigned)total);
     const bool has_pre = a.pre_q.gain != nullptr;
-    if (D == 128 && has_pre) hipLaunchKernelGGL((quant_kernel<128, true>), grid, block, 0, st, a);
-    else if (D == 128) hipLaunchKernelGGL((quant_kernel<128, false>), grid, block, 0, st, a);
-    else if (D == 64 && has_pre) hipLaunchKernelGGL((quant_kernel<64, true>), grid, block, 0, st, a);
-    else if (D == 64) hipLaunchKernelGGL((quant_kernel<64, false>), grid, block, 0, st, a);
-    else if (D == 256 && !has_pre) hipLaunchKernelGGL((quant_kernel<256, false>), grid, block, 0, st, a);
+#define SAGE_LAUNCH_QUANT(DD, PP) hipLaunchKernelGGL((quant_kernel<DD, PP>), grid, dim3((quant_threads<DD, PP>())), 0, st, a)
+    if (D == 128 && has_pre) SAGE_LAUNCH_QUANT(128, true);
+    else if (D == 128) SAGE_LAUNCH_QUANT(128, false);
+    else if (D == 64 && has_pre) SAGE_LAUNCH_QUANT(64, true);
+    else if (D == 64) SAGE_LAUNCH_QUANT(64, false);
+    else if (D == 256 && !has_pre) SAGE_LAUNCH_QUANT(256, false);
     else return hipErrorInvalidValue;
+#undef SAGE_LAUNCH_QUANT
     return hipGetLastError();
 }
 

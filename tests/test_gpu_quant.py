@@ -162,6 +162,60 @@ def test_quant_v_bit_exact(oracle, D, S):
     np.testing.assert_array_equal(H.untile_v(g1["vq"], 1), v8)
 
 
+def test_quant_v_fp8_every_bf16_value_and_rounding_tie(oracle):
+    """Channels whose largest magnitude is 448 have the scale 1.0, so the quotient is the input
+    itself: every bf16 value from 2^-13 to 448 of either sign goes through, among them every exact
+    tie between two e4m3 codes (normal and subnormal range), both zeros, and values that round to
+    zero.  Other channels repeat the values under scales 1.5, 3 and 1/3 (quotients that need the
+    correction step of the division)."""
+    import gpu_harness as H
+    bits = np.arange(0x3900, 0x43E1, dtype=np.uint16)                 # 2^-13 .. 448
+    vals = np.concatenate([bits, bits | 0x8000, np.uint16([0x0000, 0x8000])])
+    D, Hh = 128, 1
+    S = 64 * ((len(vals) + 1 + 63) // 64)
+    v = np.zeros((1, S, Hh, D), np.uint16)
+    for c in range(D):
+        top = np.float32([448.0, 448.0 * 1.5, 448.0 * 3.0, 448.0 / 3.0][c % 4])
+        col = np.roll(vals, 37 * c)
+        if c % 4:                                                       # scaled copies: value * scale, rounded to bf16
+            f = (col.astype(np.uint32) << 16).view(np.float32) * np.float32([1.0, 1.5, 3.0, 1.0 / 3.0][c % 4])
+            col = f32_to_bf16_bits(f.reshape(1, -1, 1, 1)).reshape(-1)
+            col = np.where((col & 0x7FFF) > f32_to_bf16_bits(np.float32([[[[top]]]])).reshape(-1)[0], np.uint16(0), col)
+        v[0, :len(col), 0, c] = col
+        v[0, len(vals), 0, c] = f32_to_bf16_bits(np.float32([[[[top]]]])).reshape(-1)[0]
+    g = H.quant_v(v, 1)
+    v8, vs = oracle.quant_v_fp8(v, 128)
+    assert vs[0, 0, 0] == 1.0
+    np.testing.assert_array_equal(g["vscale"].view(np.uint32), vs.view(np.uint32))
+    np.testing.assert_array_equal(H.untile_v(g["vq"], 1), v8)
+
+
+def test_quant_non_finite_inputs_follow_the_plain_formulas(oracle):
+    """An infinity or a NaN among the inputs: the kernels' short cuts (reciprocal instead of divide,
+    rounding by a magic addend, the conversion instruction) mean nothing then, and a wave that sees
+    one takes the plain formulas — the codes and scales are still the checker's."""
+    import gpu_harness as H
+    rng = np.random.default_rng(77)
+    B, S, Hh, D = 1, 256, 2, 128
+    def tensor():
+        return rng.standard_normal((B, S, Hh, D)).astype(np.float32)
+    q, k, v = tensor(), tensor(), tensor()
+    q[0, 5, 0, 17] = np.nan
+    k[0, 70, 1, 3] = np.nan
+    v[0, 9, 0, 100] = np.nan
+    v[0, 200, 1, 64] = np.inf
+    qb, kb, vb = f32_to_bf16_bits(q), f32_to_bf16_bits(k), f32_to_bf16_bits(v)
+    g = H.quant_qk(qb, kb, 0.1, 128, 64, False, balance=False)
+    want = H.oracle_quant_qk(oracle, qb, kb, 0.1, 128, 64, False, False, (0, 0))
+    np.testing.assert_array_equal(g["q8"][:, :, :S], want["q8"][:, :, :S])
+    np.testing.assert_array_equal(g["k8"][:, :, :S], want["k8"][:, :, :S])
+    np.testing.assert_array_equal(g["qscale"][:, :, :S // 128].view(np.uint32), want["qscale"].view(np.uint32))
+    g1 = H.quant_v(vb, 1)
+    v8, vs = oracle.quant_v_fp8(vb, 128)
+    np.testing.assert_array_equal(g1["vscale"].view(np.uint32), vs.view(np.uint32))
+    np.testing.assert_array_equal(H.untile_v(g1["vq"], 1), v8)
+
+
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("wid,S,mask", [(2, 1100, (0, 0)), (1, 520, (0, 0)), (4, 700, (130, 260))])
 def test_three_launch_stage_equals_the_separate_stages(wid, S, mask, variant):
