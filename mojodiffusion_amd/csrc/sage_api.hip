@@ -335,8 +335,14 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         if ((rc = internal_workspace(g_ws, c.total, st, &p))) return rc;
         ws = static_cast<uint8_t*>(p);
     }
+    // (one decision for carving and launching; slots the caller's workspace was not sized for — a
+    // forced schedule of the test switch — come from the library's per-stream buffer)
+    const int split_wgs = attn_split_workgroups(B, H, N_q, kv, D, variant);
+    // The plain forward leaves Q to the attention kernel, which encodes its own rows (same codes and
+    // scales): the quantize stage then neither reads Q nor writes its codes.
+    const bool q_in_kernel = Stats == nullptr && mask.add == nullptr && pre.q.gain == nullptr && D <= 128 && split_wgs == 0;
     QuantOut o{};
-    o.q8 = reinterpret_cast<int8_t*>(ws + c.q8);
+    o.q8 = q_in_kernel ? nullptr : reinterpret_cast<int8_t*>(ws + c.q8);
     o.k8 = reinterpret_cast<int8_t*>(ws + c.k8);
     o.qscale = reinterpret_cast<float*>(ws + c.qscale);
     o.kscale = reinterpret_cast<float*>(ws + c.kscale);
@@ -373,9 +379,11 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
         a.amask = static_cast<const uint16_t*>(mask.add) + mask.add_off;
         a.amb = mask.add_strides[0]; a.amh = mask.add_strides[1]; a.amn = mask.add_strides[2];
     }
-    // (one decision for carving and launching; slots the caller's workspace was not sized for — a
-    // forced schedule of the test switch — come from the library's per-stream buffer)
-    a.split_wgs = attn_split_workgroups(B, H, N_q, kv, D, variant);
+    if (q_in_kernel) {
+        a.q_src = q.p; a.qsb = q.sb; a.qsh = q.sh; a.qsn = q.sn;
+        a.qmul = o.qmul;
+    }
+    a.split_wgs = split_wgs;
     if (a.split_wgs > 0) {
         if (attn_split_bytes(a.split_wgs, D) <= attn_split_bytes(attn_split_rule(B, H, N_q, kv, D, variant), D)) a.split = ws + c.split;
         else if ((rc = internal_workspace(g_split_ws, attn_split_bytes(a.split_wgs, D), st, &a.split))) return rc;

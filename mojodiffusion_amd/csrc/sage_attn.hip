@@ -51,6 +51,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 
 // Byte offset of 16-byte chunk L of a tile.  Chunks are grouped into 128-byte super-rows
@@ -147,9 +148,14 @@ template <int VARIANT> struct Lazy {
 // Workgroups of the split schedule that gave up on a hand-over (see the kernel's fold-in part).
 static __device__ unsigned int g_split_faults;
 
-template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT>
+// QF: the kernel takes Q as bf16 (q_src, strides; q8 / qscale unread) and encodes its own 32 rows per
+// wave in the prologue — the quantize stage's arithmetic (quant_i8_block), so the codes and scales
+// are the ones that stage would have written — which saves the stage a read of Q and a write and
+// this kernel's read of the codes.
+template <int D, int VARIANT, bool STATS, bool ADDMASK, bool SPLIT, bool QF = false>
 __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     const int8_t* __restrict__ q8, const float* __restrict__ qscale, int blkq,
+    const uint16_t* __restrict__ q_src, int64_t qsb, int64_t qsh, int64_t qsn, const float* __restrict__ qmul,
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
     const float* __restrict__ qshift,
@@ -191,6 +197,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     __shared__ __attribute__((aligned(1024))) uint8_t lds_k[NSK][K_BYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lds_v[NSV][V_BYTES];
     __shared__ __attribute__((aligned(16))) float lds_ks[max_keys(D) / 32 + 4];
+    __shared__ float lds_qmax[QF ? 8 : 1];              // QF: largest |pre-scaled q| of each wave's 32 rows
+    static_assert(!QF || (D <= 128 && !STATS && !ADDMASK && !SPLIT), "Q is encoded in the kernel only in the plain forward");
 
     // Work items are (q tile, b*h) pairs, `total_wg` of them; an item takes `ntiles` steps (key
     // tiles).  Hardware hands consecutive workgroup ids to the 8 XCDs round-robin; each XCD gets a
@@ -259,12 +267,96 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
 
     // Q^T fragments: 16 bytes of the head dim per step, resident for the whole kernel.
     v4i qf[KSTEPS];
-    {
+    float sq;
+    if constexpr (!QF) {
         const int8_t* qp = q8 + (bh * nq_pad + qrow) * D + half * 16;
 #pragma unroll
         for (int s = 0; s < KSTEPS; s++) qf[s] = *reinterpret_cast<const v4i*>(qp + s * 32);
+        sq = qscale[bh * (nq_pad / blkq) + qrow / blkq] * kMagicUnit;
+    } else {
+        // This lane's 16 channels of every 32 (its half of the row); rows past N_q are zeros.
+        u32x4 rw[KSTEPS][2];
+        {
+            const uint16_t* qp = q_src + b * qsb + h * qsh + (int64_t)qrow * qsn + half * 16;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    rw[s][j] = u32x4{0u, 0u, 0u, 0u};
+                    if (qrow < Nq) rw[s][j] = *reinterpret_cast<const u32x4*>(qp + s * 32 + j * 8);
+                }
+        }
+        float x[KSTEPS][16];
+        float am = 0.0f;
+        {
+            const float* mp = qmul + bh * D + half * 16;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const v4f m0 = *reinterpret_cast<const v4f*>(mp + s * 32 + j * 8), m1 = *reinterpret_cast<const v4f*>(mp + s * 32 + j * 8 + 4);
+                    const float m[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        x[s][j * 8 + 2 * e] = __uint_as_float(rw[s][j][e] << 16) * m[2 * e];
+                        x[s][j * 8 + 2 * e + 1] = __uint_as_float(rw[s][j][e] & 0xFFFF0000u) * m[2 * e + 1];
+                        am = fmaxf(fmaxf(am, fabsf(x[s][j * 8 + 2 * e])), fabsf(x[s][j * 8 + 2 * e + 1]));
+                    }
+                }
+        }
+        // the row's other half, then the wave's 32 rows, then the waves that share a scale block
+        {
+            const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(am), __float_as_uint(am), false, false);
+            am = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
+        }
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+        if (blkq > 32) {
+            if (lane == 0) lds_qmax[wave] = am;
+            __syncthreads();
+            const int nwv = blkq >> 5, w0 = wave & ~(nwv - 1);
+            am = lds_qmax[w0];
+            for (int w = 1; w < nwv; w++) am = fmaxf(am, lds_qmax[w0 + w]);
+        }
+        const float sc = am > 0.0f ? am / 127.0f : 1.0f;
+        const bool fast = sc >= 0x1p-100f && sc <= 0x1p100f;
+        const float rinv = 1.0f / sc;
+        float kRound = 12582912.0f, rv = rinv;             // (see quant_i8_block)
+        asm volatile("" : "+v"(rv), "+v"(kRound));
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++) {
+            uint32_t tb[16], wd[4];
+            float dm = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+                const float t0 = fmaf(x[s][e], rv, kRound), t1 = fmaf(x[s][e + 1], rv, kRound);
+                const float d0 = fmaf(x[s][e], rv, -(t0 - kRound)), d1 = fmaf(x[s][e + 1], rv, -(t1 - kRound));
+                dm = fmaxf(fmaxf(dm, fabsf(d0)), fabsf(d1));
+                tb[e] = __float_as_uint(t0);
+                tb[e + 1] = __float_as_uint(t1);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t lo = __builtin_amdgcn_perm(tb[4 * j + 1], tb[4 * j], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm(tb[4 * j + 3], tb[4 * j + 2], 0x0c0c0400u);
+                wd[j] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            }
+            if (__builtin_expect(!fast || __any(!(dm <= 0.5f - 0x1p-16f)), 0)) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int j = 0; j < 4; j++) wd[j] = 0u;
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    float r = rint_quotient(x[s][e], sc, rinv, fast);
+                    r = r > 127.0f ? 127.0f : r;
+                    r = r < -127.0f ? -127.0f : r;
+                    wd[e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
+                }
+            }
+            qf[s] = v4i{(int)wd[0], (int)wd[1], (int)wd[2], (int)wd[3]};
+        }
+        sq = sc * kMagicUnit;
     }
-    const float sq = qscale[bh * (nq_pad / blkq) + qrow / blkq] * kMagicUnit;
     // this lane's row of the additive bias (padding rows read the last real row; their output is dropped)
     const uint16_t* mrow = ADDMASK ? amask + b * amb + h * amh + (int64_t)min(qrow, Nq - 1) * amn : nullptr;
 
@@ -950,7 +1042,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     dim3 grid((unsigned)(split > 0 ? split : total)), block(kThreads);
 #define SAGE_LAUNCH_ATTN2(STATS, ADDMASK, SPLIT)                                                                         \
     hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK, SPLIT>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
-                       a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,          \
+                       a.q_src, a.qsb, a.qsh, a.qsn, a.qmul, a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,          \
                        a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,               \
                        (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags, g_split_wait.load())
 #define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                                  \
@@ -962,7 +1054,18 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
             SAGE_LAUNCH_ATTN2(STATS, ADDMASK, false);                     \
         }                                                                 \
     } while (0)
-    if (a.amask != nullptr) {
+    if (a.q_src != nullptr) {
+        // Q encoded by the kernel: the plain forward only
+        if constexpr (D <= 128) {
+            if (a.amask != nullptr || a.stats != nullptr || split > 0 || a.qmul == nullptr) return hipErrorInvalidValue;
+            hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, false, false, false, true>), grid, block, 0, st, nullptr, nullptr, a.blkq,
+                               a.q_src, a.qsb, a.qsh, a.qsn, a.qmul, a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, nullptr,
+                               a.H, a.Nq, a.kv_valid, a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, nullptr,
+                               n_qtiles, (int)total, nullptr, 0, 0, 0, 0, nullptr, nullptr, g_split_wait.load());
+        } else {
+            return hipErrorInvalidValue;
+        }
+    } else if (a.amask != nullptr) {
         if (a.stats != nullptr) SAGE_LAUNCH_ATTN(true, true);
         else SAGE_LAUNCH_ATTN(false, true);
     } else {

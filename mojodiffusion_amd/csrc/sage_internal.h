@@ -102,6 +102,18 @@ struct QuantArgs {
 hipError_t launch_quant(const QuantArgs& a, int B, int D, hipStream_t st);
 
 // ---- attention kernel (sage_attn.hip) --------------------------------------
+// rint(x / sc) for |x / sc| <= ~127 without paying a full IEEE divide per element: x * (1/sc)
+// is within 2^-15 of the correctly rounded quotient (both below 128), so whenever it lies at
+// least 2^-12 away from a rounding tie it rounds to the same integer; the few elements near
+// a tie (and any non-finite case) take the true divide.  `fast` is false when sc is so small
+// or large that 1/sc is not a normal number.
+__device__ __forceinline__ float rint_quotient(float x, float sc, float rinv, bool fast) {
+    const float q = x * rinv;
+    float n = rintf(q);
+    if (!fast || !(fabsf(q - n) <= 0.5f - 0x1p-12f)) n = rintf(x / sc);
+    return n;
+}
+
 struct AttnArgs {
     const int8_t* q8;  const float* qscale;  int blkq;
     const int8_t* k8;  const float* kscale;  int blkk;
@@ -114,6 +126,12 @@ struct AttnArgs {
     float* stats;            // [B,H,Nq] or null
     const uint16_t* amask;   // additive bias, bf16, base + offset; null = none
     int64_t amb, amh, amn;   // its element strides for batch, head, query (key stride 1)
+    // Q taken as bf16 and encoded by the attention kernel itself (q8 / qscale unused then): base + offset,
+    // element strides of batch, head and token, and the channel multipliers [B,H,D] of the quantize stage.
+    // Only without Stats, additive bias and split schedule, at up to 128 channels.
+    const uint16_t* q_src;   // null: q8 / qscale are read
+    int64_t qsb, qsh, qsn;
+    const float* qmul;
     int split_wgs;           // workgroups of the split schedule (attn_split_workgroups), 0: one workgroup per item
     void* split;             // attn_split_bytes(split_wgs, D) bytes, 256-byte aligned (null when 0)
 };

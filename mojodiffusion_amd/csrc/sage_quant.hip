@@ -174,18 +174,6 @@ __device__ __forceinline__ void pre_apply(const PreOp& p, int b, int h, int H, i
 // (b,h); the BLK x D tile lives in registers between the absmax pass and the encode pass, so
 // HBM sees one read of bf16 and one write of int8.
 // ---------------------------------------------------------------------------
-// rint(x / sc) for |x / sc| <= ~127 without paying a full IEEE divide per element: x * (1/sc)
-// is within 2^-15 of the correctly rounded quotient (both below 128), so whenever it lies at
-// least 2^-12 away from a rounding tie it rounds to the same integer; the few elements near
-// a tie (and any non-finite case) take the true divide.  `fast` is false when sc is so small
-// or large that 1/sc is not a normal number.
-__device__ __forceinline__ float rint_quotient(float x, float sc, float rinv, bool fast) {
-    const float q = x * rinv;
-    float n = rintf(q);
-    if (!fast || !(fabsf(q - n) <= 0.5f - 0x1p-12f)) n = rintf(x / sc);
-    return n;
-}
-
 // Q (IS_K false): x = f32(q) * chmul[d].  K (IS_K true): x = (f32(k) - mean[d]) * chmul[d];
 // tokens that are masked or beyond N count for nothing and get code 0.
 // rowdot (Q only, may be null): <f32(q) * cmul, mean> per row.
