@@ -273,9 +273,19 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
 #pragma unroll
         for (int s = 0; s < KSTEPS; s++) qf[s] = *reinterpret_cast<const v4i*>(qp + s * 32);
         sq = qscale[bh * (nq_pad / blkq) + qrow / blkq] * kMagicUnit;
-    } else {
-        // This lane's 16 channels of every 32 (its half of the row); rows past N_q are zeros.
-        u32x4 rw[KSTEPS][2];
+    }
+    // QF: this lane's 16 channels of every 32 (its half of the row), rows past N_q as zeros, and the
+    // channel multipliers that go with them
+    u32x4 rw[QF ? KSTEPS : 1][2];
+    v4f qm[QF ? KSTEPS : 1][4];
+    if constexpr (QF) {
+        {
+            const float* mp = qmul + bh * D + half * 16;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) qm[s][j] = *reinterpret_cast<const v4f*>(mp + s * 32 + j * 4);
+        }
         {
             const uint16_t* qp = q_src + b * qsb + h * qsh + (int64_t)qrow * qsn + half * 16;
 #pragma unroll
@@ -286,76 +296,8 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
                     if (qrow < Nq) rw[s][j] = *reinterpret_cast<const u32x4*>(qp + s * 32 + j * 8);
                 }
         }
-        float x[KSTEPS][16];
-        float am = 0.0f;
-        {
-            const float* mp = qmul + bh * D + half * 16;
-#pragma unroll
-            for (int s = 0; s < KSTEPS; s++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const v4f m0 = *reinterpret_cast<const v4f*>(mp + s * 32 + j * 8), m1 = *reinterpret_cast<const v4f*>(mp + s * 32 + j * 8 + 4);
-                    const float m[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        x[s][j * 8 + 2 * e] = __uint_as_float(rw[s][j][e] << 16) * m[2 * e];
-                        x[s][j * 8 + 2 * e + 1] = __uint_as_float(rw[s][j][e] & 0xFFFF0000u) * m[2 * e + 1];
-                        am = fmaxf(fmaxf(am, fabsf(x[s][j * 8 + 2 * e])), fabsf(x[s][j * 8 + 2 * e + 1]));
-                    }
-                }
-        }
-        // the row's other half, then the wave's 32 rows, then the waves that share a scale block
-        {
-            const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(am), __float_as_uint(am), false, false);
-            am = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
-        }
-#pragma unroll
-        for (int off = 1; off < 32; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
-        if (blkq > 32) {
-            if (lane == 0) lds_qmax[wave] = am;
-            __syncthreads();
-            const int nwv = blkq >> 5, w0 = wave & ~(nwv - 1);
-            am = lds_qmax[w0];
-            for (int w = 1; w < nwv; w++) am = fmaxf(am, lds_qmax[w0 + w]);
-        }
-        const float sc = am > 0.0f ? am / 127.0f : 1.0f;
-        const bool fast = sc >= 0x1p-100f && sc <= 0x1p100f;
-        const float rinv = 1.0f / sc;
-        float kRound = 12582912.0f, rv = rinv;             // (see quant_i8_block)
-        asm volatile("" : "+v"(rv), "+v"(kRound));
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            uint32_t tb[16], wd[4];
-            float dm = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-                const float t0 = fmaf(x[s][e], rv, kRound), t1 = fmaf(x[s][e + 1], rv, kRound);
-                const float d0 = fmaf(x[s][e], rv, -(t0 - kRound)), d1 = fmaf(x[s][e + 1], rv, -(t1 - kRound));
-                dm = fmaxf(fmaxf(dm, fabsf(d0)), fabsf(d1));
-                tb[e] = __float_as_uint(t0);
-                tb[e + 1] = __float_as_uint(t1);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint32_t lo = __builtin_amdgcn_perm(tb[4 * j + 1], tb[4 * j], 0x0c0c0400u);
-                const uint32_t hi = __builtin_amdgcn_perm(tb[4 * j + 3], tb[4 * j + 2], 0x0c0c0400u);
-                wd[j] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-            }
-            if (__builtin_expect(!fast || __any(!(dm <= 0.5f - 0x1p-16f)), 0)) {
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int j = 0; j < 4; j++) wd[j] = 0u;
-#pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    float r = rint_quotient(x[s][e], sc, rinv, fast);
-                    r = r > 127.0f ? 127.0f : r;
-                    r = r < -127.0f ? -127.0f : r;
-                    wd[e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
-                }
-            }
-            qf[s] = v4i{(int)wd[0], (int)wd[1], (int)wd[2], (int)wd[3]};
-        }
-        sq = sc * kMagicUnit;
+        // (the arithmetic follows further down, behind the first tile copies: their latency and this
+        // one's then run side by side)
     }
     // this lane's row of the additive bias (padding rows read the last real row; their output is dropped)
     const uint16_t* mrow = ADDMASK ? amask + b * amb + h * amh + (int64_t)min(qrow, Nq - 1) * amn : nullptr;
@@ -531,6 +473,78 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     for (int x = 0; x < LEAD; x++) {
         dma_k(min(x + KOFF, last), (x + KOFF) % NSK);
         dma_v(min(x, last), x % NSV);
+    }
+    if constexpr (QF) {
+        // ---- Q of this wave's 32 rows -> int8 codes and scale (quant_i8_block's arithmetic)
+        float x[KSTEPS][16];
+        float am = 0.0f;
+        {
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const v4f m0 = qm[s][2 * j], m1 = qm[s][2 * j + 1];
+                    const float m[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        x[s][j * 8 + 2 * e] = __uint_as_float(rw[s][j][e] << 16) * m[2 * e];
+                        x[s][j * 8 + 2 * e + 1] = __uint_as_float(rw[s][j][e] & 0xFFFF0000u) * m[2 * e + 1];
+                        am = fmaxf(fmaxf(am, fabsf(x[s][j * 8 + 2 * e])), fabsf(x[s][j * 8 + 2 * e + 1]));
+                    }
+                }
+        }
+        // the row's other half, then the wave's 32 rows, then the waves that share a scale block
+        {
+            const v2u r = __builtin_amdgcn_permlane32_swap(__float_as_uint(am), __float_as_uint(am), false, false);
+            am = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
+        }
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, 64));
+        if (blkq > 32) {
+            if (lane == 0) lds_qmax[wave] = am;
+            __syncthreads();
+            const int nwv = blkq >> 5, w0 = wave & ~(nwv - 1);
+            am = lds_qmax[w0];
+            for (int w = 1; w < nwv; w++) am = fmaxf(am, lds_qmax[w0 + w]);
+        }
+        const float sc = am > 0.0f ? am / 127.0f : 1.0f;
+        const bool fast = sc >= 0x1p-100f && sc <= 0x1p100f;
+        const float rinv = 1.0f / sc;
+        float kRound = 12582912.0f, rv = rinv;             // (see quant_i8_block)
+        asm volatile("" : "+v"(rv), "+v"(kRound));
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++) {
+            uint32_t tb[16], wd[4];
+            float dm = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+                const float t0 = fmaf(x[s][e], rv, kRound), t1 = fmaf(x[s][e + 1], rv, kRound);
+                const float d0 = fmaf(x[s][e], rv, -(t0 - kRound)), d1 = fmaf(x[s][e + 1], rv, -(t1 - kRound));
+                dm = fmaxf(fmaxf(dm, fabsf(d0)), fabsf(d1));
+                tb[e] = __float_as_uint(t0);
+                tb[e + 1] = __float_as_uint(t1);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t lo = __builtin_amdgcn_perm(tb[4 * j + 1], tb[4 * j], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm(tb[4 * j + 3], tb[4 * j + 2], 0x0c0c0400u);
+                wd[j] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            }
+            if (__builtin_expect(!fast || __any(!(dm <= 0.5f - 0x1p-16f)), 0)) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int j = 0; j < 4; j++) wd[j] = 0u;
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    float r = rint_quotient(x[s][e], sc, rinv, fast);
+                    r = r > 127.0f ? 127.0f : r;
+                    r = r < -127.0f ? -127.0f : r;
+                    wd[e >> 2] |= ((uint32_t)((int)r) & 0xFFu) << ((e & 3) * 8);
+                }
+            }
+            qf[s] = v4i{(int)wd[0], (int)wd[1], (int)wd[2], (int)wd[3]};
+        }
+        sq = sc * kMagicUnit;
     }
     dma_wait<LEAD*(K_CH + V_CH)>();
     __syncthreads();
