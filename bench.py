@@ -93,13 +93,13 @@ def summarize_traffic(dirs):
     import glob
 
     def avg(d, pattern):
-        f = glob.glob(os.path.join(d, "*counter_collection.csv"))
+        f = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
         vals = [float(r["Counter_Value"]) for r in csv.DictReader(open(f[0])) if pattern in r["Kernel_Name"]]
         # the copy kernel is the one whose value is largest (torch launches helpers too)
         return sum(vals) / len(vals), len(vals)
 
     def copy_avg(d):
-        f = glob.glob(os.path.join(d, "*counter_collection.csv"))
+        f = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
         by = {}
         for r in csv.DictReader(open(f[0])):
             by.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
@@ -115,7 +115,7 @@ def summarize_traffic(dirs):
     print("# HBM traffic of sage_attn_kernel per launch, rocprofv3 --pmc (one counter per run)")
     print("# Commands (repository root on the MI355X box, after `cd /tmp && export TMPDIR=/tmp` and back; OUT = any "
           "scratch directory), C = FETCH_SIZE, then WRITE_SIZE:")
-    print("#   rocprofv3 --pmc C --output-format csv -d OUT/pmc_C_bench -o p -- python3 bench.py --skip-cpu-baseline --steps 3 --warmup 2")
+    print("#   rocprofv3 --pmc C --output-format csv -d OUT/pmc_C_bench -o p -- python3 bench.py --skip-cpu-baseline --skip-other-workloads --steps 3 --warmup 2")
     print("#   rocprofv3 --pmc C --output-format csv -d OUT/pmc_C_copy -o p -- python3 bench.py --copy-calibration")
     print("#   python3 bench.py --summarize-traffic OUT/pmc_FETCH_SIZE_bench OUT/pmc_WRITE_SIZE_bench "
           "OUT/pmc_FETCH_SIZE_copy OUT/pmc_WRITE_SIZE_copy")
@@ -189,8 +189,11 @@ def clock_probe(args, L, w, qd, kd, vd, o, st, stream):
 
 def run_workload(L, torch, w, qd, kd, vd, steps, warmup, n_events):
     """One workload through the one-shot call (wall clock over back-to-back steps) and through the
-    stage entry points with HIP events on the launch stream: the quantize stage as the one-shot call
-    runs it (three launches, mi355_sage_quant_qkv_bf16) and the attention kernel."""
+    stage entry points with HIP events on the launch stream, each stage as the one-shot call runs it:
+    the quantize stage (three launches, mi355_sage_quant_qkv_bf16) and the attention kernel.  Where the
+    one-shot call leaves the Q encode to the attention kernel (every shape but those of the split
+    schedule), so do the stages timed here: mi355_sage_quant_qkv_bf16 without Q outputs and
+    mi355_sage_attn_fwd_q16."""
     from mojodiffusion_amd import _lib
     dev = qd.device
     B, S, H, D = w.B, w.S, w.H, w.D
@@ -235,16 +238,29 @@ def run_workload(L, torch, w, qd, kd, vd, steps, warmup, n_events):
     vq = torch.empty((B, H, nkp // 64, D, 64), dtype=torch.int16 if w.variant == 0 else torch.uint8, device=dev)
     scr = torch.empty(max(L.mi355_sage_quant_scratch_bytes(B, H, S, D), 8), dtype=torch.uint8, device=dev)
 
-    def stage_quant():
+    def stage_quant(with_q):
         return L.mi355_sage_quant_qkv_bf16(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), B, H, S, S, D, w.scale, st, st, st,
-                                           0, 0, 0, w.variant, w.blkq, w.blkk, K_FLAGS, 0, 0, q8.data_ptr(), qs.data_ptr(),
+                                           0, 0, 0, w.variant, w.blkq, w.blkk, K_FLAGS, 0, 0,
+                                           q8.data_ptr() if with_q else None, qs.data_ptr() if with_q else None,
                                            k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(), kmu.data_ptr(),
                                            vq.data_ptr(), vsc.data_ptr(), scr.data_ptr(), scr.numel(), stream)
 
-    def stage_attn():
+    def attn_q8():
         return L.mi355_sage_attn_fwd(q8.data_ptr(), qs.data_ptr(), w.blkq, k8.data_ptr(), ks.data_ptr(), w.blkk,
                                      vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, 0, 0, D,
                                      o.data_ptr(), st, 0, None, None, stream)
+
+    def attn_q16():
+        return L.mi355_sage_attn_fwd_q16(qd.data_ptr(), st, 0, qm.data_ptr(), w.blkq, k8.data_ptr(), ks.data_ptr(), w.blkk,
+                                         vq.data_ptr(), vsc.data_ptr(), w.variant, B, H, S, S, S, 0, 0, D,
+                                         o.data_ptr(), st, 0, stream)
+
+    assert stage_quant(True) == 0
+    rc = attn_q16()                       # -2: a shape of the split schedule, whose Q the quantize stage encodes
+    if rc not in (0, -2):
+        raise RuntimeError("mi355_sage_attn_fwd_q16 rc=%d" % rc)
+    q_in_kernel = rc == 0
+    stage_attn = attn_q16 if q_in_kernel else attn_q8
 
     def time_stage(fn, n):
         for _ in range(3):
@@ -259,10 +275,10 @@ def run_workload(L, torch, w, qd, kd, vd, steps, warmup, n_events):
         ts = sorted(a.elapsed_time(b) for a, b in evs)
         return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
 
-    qt_avg, qt_med, qt_min = time_stage(stage_quant, n_events)
+    qt_avg, qt_med, qt_min = time_stage(lambda: stage_quant(not q_in_kernel), n_events)
     at_avg, at_med, at_min = time_stage(stage_attn, n_events)
     return dict(step=step, ms_per_step=ms_per_step, ramp_steps=ramp_steps, quant=(qt_avg, qt_med, qt_min),
-                attn=(at_avg, at_med, at_min), keep=(o, ws, q8, k8, qs, ks, km, qm, kmu, vsc, vq, scr))
+                attn=(at_avg, at_med, at_min), q_in_kernel=q_in_kernel, keep=(o, ws, q8, k8, qs, ks, km, qm, kmu, vsc, vq, scr))
 
 
 def main():
@@ -361,9 +377,12 @@ def main():
     at_avg, at_med, at_min = r["attn"]
     attn_tops = w.ops / (at_avg * 1e-3) / 1e12
     peak = PEAK_INT8_TOPS if w.variant == 0 else PEAK_FP8_TOPS
-    # algorithmic HBM bytes of the quantize stage: Q,K,V read once as bf16; int8 Q/K and fp16/e4m3 V written
+    # algorithmic HBM bytes of the quantize stage: K and V (and Q, where this stage encodes it) read once
+    # as bf16; int8 K (and Q) and fp16 / e4m3 V written
     elems = B * H * S * D
-    quant_bytes = 3 * elems * 2 + 2 * elems + elems * (2 if w.variant == 0 else 1)
+    fused = r["q_in_kernel"]
+    vbytes = 2 if w.variant == 0 else 1
+    quant_bytes = (2 if fused else 3) * elems * 2 + (1 if fused else 2) * elems + elems * vbytes
     quant_gbs = quant_bytes / (qt_avg * 1e-3) / 1e9
 
     out = {
@@ -389,28 +408,31 @@ def main():
             "peak_tops_used": peak,
             # HIP-event pairs on the launch stream around the quantize stage as the step runs it (three
             # launches through mi355_sage_quant_qkv_bf16) and around the attention launch
-            "stage_ms": {"quant_qkv": round(qt_avg, 5), "attn": round(at_avg, 5)},
+            "stage_ms": {"quantize": round(qt_avg, 5), "attn": round(at_avg, 5)},
+            "q_encoded_by": "attention kernel (prologue)" if fused else "quantize stage",
             "graph_replay_ms": None if graph_ms is None else round(graph_ms, 5),
             "graph_replays": 200,
             "clock_ramp_steps": r["ramp_steps"],      # untimed steps run before the warm-up, see run_workload
             "device": torch.cuda.get_device_name(0),
         },
         "roofline": {
-            "kernel": "sage_attn_kernel<%d,%d>" % (D, w.variant),
+            "kernel": "sage_attn_kernel<%d,%d%s>" % (D, w.variant, ", Q encoded in the prologue" if fused else ""),
             "bound": "mfma",
             "achieved": round(attn_tops, 2),
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(attn_tops / peak, 4),
             "traffic": measured_traffic(w.name),
-            # int8 Q and K read once, V^T tiles (fp16 or e4m3) read once, bf16 O written once
-            "algorithmic_bytes_per_launch": 2 * elems + elems * (2 if w.variant == 0 else 1) + 2 * elems,
+            # Q (bf16, or int8 where the quantize stage encodes it) and int8 K read once, V^T tiles (fp16 or
+            # e4m3) read once, bf16 O written once
+            "algorithmic_bytes_per_launch": (2 if fused else 1) * elems + elems + elems * vbytes + 2 * elems,
             "avg_ms": round(at_avg, 5), "median_ms": round(at_med, 5), "min_ms": round(at_min, 5),
             "algorithmic_ops_per_launch": w.ops,
         },
         # the HBM-bound part of the step: prep_kernel, stats_final_kernel, quant_kernel together
         "roofline_quantize": {
-            "kernels": "prep_kernel + stats_final_kernel + quant_kernel (one event pair around the three launches)",
+            "kernels": "prep_kernel + stats_final_kernel + quant_kernel (one event pair around the three launches)%s" % (
+                "; K and V only" if fused else ""),
             "bound": "hbm",
             "achieved": round(quant_gbs, 1),
             "peak": PEAK_HBM_GBS,
@@ -436,7 +458,7 @@ def main():
             others[ww.name] = {"steps": n_steps, "warmup": n_warm, "ms_per_step": round(rr["ms_per_step"], 4),
                                "TOPS": round(t_, 1), "pct_of_peak": round(100.0 * t_ / pk, 2),
                                "attn_kernel_avg_ms": round(rr["attn"][0], 4), "attn_kernel_frac_of_peak": round(a_ / pk, 4),
-                               "quant_qkv_avg_ms": round(rr["quant"][0], 4), "dtype": "int8/f16" if ww.variant == 0 else "int8/f8e4m3"}
+                               "quantize_avg_ms": round(rr["quant"][0], 4), "q_in_attention_kernel": rr["q_in_kernel"], "dtype": "int8/f16" if ww.variant == 0 else "int8/f8e4m3"}
             del rr, qq, kk, vv
             torch.cuda.empty_cache()
         out["config"]["other_workloads"] = others

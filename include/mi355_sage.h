@@ -299,6 +299,7 @@ int mi355_sage_quant_qk_norm_rope_bf16(
  * with the K statistics, the e4m3 V encode with the Q / K encoders): same outputs, bit for bit, as
  * mi355_sage_quant_qk_bf16 followed by mi355_sage_quant_v_f16 / _fp8, which take five.  vq is v16
  * or v8 by `variant`; vscale is written for MI355_SAGE_PV_FP8 only (may be NULL otherwise).
+ * q8 == qscale == NULL: Q is not encoded here (mi355_sage_attn_fwd_q16 does it); qmul is still written.
  * scratch as for mi355_sage_quant_qk_bf16. */
 int mi355_sage_quant_qkv_bf16(
     const void* Q, const void* K, const void* V,
@@ -333,6 +334,21 @@ int mi355_sage_attn_fwd(
     int B, int H, int N_q, int N_kv, int kv_valid, int mask_lo, int mask_hi, int D,
     void* O, const int64_t* o_strides, int64_t o_offset_elems,
     const void* qshift, void* stats, void* stream);
+
+/* The attention stage as the plain forward (no Stats, no additive mask) runs it: Q comes as bf16
+ * (any [B,H,N,D] view with 16-byte aligned rows) together with the channel multipliers `qmul`
+ * [B,H,D] of the quantize stage, and the kernel encodes its own rows while its first K / V tiles
+ * are on their way — the same codes and scales mi355_sage_quant_qkv_bf16 writes, so O has the
+ * same bits as mi355_sage_attn_fwd on that stage's q8 / qscale.  mi355_sage_quant_qkv_bf16 with
+ * q8 == qscale == NULL is the quantize stage that goes with it (K and V only, qmul still written).
+ * Head dims 64 and 128; a shape that the split schedule takes returns -2 (use mi355_sage_attn_fwd).
+ * The rest of the arguments as in mi355_sage_attn_fwd.  (A stage of this library's own; the
+ * reference's boundary is the one-shot call, serenitymojo/ops/cshim/cudnn_sdpa.cpp:370-393.) */
+int mi355_sage_attn_fwd_q16(
+    const void* Q, const int64_t* q_strides, int64_t q_offset_elems, const void* qmul, int blkq,
+    const void* k8, const void* kscale, int blkk, const void* vq, const void* vscale, int variant,
+    int B, int H, int N_q, int N_kv, int kv_valid, int mask_lo, int mask_hi, int D,
+    void* O, const int64_t* o_strides, int64_t o_offset_elems, void* stream);
 
 /* Scheduling of the attention kernel (no counterpart in the reference).
  * One workgroup computes 256 query rows of one head against all keys.  A shape whose row tiles

@@ -51,6 +51,8 @@ SIGNATURES = {
     "mi355_sage_quant_v_fp8": (_int, [_vp] + [_int] * 4 + [_i64p, _i64, _int, _int, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "mi355_sage_attn_fwd": (_int, [_vp, _vp, _int, _vp, _vp, _int, _vp, _vp, _int] + [_int] * 8
                             + [_vp, _i64p, _i64, _vp, _vp, _vp]),
+    "mi355_sage_attn_fwd_q16": (_int, [_vp, _i64p, _i64, _vp, _int, _vp, _vp, _int, _vp, _vp, _int] + [_int] * 8
+                                + [_vp, _i64p, _i64, _vp]),
     "mi355_sage_attn_split_faults": (_int, [_int]),
     "mi355_sage_attn_split_rule": (_int, [_int] * 6),
     "mi355_sage_set_attn_split": (_int, [_int]),

@@ -622,7 +622,8 @@ int mi355_sage_quant_qkv_bf16(const void* Q, const void* K, const void* V, int B
                               int variant, int blkq, int blkk, int k_flags, int mask_lo, int mask_hi,
                               void* q8, void* qscale, void* k8, void* kscale, void* kmean, void* qmul, void* kmul,
                               void* vq, void* vscale, void* scratch, size_t scratch_bytes, void* stream) {
-    if (!Q || !K || !V || !q8 || !qscale || !k8 || !kscale || !kmean || !qmul || !kmul || !vq || !scratch) return MI355_SAGE_EINVAL;
+    if (!Q || !K || !V || !k8 || !kscale || !kmean || !qmul || !kmul || !vq || !scratch) return MI355_SAGE_EINVAL;
+    if ((q8 == nullptr) != (qscale == nullptr)) return MI355_SAGE_EINVAL;      // both NULL: Q is left to mi355_sage_attn_fwd_q16
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
     if (!q_strides || !k_strides || !v_strides) return MI355_SAGE_EINVAL;
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
@@ -723,6 +724,35 @@ int mi355_sage_attn_fwd(const void* q8, const void* qscale, int blkq, const void
     a.split_wgs = attn_split_workgroups(B, H, N_q, kv_valid, D, variant);
     const size_t split_bytes = attn_split_bytes(a.split_wgs, D);
     if (split_bytes > 0 && (rc = internal_workspace(g_split_ws, split_bytes, static_cast<hipStream_t>(stream), &a.split))) return rc;
+    SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
+    return MI355_SAGE_OK;
+}
+
+int mi355_sage_attn_fwd_q16(const void* Q, const int64_t* q_strides, int64_t q_off, const void* qmul, int blkq,
+                            const void* k8, const void* kscale, int blkk, const void* vq, const void* vscale, int variant,
+                            int B, int H, int N_q, int N_kv, int kv_valid, int mask_lo, int mask_hi, int D,
+                            void* O, const int64_t* o_strides, int64_t o_off, void* stream) {
+    if (!Q || !q_strides || !qmul || !k8 || !kscale || !vq || !O || !o_strides) return MI355_SAGE_EINVAL;
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
+    if (kv_valid <= 0 || kv_valid > N_kv) return MI355_SAGE_EINVAL;
+    if (variant == MI355_SAGE_PV_FP8 && !vscale) return MI355_SAGE_EINVAL;
+    if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
+    if (!dims_ok(D) || D > 128 || !blk_ok(blkq) || !blk_ok(blkk)) return MI355_SAGE_EUNSUPPORTED;
+    int rc;
+    if ((rc = check_kv_len(N_kv, blkk, D))) return rc;
+    if ((rc = check_view("Q", Q, q_strides, q_off)) || (rc = check_view("O", O, o_strides, o_off))) return rc;
+    // (shapes of the split schedule keep the encoded-Q form: the one-shot calls do the same)
+    if (attn_split_workgroups(B, H, N_q, kv_valid, D, variant) > 0) return MI355_SAGE_EUNSUPPORTED;
+    AttnArgs a{};
+    const View q = make_view(Q, q_strides, q_off);
+    a.q_src = q.p; a.qsb = q.sb; a.qsh = q.sh; a.qsn = q.sn; a.qmul = static_cast<const float*>(qmul); a.blkq = blkq;
+    a.k8 = static_cast<const int8_t*>(k8); a.kscale = static_cast<const float*>(kscale); a.blkk = blkk;
+    a.vq = vq; a.vscale = static_cast<const float*>(vscale);
+    a.variant = variant;
+    if (clip_mask(kv_valid, mask_lo, mask_hi, &a.km) <= 0) return MI355_SAGE_EINVAL;
+    a.B = B; a.H = H; a.Nq = N_q; a.Nkv = N_kv; a.kv_valid = kv_valid; a.D = D;
+    a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(N_kv, kPadKV);
+    a.o = static_cast<uint16_t*>(O) + o_off; a.osb = o_strides[0]; a.osh = o_strides[1]; a.osn = o_strides[2];
     SAGE_HIP(launch_attn(a, static_cast<hipStream_t>(stream)));
     return MI355_SAGE_OK;
 }

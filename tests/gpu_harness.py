@@ -115,8 +115,9 @@ def quant_v(v_bits, variant, mask=(0, 0), strides=None, v_off=0, shape=None):
     return dict(vq=out.cpu().numpy(), vscale=vs.cpu().numpy(), dev=dict(vq=out, vscale=vs))
 
 
-def quant_qkv(q_bits, k_bits, v_bits, scale, variant, blkq, blkk, mask=(0, 0)):
-    """mi355_sage_quant_qkv_bf16: the three launches of the one-shot calls.  Same dict as quant_qk plus vq, vscale."""
+def quant_qkv(q_bits, k_bits, v_bits, scale, variant, blkq, blkk, mask=(0, 0), encode_q=True):
+    """mi355_sage_quant_qkv_bf16: the three launches of the one-shot calls.  Same dict as quant_qk plus vq, vscale.
+    encode_q False: q8 and qscale are passed as NULL (Q is left to mi355_sage_attn_fwd_q16)."""
     L = _lib.lib()
     B, Sq, H, D = q_bits.shape
     Skv = k_bits.shape[1]
@@ -132,7 +133,8 @@ def quant_qkv(q_bits, k_bits, v_bits, scale, variant, blkq, blkk, mask=(0, 0)):
     scr = torch.full((max(L.mi355_sage_quant_scratch_bytes(B, H, Skv, D), 8),), 0xAB, dtype=torch.uint8, device="cuda")
     rc = L.mi355_sage_quant_qkv_bf16(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), B, H, Sq, Skv, D, scale, sq, sk, sk, 0, 0, 0,
                                      variant, blkq, blkk, _lib.K_SMOOTH | _lib.K_BALANCE, mask[0], mask[1],
-                                     q8.data_ptr(), qs.data_ptr(), k8.data_ptr(), ks.data_ptr(), km.data_ptr(), qm.data_ptr(),
+                                     q8.data_ptr() if encode_q else None, qs.data_ptr() if encode_q else None, k8.data_ptr(),
+                                     ks.data_ptr(), km.data_ptr(), qm.data_ptr(),
                                      kmu.data_ptr(), vq.data_ptr(), vs.data_ptr(), scr.data_ptr(), scr.numel(), stream())
     assert rc == 0, rc
     torch.cuda.synchronize()
@@ -157,6 +159,21 @@ def attn_fwd(q8, qscale, blkq, k8, kscale, blkk, vq, vscale, variant, Sq, Skv, k
     assert rc == 0, rc
     torch.cuda.synchronize()
     return to_bits(o), (stats.cpu().numpy() if want_stats else None)
+
+
+def attn_fwd_q16(q_bits, qmul, blkq, k8, kscale, blkk, vq, vscale, variant, Skv, kv_valid=None, mask=(0, 0)):
+    """mi355_sage_attn_fwd_q16: Q as bf16 bits [B,Sq,H,D] (host), the other operands as device tensors.
+    Returns the return code and O bits."""
+    L = _lib.lib()
+    B, Sq, H, D = q_bits.shape
+    qd = dev_bf16(q_bits)
+    o = torch.zeros((B, Sq, H, D), dtype=torch.bfloat16, device="cuda")
+    st = _lib.strides_bhnd(Sq, H, D)
+    rc = L.mi355_sage_attn_fwd_q16(qd.data_ptr(), st, 0, qmul.data_ptr(), blkq, k8.data_ptr(), kscale.data_ptr(), blkk,
+                                   vq.data_ptr(), vscale.data_ptr() if vscale is not None else None, variant,
+                                   B, H, Sq, Skv, kv_valid or Skv, mask[0], mask[1], D, o.data_ptr(), st, 0, stream())
+    torch.cuda.synchronize()
+    return rc, to_bits(o)
 
 
 def cos_maxabs(a, b):

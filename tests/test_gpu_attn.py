@@ -111,6 +111,31 @@ def test_one_shot_equals_stage_pipeline(wid, S, smooth):
     np.testing.assert_array_equal(got, staged)
 
 
+@pytest.mark.parametrize("variant,blkq,D,S", [(0, 128, 128, 700), (0, 64, 128, 333), (1, 32, 128, 520), (0, 32, 64, 1024),
+                                               (1, 128, 64, 77)])
+def test_attention_stage_that_encodes_q_itself(variant, blkq, D, S):
+    """mi355_sage_attn_fwd_q16 (bf16 Q + the stage's channel multipliers) gives the bits of
+    mi355_sage_attn_fwd on the stage's q8 / qscale — the kernel's own Q encode is the quantizer's —
+    and of the one-shot call, which takes this route; shapes of the split schedule are refused."""
+    import gpu_harness as H
+    w = WORKLOADS[1 if D == 64 else 2].scaled(B=2, H=3, S=S)
+    q, k, v = make_inputs(w)
+    g = H.quant_qk(q, k, w.scale, blkq, 64, True)["dev"]
+    gv = H.quant_v(v, variant)["dev"]
+    staged, _ = H.attn_fwd(g["q8"], g["qscale"], blkq, g["k8"], g["kscale"], 64, gv["vq"], gv["vscale"], variant, S, S)
+    rc, fused = H.attn_fwd_q16(q, g["qmul"], blkq, g["k8"], g["kscale"], 64, gv["vq"], gv["vscale"], variant, S)
+    assert rc == 0, rc
+    np.testing.assert_array_equal(fused, staged)
+    np.testing.assert_array_equal(_one_shot(q, k, v, w.scale, variant, blkq, 64), staged)
+    big = WORKLOADS[2].scaled(B=1, H=33, S=2048)             # 264 items: the split schedule's
+    if _lib.lib().mi355_sage_attn_split_rule(big.B, big.H, big.S, big.S, big.D, 0) > 0:
+        qb, kb, vb = make_inputs(big)
+        gb = H.quant_qk(qb, kb, big.scale, 128, 64, True)["dev"]
+        gvb = H.quant_v(vb, 0)["dev"]
+        rc, _ = H.attn_fwd_q16(qb, gb["qmul"], 128, gb["k8"], gb["kscale"], 64, gvb["vq"], None, 0, big.S)
+        assert rc == -2, rc
+
+
 def test_default_recipe_entry_point(oracle):
     """mi355_sage_sdpa_bf16 without the recipe arguments: blkq 128 / blkk 64 / smoothing and balancing on."""
     import gpu_harness as H

@@ -236,6 +236,11 @@ def test_three_launch_stage_equals_the_separate_stages(wid, S, mask, variant):
     np.testing.assert_array_equal(got["vq"], vv["vq"])
     if variant == 1:
         np.testing.assert_array_equal(got["vscale"].view(np.uint32), vv["vscale"].view(np.uint32))
+    # without the Q encode (q8 == qscale == NULL): everything else as before, the Q outputs untouched
+    rest = H.quant_qkv(q, k, v, w.scale, variant, blkq, 64, mask=mask, encode_q=False)
+    for name in ("k8", "kscale", "kmean", "qmul", "kmul", "vq"):
+        np.testing.assert_array_equal(rest[name], got[name], err_msg=name)
+    assert np.all(rest["q8"] == 77) and np.all(rest["qscale"] == -1.0)
 
 
 def test_quant_full_size_properties():
