@@ -73,7 +73,8 @@ extern "C" {
  * while its stream is being captured into a graph returns -3.  Otherwise
  * workspace_bytes must be at least mi355_sage_workspace_bytes(...) and the
  * pointer 256-byte aligned; calls that share one workspace must be ordered on one
- * stream.  `causal` must be 0.
+ * stream.  `causal` != 0 (cudnn_sdpa.cpp:190-192, cuDNN's set_causal_mask): query i sees keys j <= i only,
+ * aligned at the top left when N_q != N_kv; the key tiles past a workgroup's last row are never read.
  * ---------------------------------------------------------------------- */
 int mi355_sage_sdpa_bf16(
     const void* Q, const void* K, const void* V, void* O,

@@ -290,7 +290,6 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     if (!Q || !K || !V || !O) return MI355_SAGE_EINVAL;
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return MI355_SAGE_EINVAL;
     if (!qs || !ks || !vs || !os) return MI355_SAGE_EINVAL;
-    if (causal) { SAGE_LOG("causal attention is not supported"); return MI355_SAGE_EUNSUPPORTED; }
     if (!dims_ok(D)) { SAGE_LOG("head dim %d not supported (64, 128 or 256)", D); return MI355_SAGE_EUNSUPPORTED; }
     if (D == 256 && pre.q.gain != nullptr) { SAGE_LOG("the fused RMSNorm / RoPE are built for head dims 64 and 128"); return MI355_SAGE_EUNSUPPORTED; }
     if (variant != MI355_SAGE_PV_FP16 && variant != MI355_SAGE_PV_FP8) return MI355_SAGE_EUNSUPPORTED;
@@ -337,7 +336,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     }
     // (one decision for carving and launching; slots the caller's workspace was not sized for — a
     // forced schedule of the test switch — come from the library's per-stream buffer)
-    const int split_wgs = attn_split_workgroups(B, H, N_q, kv, D, variant);
+    const int split_wgs = causal ? 0 : attn_split_workgroups(B, H, N_q, kv, D, variant);
     // The plain forward leaves Q to the attention kernel, which encodes its own rows (same codes and
     // scales): the quantize stage then neither reads Q nor writes its codes.
     const bool q_in_kernel = Stats == nullptr && mask.add == nullptr && pre.q.gain == nullptr && D <= 128 && split_wgs == 0;
@@ -372,6 +371,7 @@ int sdpa_impl(const void* Q, const void* K, const void* V, void* O, void* Stats,
     a.variant = variant;
     a.km = km;
     a.B = B; a.H = H; a.Nq = N_q; a.Nkv = kv; a.kv_valid = kv; a.D = D;
+    a.causal = causal ? 1 : 0;
     a.nq_pad = pad_to(N_q, kTileQ); a.nkv_pad = pad_to(kv, kPadKV);
     a.o = static_cast<uint16_t*>(O) + o_off; a.osb = os[0]; a.osh = os[1]; a.osn = os[2];
     a.stats = Stats ? static_cast<float*>(Stats) + stats_off : nullptr;

@@ -159,7 +159,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     const int8_t* __restrict__ k8, const float* __restrict__ kscale, int blkk,
     const uint8_t* __restrict__ vq, const float* __restrict__ vscale,
     const float* __restrict__ qshift,
-    int H, int Nq, int kv_valid, int mask_lo, int mask_hi, int64_t nq_pad, int64_t nkv_pad,
+    int H, int Nq, int kv_valid_all, int mask_lo, int mask_hi, int causal, int64_t nq_pad, int64_t nkv_pad,
     uint16_t* __restrict__ o, int64_t osb, int64_t osh, int64_t osn,
     float* __restrict__ stats, int n_qtiles, int total_wg,
     const uint16_t* __restrict__ amask, int64_t amb, int64_t amh, int64_t amn,
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     const int xcd_full = total_wg - (items_per - 1) * 8;        // XCDs that own `items_per` items (1..8)
     const int n_items = xcd < xcd_full ? items_per : items_per - 1;
     const int item0 = xcd < xcd_full ? xcd * items_per : xcd_full * items_per + (xcd - xcd_full) * (items_per - 1);
-    const int ntiles_item = (kv_valid + kTileKV - 1) / kTileKV;
+    const int ntiles_item = (kv_valid_all + kTileKV - 1) / kTileKV;
     // (the launcher has checked that steps x workgroups stays inside 32 bits)
     const uint32_t xcd_steps = (uint32_t)n_items * (uint32_t)ntiles_item;
     auto span_lo = [&](int j) -> int {
@@ -248,11 +248,15 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     const int item_local = SPLIT ? (int)((uint32_t)(span_end - 1) / (uint32_t)ntiles_div) : wg_j;
     const int item_base = item_local * ntiles_item;
     const int t_off = SPLIT ? max(span_begin, item_base) - item_base : 0;
-    const int ntiles = SPLIT ? span_end - item_base - t_off : ntiles_item;
-    const bool seg_finishes = !SPLIT || t_off + ntiles == ntiles_item;   // holds the item's last key tile: writes the output
-    span_end = item_base + t_off;
     const int wg = item0 + item_local;
     const int qt = (int)((uint32_t)wg % (uint32_t)qtiles_div);
+    // Causal (query i sees keys j <= i, cuDNN's top-left alignment): the keys past this workgroup's last
+    // row are masked for every one of its rows — they are treated as the ragged end, so their tiles are
+    // never copied — and the steps on a wave's diagonal mask key > row element by element (below).
+    const int kv_valid = (!SPLIT && causal) ? min(kv_valid_all, (qt + 1) * ROWS_WG) : kv_valid_all;
+    const int ntiles = SPLIT ? span_end - item_base - t_off : (kv_valid + kTileKV - 1) / kTileKV;
+    const bool seg_finishes = !SPLIT || t_off + ntiles == ntiles_item;   // holds the item's last key tile: writes the output
+    span_end = item_base + t_off;
     const int64_t bh = (uint32_t)wg / (uint32_t)qtiles_div;
     const int b = (int)((uint32_t)bh / (uint32_t)heads_div), h = (int)((uint32_t)bh % (uint32_t)heads_div);
     // (through an empty statement: what is derived from the lane number — row addresses, fragment
@@ -263,6 +267,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
     const int l32 = lane & 31, half = lane >> 5;
     const int row_in_tile = wave * 32 + l32;
     const int qrow = qt * ROWS_WG + row_in_tile;        // this lane's query (padded index)
+    const int wave_row0 = qt * ROWS_WG + wave * 32;     // the wave's first query (the same for all its lanes)
     if constexpr (SPLIT) __syncthreads();               // every wave has left the previous segment's LDS
 
     // Q^T fragments: 16 bytes of the head dim per step, resident for the whole kernel.
@@ -622,14 +627,15 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
         // A masked score becomes -inf (as an integer: below every real accumulator), which the
         // exponent path below turns into p = 0 without any further test.
         const int key0 = t_off * kTileKV + h * SK;
-        if (!TRIP && __builtin_expect(key0 + SK > kv_valid || (key0 < mask_hi && key0 + SK > mask_lo), 0)) {
+        if (!TRIP && __builtin_expect(key0 + SK > kv_valid || (key0 < mask_hi && key0 + SK > mask_lo) ||
+                                      (causal && key0 + SK - 1 > wave_row0), 0)) {
             asm volatile("" ::: "memory");
 #pragma unroll
             for (int kb = 0; kb < SKB; kb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int key = key0 + kb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                    if (key >= kv_valid || (key >= mask_lo && key < mask_hi)) s[X][kb][i] = (int)0xFF800000;
+                    if (key >= kv_valid || (key >= mask_lo && key < mask_hi) || (causal && key > qrow)) s[X][kb][i] = (int)0xFF800000;
                 }
         }
         // biased scores in the log2 domain, without the reference maximum (ADDMASK only)
@@ -848,6 +854,7 @@ __global__ __launch_bounds__(D > 128 ? 256 : 512) void sage_attn_kernel(
         int clean = (kv_valid - t_off * kTileKV) / SK;
         if (mask_hi > mask_lo && t_off * kTileKV < mask_hi) clean = min(clean, max(mask_lo - t_off * kTileKV, 0) / SK);
         if (exact_bias) clean = 0;
+        if (causal) clean = min(clean, (wave_row0 + 1) / SK);       // steps whose every key is <= the wave's first row
         // (... and in front of the last tiles, so that the copies a trip starts need no clamping)
         const int trip_end = min(last_step - SPT * (KOFF + LEAD) + (SPT - 1), clean);
         for (; hs + PERIOD <= trip_end; hs += PERIOD) {
@@ -1043,7 +1050,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
     const int n_qtiles = (int)(a.nq_pad / (kThreads / 2));
     const int64_t total = (int64_t)n_qtiles * a.B * a.H;
     if (total <= 0 || total > 0x7FFFFFFF) return hipErrorInvalidValue;
-    const int split = (D <= 128 && VARIANT == 0) ? a.split_wgs : 0;
+    const int split = (D <= 128 && VARIANT == 0 && !a.causal) ? a.split_wgs : 0;
     int* flags = nullptr;
     float* part = nullptr;
     if (split > 0) {
@@ -1057,7 +1064,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
 #define SAGE_LAUNCH_ATTN2(STATS, ADDMASK, SPLIT)                                                                         \
     hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, STATS, ADDMASK, SPLIT>), grid, block, 0, st, a.q8, a.qscale, a.blkq, \
                        a.q_src, a.qsb, a.qsh, a.qsn, a.qmul, a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, a.qshift, a.H, a.Nq, a.kv_valid,          \
-                       a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,               \
+                       a.km.lo, a.km.hi, a.causal, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, a.stats, n_qtiles,               \
                        (int)total, a.amask, a.amb, a.amh, a.amn, split >> 3, part, flags, g_split_wait.load())
 #define SAGE_LAUNCH_ATTN(STATS, ADDMASK)                                  \
     do {                                                                  \
@@ -1074,7 +1081,7 @@ static hipError_t launch_attn_dv(const AttnArgs& a, hipStream_t st) {
             if (a.amask != nullptr || a.stats != nullptr || split > 0 || a.qmul == nullptr) return hipErrorInvalidValue;
             hipLaunchKernelGGL((sage_attn_kernel<D, VARIANT, false, false, false, true>), grid, block, 0, st, nullptr, nullptr, a.blkq,
                                a.q_src, a.qsb, a.qsh, a.qsn, a.qmul, a.k8, a.kscale, a.blkk, (const uint8_t*)a.vq, a.vscale, nullptr,
-                               a.H, a.Nq, a.kv_valid, a.km.lo, a.km.hi, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, nullptr,
+                               a.H, a.Nq, a.kv_valid, a.km.lo, a.km.hi, a.causal, a.nq_pad, a.nkv_pad, a.o, a.osb, a.osh, a.osn, nullptr,
                                n_qtiles, (int)total, nullptr, 0, 0, 0, 0, nullptr, nullptr, g_split_wait.load());
         } else {
             return hipErrorInvalidValue;

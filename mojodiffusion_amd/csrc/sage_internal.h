@@ -121,6 +121,7 @@ struct AttnArgs {
     int variant;
     KeyMask km;
     int B, H, Nq, Nkv, kv_valid, D;
+    int causal;              // 1: query i sees keys j <= i only (never together with the split schedule)
     int64_t nq_pad, nkv_pad;
     uint16_t* o; int64_t osb, osh, osn;
     float* stats;            // [B,H,Nq] or null

@@ -96,8 +96,6 @@ def test_argument_validation_without_device():
     assert call(fake, fake, fake, fake, (1, 2, 128, -4, 128), st) == -1
     assert call(fake, fake, fake, fake, ok_dims, None) == -1
     # unsupported configurations -> -2
-    assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
-                                  0, 0, 0, 0, 1, None, 0, None, 0) == -2          # causal
     assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 96, 0.1, st, st, st, st,
                                   0, 0, 0, 0, 0, None, 0, None, 0) == -2          # head dim
     assert L.mi355_sage_sdpa_bf16(fake, fake, fake, fake, 1, 2, 128, 128, 128, 0.1, st, st, st, st,
