@@ -243,10 +243,9 @@ int quantize(const View& q, const View& k, const View* v, int B, int H, int Nq, 
     PrepArgs p{};
     p.k = k; p.H = H; p.Nkv = Nkv; p.nkv_pad = nkp; p.km = km; p.pre_k = pre.k;
     p.vmode = 2;
-    if (v != nullptr) {
+    if (v != nullptr && variant != MI355_SAGE_PV_FP16) {
         p.v = *v;
-        p.vmode = variant == MI355_SAGE_PV_FP16 ? 0 : 1;
-        p.v16 = static_cast<uint16_t*>(vq);
+        p.vmode = 1;                       // (the fp16 repack needs no statistics: it goes with launch 3)
         p.vpart = vpart;
     }
     p.kpart_sum = kstats ? o.kpart_sum : nullptr;
@@ -267,6 +266,7 @@ int quantize(const View& q, const View& k, const View* v, int B, int H, int Nq, 
     a.kmean = o.kmean; a.qmul = o.qmul; a.kmul = o.kmul; a.vscale = vscale;
     a.q8 = o.q8; a.qscale = o.qscale; a.rowdot = o.rowdot; a.k8 = o.k8; a.kscale = o.kscale;
     if (p.vmode == 1) { a.v = *v; a.v8 = static_cast<uint8_t*>(vq); }
+    else if (v != nullptr) { a.v = *v; a.v16 = static_cast<uint16_t*>(vq); }
     a.pre_q = pre.q; a.pre_k = pre.k;
     SAGE_HIP(launch_quant(a, B, D, st));
     return 0;

@@ -95,7 +95,8 @@ struct QuantArgs {
     float* rowdot;                   // [B,H,nq_pad] <f32(q)*cmul, kmean>, or null
     int8_t* k8;
     float* kscale;
-    uint8_t* v8;
+    uint8_t* v8;                     // e4m3 V tiles (needs vscale), or
+    uint16_t* v16;                   // fp16 V tiles (the repack needs no statistics; it rides here so that launch 1 is short)
     PreOp pre_q, pre_k;
     int nq_blk, nk_blk, nv_tile, n_bh;     // filled by the launcher
 };

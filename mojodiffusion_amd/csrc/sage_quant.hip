@@ -783,10 +783,8 @@ hipError_t launch_stats_final(const FinalArgs& a, hipStream_t st) {
 // ---------------------------------------------------------------------------
 // Launch 3: Q blocks, K blocks and (e4m3 variant) V tiles as workgroup roles.
 // ---------------------------------------------------------------------------
-// Threads per workgroup: 512 at 128 channels — a block of 128 tokens is then four 16-byte chunks
-// per thread, few enough registers for eight waves per SIMD, which is what keeps loads in flight
-// while other waves encode (a workgroup loads, reduces, encodes and stores in turn).
-template <int D, bool PRE> constexpr int quant_threads() { return D == 128 && !PRE ? 256 : 256; }
+// Threads per workgroup (512 at 128 channels, i.e. fewer registers and more waves per SIMD, measured slower).
+template <int D, bool PRE> constexpr int quant_threads() { return 256; }
 
 template <int D, bool PRE>
 __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
@@ -794,6 +792,7 @@ __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
     union Smem {
         float red[NT / 64];
         uint8_t tile8[64 * (D + 16)];
+        uint16_t tile16[64 * D];
     };
     __shared__ __attribute__((aligned(16))) Smem sm;
     // consecutive workgroups take the same rows of consecutive heads: in [.., N, H, D] memory those
@@ -820,6 +819,8 @@ __global__ __launch_bounds__(256) void quant_kernel(QuantArgs a) {
         else if (a.blkk == 64) SAGE_K(64);
         else SAGE_K(32);
 #undef SAGE_K
+    } else if (a.v16 != nullptr) {
+        quant_v_f16_body<D>(r - a.nq_blk - a.nk_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km, a.v16, sm.tile16);
     } else {
         quant_v_fp8_body<D, NT>(r - a.nq_blk - a.nk_blk, h, b, a.v.p, a.v.sb, a.v.sh, a.v.sn, a.Nkv, a.H, a.nkv_pad, a.km,
                             a.vscale, a.v8, sm.tile8);
@@ -830,7 +831,7 @@ hipError_t launch_quant(const QuantArgs& a_in, int B, int D, hipStream_t st) {
     QuantArgs a = a_in;
     a.nq_blk = a.q8 != nullptr ? (int)(a.nq_pad / a.blkq) : 0;
     a.nk_blk = a.k8 != nullptr ? (int)(a.nkv_pad / a.blkk) : 0;
-    a.nv_tile = a.v8 != nullptr ? (int)(a.nkv_pad / 64) : 0;
+    a.nv_tile = (a.v8 != nullptr || a.v16 != nullptr) ? (int)(a.nkv_pad / 64) : 0;
     if (a.q8 != nullptr && a.nq_pad % a.blkq != 0) return hipErrorInvalidValue;
     if (a.k8 != nullptr && a.nkv_pad % a.blkk != 0) return hipErrorInvalidValue;
     a.n_bh = B * a.H;
