@@ -354,9 +354,12 @@ __device__ __forceinline__ void kstats_group_body(
         if (g >= 0 && key_kept(s0 + i, N, km)) w[i] = *reinterpret_cast<const u32x4*>(src + (int64_t)(s0 + i) * sn);
     }
     double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    float mn[8], mx[8];
+    float mn[8], mx[8], xprev[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) { mn[e] = INFINITY; mx[e] = -INFINITY; }
+    for (int e = 0; e < 8; e++) { mn[e] = INFINITY; mx[e] = -INFINITY; xprev[e] = 0.0f; }
+    // every token of this leaf counts (no ragged end, no masked range inside it)
+    const bool all_kept = g >= 0 && s0 + kLeaf <= N && !(s0 < km.hi && s0 + kLeaf > km.lo);
+    static_assert(kLeaf % 2 == 0, "tokens are taken in pairs");
 #pragma unroll
     for (int i = 0; i < kLeaf; i++) {
         float x[8];
@@ -366,7 +369,21 @@ __device__ __forceinline__ void kstats_group_body(
         // tokens that do not count are +0.0 here, which leaves a double sum unchanged
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] += (double)x[e];
-        if (kept) {
+        if (all_kept) {
+            // (the common case, two tokens per three-operand instruction; written as instructions because the
+            // compiler puts a canonicalising v_max in front of every operand of fminf / fmaxf that comes out of
+            // bit operations — six instructions per element instead of one)
+            if (i & 1) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    asm("v_min3_f32 %0, %0, %1, %2" : "+v"(mn[e]) : "v"(xprev[e]), "v"(x[e]));
+                    asm("v_max3_f32 %0, %0, %1, %2" : "+v"(mx[e]) : "v"(xprev[e]), "v"(x[e]));
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) xprev[e] = x[e];
+            }
+        } else if (kept) {
 #pragma unroll
             for (int e = 0; e < 8; e++) { mn[e] = fminf(mn[e], x[e]); mx[e] = fmaxf(mx[e], x[e]); }
         }
